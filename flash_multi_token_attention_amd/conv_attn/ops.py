@@ -1,0 +1,242 @@
+"""Op layer of conv-attention: the functions the reference binds with pybind11
+(``forward``, ``dq_backward``, ``dkdv_backward`` in conv_attn/bindings.cpp:46-56,
+``forward_inference`` in conv_attn/fwd_inference_bindings.cpp:20-23), same
+argument order, calling the C ABI of libconvattn_hip.so through ctypes.
+
+Python owns every allocation; launches go on torch's current stream.
+
+Differences from the reference ops, all deliberate:
+  * rectangular windows (c_q != c_k) work; the reference dispatches square ones only
+  * Q, K, V, dO may be bfloat16 or float32 (float32 runs the fp32-arithmetic kernels)
+  * ``conv_kernel`` is used at fp32 precision whatever dtype it arrives in
+  * statistics (M, L, D, LSE) are fp32; ``D`` / ``L`` arguments in other dtypes are upcast
+  * ``out_dtype`` picks the dtype of O / dQ / dK / dV (default float32, as the reference returns)
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional, Tuple
+
+import torch
+
+from .. import _lib
+
+_DT = {torch.bfloat16: _lib.BF16, torch.float32: _lib.F32}
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return C.c_void_p(t.data_ptr()) if t is not None else C.c_void_p(0)
+
+
+def _stream(t: torch.Tensor):
+    return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _check_input(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+
+
+def _check_qkv(Q, K, V, names=("Q", "K", "V")):
+    for t, n in zip((Q, K, V), names):
+        _check_input(t, n)
+        if t.dim() != 4:
+            raise RuntimeError(f"{n} must be [batch, heads, seq_len, d_head]")
+    if Q.dtype not in _DT:
+        raise RuntimeError("Q must be bfloat16 or float32")
+    if K.dtype != Q.dtype or V.dtype != Q.dtype:
+        raise RuntimeError("K and V must have the dtype of Q")
+    B, H, Nq, d = Q.shape
+    if K.shape[0] != B or V.shape[0] != B:
+        raise RuntimeError("K batch size must match Q" if K.shape[0] != B else "V batch size must match Q")
+    if K.shape[1] != H or V.shape[1] != H:
+        raise RuntimeError("K num_heads must match Q" if K.shape[1] != H else "V num_heads must match Q")
+    if K.shape[3] != d or V.shape[3] != d:
+        raise RuntimeError("K d_head must match Q" if K.shape[3] != d else "V d_head must match Q")
+    if V.shape[2] != K.shape[2]:
+        raise RuntimeError("V seq_len must match K")
+    if Q.device != K.device or Q.device != V.device:
+        raise RuntimeError("Q, K and V must be on the same device")
+
+
+def _weights(conv_kernel: torch.Tensor, H: int, pad_q: int, pad_k: int, device) -> torch.Tensor:
+    if conv_kernel.dim() != 3 or conv_kernel.shape[0] != H:
+        raise RuntimeError("conv_kernel must be [heads, kernel_size_q, kernel_size_k]")
+    c_q, c_k = conv_kernel.shape[1], conv_kernel.shape[2]
+    if c_k % 2 == 0:
+        raise RuntimeError(f"Unsupported kernel size: {c_q}x{c_k} (kernel_size_k must be odd)")
+    if pad_q != c_q - 1 or pad_k != (c_k - 1) // 2:
+        raise RuntimeError(
+            f"pad_q/pad_k must be kernel_size_q-1 and (kernel_size_k-1)//2 "
+            f"(got {pad_q}, {pad_k} for a {c_q}x{c_k} kernel)")
+    if not conv_kernel.is_cuda:
+        raise RuntimeError("conv_kernel must be a CUDA tensor")
+    return conv_kernel.detach().to(device=device, dtype=torch.float32).contiguous()
+
+
+def _desc(Q, K, W, scale, causal, out_dtype, n_splits=1, exact=False) -> _lib.Desc:
+    if out_dtype not in _DT:
+        raise RuntimeError("out_dtype must be bfloat16 or float32")
+    B, H, Nq, d = Q.shape
+    return _lib.Desc(B, H, Nq, K.shape[2], d, W.shape[1], W.shape[2], float(scale), int(bool(causal)),
+                     _DT[Q.dtype], _DT[out_dtype], int(n_splits), _lib.FLAG_EXACT if exact else 0)
+
+
+def _stat(t: torch.Tensor, name: str, like: torch.Tensor) -> torch.Tensor:
+    _check_input(t, name)
+    if tuple(t.shape) != tuple(like.shape[:3]):
+        raise RuntimeError(f"{name} must be [batch, heads, seq_len]")
+    return t if t.dtype == torch.float32 else t.float()
+
+
+def kernel_path(Q, K, conv_kernel, causal=True, op="fwd", exact=False) -> str:
+    """'mfma' or 'fp32': which kernel family a call with these tensors runs."""
+    W = conv_kernel
+    desc = _desc(Q, K, W, 1.0, causal, Q.dtype if Q.dtype in _DT else torch.float32, exact=exact)
+    code = _lib.load().convattn_kernel_path(C.byref(desc), {"fwd": 0, "bwd": 1, "decode": 2}[op])
+    _lib.check(min(code, 0), "convattn_kernel_path")
+    return "mfma" if code == 1 else "fp32"
+
+
+def forward(Q, K, V, conv_kernel, scale, pad_q, pad_k, causal, out_dtype=torch.float32,
+            exact=False) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Training forward -> (O [B,H,N,d], M [B,H,N], L [B,H,N]); M is the row max of
+    the convolved scores and L the sum of exp(C - M)."""
+    _check_qkv(Q, K, V)
+    W = _weights(conv_kernel, Q.shape[1], pad_q, pad_k, Q.device)
+    desc = _desc(Q, K, W, scale, causal, out_dtype, exact=exact)
+    B, H, Nq, d = Q.shape
+    O = torch.empty((B, H, Nq, d), dtype=out_dtype, device=Q.device)
+    M = torch.empty((B, H, Nq), dtype=torch.float32, device=Q.device)
+    L = torch.empty((B, H, Nq), dtype=torch.float32, device=Q.device)
+    rc = _lib.load().convattn_fwd(C.byref(desc), _ptr(Q), _ptr(K), _ptr(V), _ptr(W), _ptr(O), _ptr(M),
+                                  _ptr(L), _stream(Q))
+    _lib.check(rc, "conv_attn.forward")
+    return O, M, L
+
+
+def bwd_preprocess(O, dO, M, L) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(D, LSE) = (rowsum(dO * O), M + log L) in fp32, fused in one kernel."""
+    _check_input(O, "O")
+    _check_input(dO, "dO")
+    B, H, Nq, d = O.shape
+    if dO.shape != O.shape:
+        raise RuntimeError("dO must have the shape of O")
+    if dO.dtype not in _DT or O.dtype not in _DT:
+        raise RuntimeError("O and dO must be bfloat16 or float32")
+    M = _stat(M, "M", O)
+    L = _stat(L, "L", O)
+    desc = _lib.Desc(B, H, Nq, Nq, d, 1, 1, 1.0, 0, _DT[dO.dtype], _DT[O.dtype], 1, 0)
+    D = torch.empty((B, H, Nq), dtype=torch.float32, device=O.device)
+    LSE = torch.empty((B, H, Nq), dtype=torch.float32, device=O.device)
+    rc = _lib.load().convattn_bwd_preprocess(C.byref(desc), _ptr(O), _ptr(dO), _ptr(M), _ptr(L),
+                                             _ptr(D), _ptr(LSE), _stream(O))
+    _lib.check(rc, "conv_attn.bwd_preprocess")
+    return D, LSE
+
+
+def _bwd_common(Q, K, V, dO, D, L, conv_kernel, scale, pad_q, pad_k, causal, out_dtype, exact):
+    _check_qkv(Q, K, V)
+    _check_input(dO, "dO")
+    if dO.shape != Q.shape or dO.dtype != Q.dtype:
+        raise RuntimeError("dO must have the shape and dtype of Q")
+    W = _weights(conv_kernel, Q.shape[1], pad_q, pad_k, Q.device)
+    D = _stat(D, "D", Q)
+    L = _stat(L, "L", Q)
+    return W, D, L, _desc(Q, K, W, scale, causal, out_dtype, exact=exact)
+
+
+def dq_backward(Q, K, V, dO, D, L, conv_kernel, scale, pad_q, pad_k, causal,
+                out_dtype=torch.float32, exact=False) -> Tuple[torch.Tensor, torch.Tensor]:
+    """-> (dQ [B,H,N,d], dconv_kernel [H,c_q,c_k] fp32).  ``L`` is the log-sum-exp
+    M + log L and ``D`` is rowsum(dO * O), as the reference passes them."""
+    W, D, L, desc = _bwd_common(Q, K, V, dO, D, L, conv_kernel, scale, pad_q, pad_k, causal,
+                                out_dtype, exact)
+    lib = _lib.load()
+    dQ = torch.empty(Q.shape, dtype=out_dtype, device=Q.device)
+    nbytes = lib.convattn_dw_partial_bytes(C.byref(desc))
+    if nbytes == 0:
+        _lib.check(lib.convattn_validate(C.byref(desc), _lib.OP_BWD), "conv_attn.dq_backward")
+    part = torch.empty(nbytes // 4, dtype=torch.float32, device=Q.device)
+    dW = torch.empty(W.shape, dtype=torch.float32, device=Q.device)
+    st = _stream(Q)
+    rc = lib.convattn_bwd_dq_dw(C.byref(desc), _ptr(Q), _ptr(K), _ptr(V), _ptr(dO), _ptr(D), _ptr(L),
+                                _ptr(W), _ptr(dQ), _ptr(part), st)
+    _lib.check(rc, "conv_attn.dq_backward")
+    rc = lib.convattn_dw_reduce(C.byref(desc), _ptr(part), _ptr(dW), st)
+    _lib.check(rc, "conv_attn.dq_backward (dW reduce)")
+    return dQ, dW
+
+
+def dkdv_backward(Q, K, V, dO, D, L, conv_kernel, scale, pad_q, pad_k, causal,
+                  out_dtype=torch.float32, exact=False) -> Tuple[torch.Tensor, torch.Tensor]:
+    """-> (dK, dV) [B,H,N,d]; same arguments as ``dq_backward``."""
+    W, D, L, desc = _bwd_common(Q, K, V, dO, D, L, conv_kernel, scale, pad_q, pad_k, causal,
+                                out_dtype, exact)
+    dK = torch.empty(K.shape, dtype=out_dtype, device=Q.device)
+    dV = torch.empty(V.shape, dtype=out_dtype, device=Q.device)
+    rc = _lib.load().convattn_bwd_dkdv(C.byref(desc), _ptr(Q), _ptr(K), _ptr(V), _ptr(dO), _ptr(D),
+                                       _ptr(L), _ptr(W), _ptr(dK), _ptr(dV), _stream(Q))
+    _lib.check(rc, "conv_attn.dkdv_backward")
+    return dK, dV
+
+
+def default_k_splits(B: int, H: int, Nk: int) -> int:
+    """Enough (batch, head, split) workgroups to fill 256 CUs a few times over."""
+    want = max(1, (4 * 256 + B * H - 1) // (B * H))
+    return max(1, min(want, Nk // 256 if Nk >= 256 else 1, 1024))
+
+
+def decode(Q, K, V, conv_kernel, k_splits, scale, causal=False, out_dtype=torch.float32,
+           exact=False, workspace=None):
+    """Decode step -> (O [B,H,1,d], M, L [B,H,1], partials).  Q holds the resident
+    last rows (1..16).  ``k_splits`` None/0 picks a split count from the shape."""
+    _check_qkv(Q, K, V)
+    B, H, r, d = Q.shape
+    c_q, c_k = conv_kernel.shape[1], conv_kernel.shape[2]
+    W = _weights(conv_kernel, H, c_q - 1, (c_k - 1) // 2, Q.device)
+    if not k_splits:
+        k_splits = default_k_splits(B, H, K.shape[2])
+    desc = _desc(Q, K, W, scale, causal, out_dtype, n_splits=k_splits, exact=exact)
+    lib = _lib.load()
+    rc = lib.convattn_validate(C.byref(desc), _lib.OP_DECODE)
+    if rc == _lib.ERR_QROWS:
+        raise ValueError(f"Q sequence length must be <= 16 for inference, got {r}")
+    _lib.check(rc, "conv_attn.forward_inference")
+    if workspace is None:
+        O_part = torch.empty((B, H, k_splits, d), dtype=torch.float32, device=Q.device)
+        M_part = torch.empty((B, H, k_splits), dtype=torch.float32, device=Q.device)
+        L_part = torch.empty((B, H, k_splits), dtype=torch.float32, device=Q.device)
+    else:
+        O_part, M_part, L_part = workspace
+    O = torch.empty((B, H, 1, d), dtype=out_dtype, device=Q.device)
+    M = torch.empty((B, H, 1), dtype=torch.float32, device=Q.device)
+    L = torch.empty((B, H, 1), dtype=torch.float32, device=Q.device)
+    st = _stream(Q)
+    rc = lib.convattn_decode(C.byref(desc), _ptr(Q), _ptr(K), _ptr(V), _ptr(W), _ptr(O_part),
+                             _ptr(M_part), _ptr(L_part), st)
+    _lib.check(rc, "conv_attn.forward_inference")
+    rc = lib.convattn_decode_combine(C.byref(desc), _ptr(O_part), _ptr(M_part), _ptr(L_part), _ptr(O),
+                                     _ptr(M), _ptr(L), st)
+    _lib.check(rc, "conv_attn.forward_inference (combine)")
+    return O, M, L, (O_part, M_part, L_part)
+
+
+def forward_inference(Q, K, V, conv_kernel, k_splits, scale, pad_q, pad_k, causal,
+                      num_k_blocks=None):
+    """Reference-shaped decode op -> (O [B,H,k_splits,d], M, L [B,H,k_splits]) fp32
+    whose slot 0 holds the merged, normalised result (the other slots keep the
+    per-split partials).  ``num_k_blocks`` is accepted and ignored: tiling is
+    chosen by the kernel."""
+    if k_splits is None or k_splits <= 0:
+        raise RuntimeError("k_splits must be positive")
+    if Q.dim() == 4 and not (0 < Q.shape[2] <= 16):
+        raise RuntimeError("Q sequence length must be between 1 and 16 for inference")
+    _weights(conv_kernel, Q.shape[1], pad_q, pad_k, Q.device)  # checks pad_q / pad_k
+    O, M, L, (O_part, M_part, L_part) = decode(Q, K, V, conv_kernel, k_splits, scale, causal)
+    O_part[:, :, 0, :] = O[:, :, 0, :]
+    M_part[:, :, 0] = M[:, :, 0]
+    L_part[:, :, 0] = L[:, :, 0]
+    return O_part, M_part, L_part

@@ -1,0 +1,187 @@
+// C ABI of the conv-attention library: host-side argument checks, kernel-family
+// selection and launches.  Nothing here allocates or synchronises.
+#include <math.h>
+#include <string.h>
+
+#include "common.hpp"
+
+using namespace convattn;
+
+namespace {
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int check_dtype(int dt) { return (dt == CONVATTN_BF16 || dt == CONVATTN_F32) ? 0 : CONVATTN_ERR_DTYPE; }
+
+int validate(const convattn_desc *d, int op, Problem *out) {
+    if (!d) return CONVATTN_ERR_NULL;
+    if (op != CONVATTN_OP_FWD && op != CONVATTN_OP_BWD && op != CONVATTN_OP_DECODE)
+        return CONVATTN_ERR_SHAPE;
+    if (d->B <= 0 || d->H <= 0 || d->Nq <= 0 || d->Nk <= 0 || d->d <= 0) return CONVATTN_ERR_SHAPE;
+    if (d->d % 8 != 0 || d->d > kMaxD) return CONVATTN_ERR_HEAD_DIM;
+    if (d->c_q < 1 || d->c_q > kMaxCq || d->c_k < 1 || d->c_k > kMaxCk || d->c_k % 2 == 0)
+        return CONVATTN_ERR_KERNEL_SIZE;
+    if (check_dtype(d->in_dtype) || check_dtype(d->out_dtype)) return CONVATTN_ERR_DTYPE;
+    if (!isfinite(d->scale)) return CONVATTN_ERR_SCALE;
+    if ((long long)d->B * d->H > 0x7fffffffLL / 64) return CONVATTN_ERR_TOO_LARGE;
+    if (d->B > 65535 || d->H > 65535) return CONVATTN_ERR_TOO_LARGE;
+    Problem p;
+    p.B = d->B; p.H = d->H; p.Nq = d->Nq; p.Nk = d->Nk; p.d = d->d;
+    p.c_q = d->c_q; p.c_k = d->c_k; p.pq = d->c_q - 1; p.pk = (d->c_k - 1) / 2;
+    p.scale = d->scale; p.causal = d->causal ? 1 : 0; p.n_splits = 1;
+    if (op == CONVATTN_OP_DECODE) {
+        if (d->Nq > 16) return CONVATTN_ERR_QROWS;
+        if (d->n_splits < 1 || d->n_splits > d->Nk || d->n_splits > 1024) return CONVATTN_ERR_SPLITS;
+        p.n_splits = d->n_splits;
+        if (generic_decode_lds(p) > kLdsBytes) return CONVATTN_ERR_LDS;
+    } else {
+        if (p.causal && d->Nq != d->Nk) return CONVATTN_ERR_CAUSAL_SHAPE;
+        const size_t lds = (op == CONVATTN_OP_FWD) ? generic_fwd_lds(p) : generic_bwd_lds(p);
+        if (lds > kLdsBytes) return CONVATTN_ERR_LDS;
+    }
+    if (out) *out = p;
+    return CONVATTN_OK;
+}
+
+// 0 = fp32-arithmetic kernels, 1 = bf16 MFMA kernels.
+int pick_path(const convattn_desc *d, const Problem &p, int op) {
+    (void)d; (void)p; (void)op;
+    return 0;
+}
+
+int dw_tiles(const convattn_desc *d, const Problem &p) {
+    (void)d;
+    return generic_q_tiles(p);
+}
+
+#define REQUIRE_PTR(x)                                   \
+    do {                                                 \
+        if (!(x)) return CONVATTN_ERR_NULL;              \
+        if (!aligned16(x)) return CONVATTN_ERR_ALIGN;    \
+    } while (0)
+
+}  // namespace
+
+extern "C" {
+
+int convattn_version(void) { return CONVATTN_VERSION; }
+
+const char *convattn_strerror(int code) {
+    switch (code) {
+        case CONVATTN_OK: return "ok";
+        case CONVATTN_ERR_NULL: return "a required pointer is NULL";
+        case CONVATTN_ERR_SHAPE: return "B, H, Nq, Nk and d must be positive";
+        case CONVATTN_ERR_HEAD_DIM: return "Unsupported head dimension: d must be a multiple of 8 and at most 128";
+        case CONVATTN_ERR_KERNEL_SIZE: return "Unsupported kernel size: c_q must be in 1..16 and c_k odd in 1..33";
+        case CONVATTN_ERR_DTYPE: return "tensors must be bfloat16 or float32";
+        case CONVATTN_ERR_ALIGN: return "device pointers must be 16-byte aligned";
+        case CONVATTN_ERR_SPLITS: return "k_splits must be positive and cannot be larger than seq_len_k (or 1024)";
+        case CONVATTN_ERR_QROWS: return "Q sequence length must be between 1 and 16 for inference";
+        case CONVATTN_ERR_SCALE: return "scale must be finite";
+        case CONVATTN_ERR_CAUSAL_SHAPE: return "causal conv-attention needs seq_len_q == seq_len_k";
+        case CONVATTN_ERR_LDS: return "convolution window too large for the 160 KB of LDS at this head dimension";
+        case CONVATTN_ERR_TOO_LARGE: return "batch or head count too large for one launch";
+        default: break;
+    }
+    if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
+    return "unknown convattn status";
+}
+
+int convattn_validate(const convattn_desc *desc, int op) { return validate(desc, op, nullptr); }
+
+int convattn_kernel_path(const convattn_desc *desc, int op) {
+    Problem p;
+    int rc = validate(desc, op, &p);
+    if (rc) return rc;
+    return pick_path(desc, p, op);
+}
+
+int convattn_fwd(const convattn_desc *desc, const void *q, const void *k, const void *v,
+                 const float *w, void *o, float *m, float *l, void *stream) {
+    Problem p;
+    int rc = validate(desc, CONVATTN_OP_FWD, &p);
+    if (rc) return rc;
+    REQUIRE_PTR(q); REQUIRE_PTR(k); REQUIRE_PTR(v); REQUIRE_PTR(w);
+    REQUIRE_PTR(o); REQUIRE_PTR(m); REQUIRE_PTR(l);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return (int)generic_fwd(p, desc->in_dtype, desc->out_dtype, q, k, v, w, o, m, l, s);
+}
+
+int convattn_bwd_preprocess(const convattn_desc *desc, const void *o, const void *d_o,
+                            const float *m, const float *l, float *D, float *lse, void *stream) {
+    Problem p;
+    int rc = validate(desc, CONVATTN_OP_BWD, &p);
+    if (rc) return rc;
+    REQUIRE_PTR(o); REQUIRE_PTR(d_o); REQUIRE_PTR(m); REQUIRE_PTR(l); REQUIRE_PTR(D); REQUIRE_PTR(lse);
+    return (int)bwd_preprocess(p, desc->in_dtype, desc->out_dtype, o, d_o, m, l, D, lse,
+                               static_cast<hipStream_t>(stream));
+}
+
+size_t convattn_dw_partial_bytes(const convattn_desc *desc) {
+    Problem p;
+    if (validate(desc, CONVATTN_OP_BWD, &p)) return 0;
+    return (size_t)p.B * p.H * dw_tiles(desc, p) * p.c_q * p.c_k * sizeof(float);
+}
+
+int convattn_bwd_dq_dw(const convattn_desc *desc, const void *q, const void *k, const void *v,
+                       const void *d_o, const float *D, const float *lse, const float *w, void *dq,
+                       float *dw_partial, void *stream) {
+    Problem p;
+    int rc = validate(desc, CONVATTN_OP_BWD, &p);
+    if (rc) return rc;
+    REQUIRE_PTR(q); REQUIRE_PTR(k); REQUIRE_PTR(v); REQUIRE_PTR(d_o); REQUIRE_PTR(D);
+    REQUIRE_PTR(lse); REQUIRE_PTR(w); REQUIRE_PTR(dq); REQUIRE_PTR(dw_partial);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return (int)generic_bwd_dq_dw(p, desc->in_dtype, desc->out_dtype, q, k, v, d_o, D, lse, w, dq,
+                                  dw_partial, s);
+}
+
+int convattn_dw_reduce(const convattn_desc *desc, const float *dw_partial, float *dw, void *stream) {
+    Problem p;
+    int rc = validate(desc, CONVATTN_OP_BWD, &p);
+    if (rc) return rc;
+    REQUIRE_PTR(dw_partial); REQUIRE_PTR(dw);
+    return (int)dw_reduce(p, dw_tiles(desc, p), dw_partial, dw, static_cast<hipStream_t>(stream));
+}
+
+int convattn_bwd_dkdv(const convattn_desc *desc, const void *q, const void *k, const void *v,
+                      const void *d_o, const float *D, const float *lse, const float *w, void *dk,
+                      void *dv, void *stream) {
+    Problem p;
+    int rc = validate(desc, CONVATTN_OP_BWD, &p);
+    if (rc) return rc;
+    REQUIRE_PTR(q); REQUIRE_PTR(k); REQUIRE_PTR(v); REQUIRE_PTR(d_o); REQUIRE_PTR(D);
+    REQUIRE_PTR(lse); REQUIRE_PTR(w); REQUIRE_PTR(dk); REQUIRE_PTR(dv);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return (int)generic_bwd_dkdv(p, desc->in_dtype, desc->out_dtype, q, k, v, d_o, D, lse, w, dk, dv, s);
+}
+
+size_t convattn_decode_partial_bytes(const convattn_desc *desc) {
+    Problem p;
+    if (validate(desc, CONVATTN_OP_DECODE, &p)) return 0;
+    return (size_t)p.B * p.H * p.n_splits * p.d * sizeof(float);
+}
+
+int convattn_decode(const convattn_desc *desc, const void *q, const void *k, const void *v,
+                    const float *w, float *o_part, float *m_part, float *l_part, void *stream) {
+    Problem p;
+    int rc = validate(desc, CONVATTN_OP_DECODE, &p);
+    if (rc) return rc;
+    REQUIRE_PTR(q); REQUIRE_PTR(k); REQUIRE_PTR(v); REQUIRE_PTR(w);
+    REQUIRE_PTR(o_part); REQUIRE_PTR(m_part); REQUIRE_PTR(l_part);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return (int)generic_decode(p, desc->in_dtype, q, k, v, w, o_part, m_part, l_part, s);
+}
+
+int convattn_decode_combine(const convattn_desc *desc, const float *o_part, const float *m_part,
+                            const float *l_part, void *o, float *m, float *l, void *stream) {
+    Problem p;
+    int rc = validate(desc, CONVATTN_OP_DECODE, &p);
+    if (rc) return rc;
+    REQUIRE_PTR(o_part); REQUIRE_PTR(m_part); REQUIRE_PTR(l_part);
+    REQUIRE_PTR(o); REQUIRE_PTR(m); REQUIRE_PTR(l);
+    return (int)decode_combine(p, desc->out_dtype, o_part, m_part, l_part, o, m, l,
+                               static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,95 @@
+// Small bandwidth-bound helpers around the conv-attention kernels:
+// backward preparation (D, LSE), the ordered dW reduction and the decode
+// split merge.
+#include "common.hpp"
+
+namespace convattn {
+namespace {
+
+// One wave per query row: D = <dO, O>, LSE = M + log L.
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void preprocess_kernel(size_t rows, int d, const TO *__restrict__ O,
+                                                         const TI *__restrict__ dO,
+                                                         const float *__restrict__ M,
+                                                         const float *__restrict__ L,
+                                                         float *__restrict__ D, float *__restrict__ LSE) {
+    const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (row >= rows) return;
+    float s = 0.f;
+    for (int c = lane; c < d; c += kWave) s = fmaf(to_f32(O[row * d + c]), to_f32(dO[row * d + c]), s);
+    s = wave_sum(s);
+    if (lane == 0) {
+        D[row] = s;
+        LSE[row] = M[row] + __logf(L[row]);
+    }
+}
+
+// dW[h][tap] = sum over (batch, tile) of the partials, in index order.
+__global__ void dw_reduce_kernel(int B, int H, int n_tiles, int ntap, const float *__restrict__ part,
+                                 float *__restrict__ dW) {
+    const int h = blockIdx.x;
+    for (int tap = threadIdx.x; tap < ntap; tap += blockDim.x) {
+        float s = 0.f;
+        for (int b = 0; b < B; ++b) {
+            const float *src = part + ((size_t)b * H + h) * n_tiles * ntap + tap;
+            for (int t = 0; t < n_tiles; ++t) s += src[(size_t)t * ntap];
+        }
+        dW[(size_t)h * ntap + tap] = s;
+    }
+}
+
+// One workgroup per (batch, head): m = max m_s, l = sum l_s e^{m_s - m},
+// o = sum o_s e^{m_s - m} / l.
+template <typename TO>
+__global__ void combine_kernel(int n_splits, int d, const float *__restrict__ O_part,
+                               const float *__restrict__ M_part, const float *__restrict__ L_part,
+                               TO *__restrict__ O, float *__restrict__ M, float *__restrict__ L) {
+    const size_t bh = blockIdx.x;
+    const float *mp = M_part + bh * n_splits;
+    const float *lp = L_part + bh * n_splits;
+    float m = kNegInf;
+    for (int s = 0; s < n_splits; ++s) m = fmaxf(m, mp[s]);
+    float l = 0.f;
+    for (int s = 0; s < n_splits; ++s) l += (mp[s] == kNegInf) ? 0.f : lp[s] * __expf(mp[s] - m);
+    for (int c = threadIdx.x; c < d; c += blockDim.x) {
+        float o = 0.f;
+        for (int s = 0; s < n_splits; ++s)
+            if (mp[s] != kNegInf) o = fmaf(O_part[(bh * n_splits + s) * d + c], __expf(mp[s] - m), o);
+        O[bh * d + c] = from_f32<TO>(o / l);
+    }
+    if (threadIdx.x == 0) { M[bh] = m; L[bh] = l; }
+}
+
+}  // namespace
+
+hipError_t bwd_preprocess(const Problem &p, int in_dt, int out_dt, const void *o, const void *d_o,
+                          const float *m, const float *l, float *D, float *lse, hipStream_t s) {
+    const size_t rows = (size_t)p.B * p.H * p.Nq;
+    const unsigned grid = (unsigned)((rows + 3) / 4);
+#define CALL(TI, TO) \
+    preprocess_kernel<TI, TO><<<grid, 256, 0, s>>>(rows, p.d, (const TO *)o, (const TI *)d_o, m, l, D, lse)
+    if (in_dt == CONVATTN_BF16 && out_dt == CONVATTN_BF16) CALL(bf16_t, bf16_t);
+    else if (in_dt == CONVATTN_BF16) CALL(bf16_t, float);
+    else if (out_dt == CONVATTN_BF16) CALL(float, bf16_t);
+    else CALL(float, float);
+#undef CALL
+    return hipGetLastError();
+}
+
+hipError_t dw_reduce(const Problem &p, int n_tiles, const float *dw_part, float *dw, hipStream_t s) {
+    dw_reduce_kernel<<<p.H, 256, 0, s>>>(p.B, p.H, n_tiles, p.c_q * p.c_k, dw_part, dw);
+    return hipGetLastError();
+}
+
+hipError_t decode_combine(const Problem &p, int out_dt, const float *o_part, const float *m_part,
+                          const float *l_part, void *o, float *m, float *l, hipStream_t s) {
+    const unsigned grid = (unsigned)(p.B * p.H);
+    if (out_dt == CONVATTN_BF16)
+        combine_kernel<bf16_t><<<grid, 128, 0, s>>>(p.n_splits, p.d, o_part, m_part, l_part, (bf16_t *)o, m, l);
+    else
+        combine_kernel<float><<<grid, 128, 0, s>>>(p.n_splits, p.d, o_part, m_part, l_part, (float *)o, m, l);
+    return hipGetLastError();
+}
+
+}  // namespace convattn

@@ -1,0 +1,178 @@
+/*
+ * convattn.h - C ABI of the MI355X (gfx950) fused conv-attention library.
+ *
+ * Conv-attention: scores S = scale * Q K^T pass through a per-head causal 2-D
+ * cross-correlation over a (c_q x c_k) query/key window before the softmax:
+ *
+ *   S_m[i,j] = S[i,j]                       (0 where causal and j > i)
+ *   C[i,j]   = sum_{a<c_q} sum_{b<c_k} W[h,a,b] * S_m[i+a-(c_q-1), j+b-(c_k-1)/2]
+ *   C[i,j]   = -inf where causal and j > i
+ *   M = rowmax C, L = rowsum exp(C-M), O = softmax(C) V
+ *
+ * Conventions
+ *   - Every tensor pointer is a DEVICE address of a dense row-major array:
+ *     Q [B,H,Nq,d], K,V [B,H,Nk,d], W [H,c_q,c_k] (always fp32), statistics
+ *     M, L, D, LSE [B,H,Nq] (always fp32).  Pointers must be 16-byte aligned.
+ *   - The library never allocates, frees or keeps device memory: the caller
+ *     owns inputs, outputs and the partial buffers whose sizes the
+ *     *_partial_bytes() queries return.
+ *   - Every launch is asynchronous on the hipStream_t passed as `stream`
+ *     (NULL = the null stream); no entry point synchronises the device.
+ *   - Return value: 0 = ok, < 0 = convattn_status (argument rejected before any
+ *     HIP call), > 0 = hipError_t of a failed launch.
+ *   - The functions are re-entrant and keep no state between calls.
+ *
+ * Each entry point names the interface of Gusanidas/flash-multi-token-attention
+ * that it replaces (paths relative to flash_multi_token_attention/).
+ */
+#ifndef CONVATTN_H
+#define CONVATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CONVATTN_VERSION 100 /* major*10000 + minor*100 + patch */
+
+typedef enum convattn_dtype {
+    CONVATTN_BF16 = 0,
+    CONVATTN_F32 = 1
+} convattn_dtype;
+
+typedef enum convattn_op {
+    CONVATTN_OP_FWD = 0,
+    CONVATTN_OP_BWD = 1,
+    CONVATTN_OP_DECODE = 2
+} convattn_op;
+
+typedef enum convattn_status {
+    CONVATTN_OK = 0,
+    CONVATTN_ERR_NULL = -1,        /* a required pointer is NULL */
+    CONVATTN_ERR_SHAPE = -2,       /* B, H, Nq, Nk or d not positive / mismatched */
+    CONVATTN_ERR_HEAD_DIM = -3,    /* d not a multiple of 8 or > 128 */
+    CONVATTN_ERR_KERNEL_SIZE = -4, /* c_q not in 1..16, c_k even or not in 1..33 */
+    CONVATTN_ERR_DTYPE = -5,       /* unknown dtype code */
+    CONVATTN_ERR_ALIGN = -6,       /* pointer not 16-byte aligned */
+    CONVATTN_ERR_SPLITS = -7,      /* decode: n_splits not in 1..Nk (or > 1024) */
+    CONVATTN_ERR_QROWS = -8,       /* decode: resident query rows not in 1..16 */
+    CONVATTN_ERR_SCALE = -9,       /* scale is not finite */
+    CONVATTN_ERR_CAUSAL_SHAPE = -10, /* causal training pass needs Nq == Nk */
+    CONVATTN_ERR_LDS = -11,        /* the window needs more LDS than a CU has */
+    CONVATTN_ERR_TOO_LARGE = -12   /* a launch dimension would overflow */
+} convattn_status;
+
+/* Flags for convattn_desc.flags */
+#define CONVATTN_FLAG_EXACT 1u /* force the fp32-arithmetic kernels (no MFMA, no
+                                  fp16 score tile); what "fp32 mode" runs */
+
+/*
+ * Problem descriptor (plain data, passed by pointer, read during the call only).
+ * Training passes: Nq == Nk when causal.  Decode: Nq = number of resident query
+ * rows (the last Nq positions, 1..16), Nk = KV-cache length; one output row.
+ */
+typedef struct convattn_desc {
+    int32_t B, H, Nq, Nk, d;
+    int32_t c_q, c_k;   /* window: c_q query taps (pad_q = c_q-1 rows back),
+                           c_k key taps (pad_k = (c_k-1)/2 either side, c_k odd) */
+    float scale;        /* softmax scale, usually 1/sqrt(d) */
+    int32_t causal;     /* 0 / 1 */
+    int32_t in_dtype;   /* Q, K, V, dO */
+    int32_t out_dtype;  /* O, dQ, dK, dV */
+    int32_t n_splits;   /* decode only: partitions of the key range (>= 1) */
+    uint32_t flags;
+} convattn_desc;
+
+/* Library version (CONVATTN_VERSION it was built from). */
+int convattn_version(void);
+
+/* Text for a return code of this library (negative) or of HIP (positive). */
+const char *convattn_strerror(int code);
+
+/*
+ * Host-only argument check for one operation; touches no GPU state.  Mirrors the
+ * TORCH_CHECKs of conv_attn/kernels/fwd_wrapper.cu:25-33,72,94,
+ * dq_bwd_wrapper.cu:25-43 and fwd_inference_wrapper.cu:25-66.
+ */
+int convattn_validate(const convattn_desc *desc, int op);
+
+/*
+ * Which kernel family a call with this descriptor runs: 0 = fp32-arithmetic
+ * kernels, 1 = bf16 MFMA kernels.  Negative = convattn_status.
+ */
+int convattn_kernel_path(const convattn_desc *desc, int op);
+
+/*
+ * Training forward.  Replaces flash_conv_attention_forward
+ * (conv_attn/kernels/fwd_wrapper.cu:15-100, bound as `forward` in
+ * conv_attn/bindings.cpp:46-48) and fwd_kernel (conv_attn/kernels/fwd.cu:21-310).
+ * Writes O [B,H,Nq,d] (out_dtype), M, L [B,H,Nq] fp32.
+ */
+int convattn_fwd(const convattn_desc *desc, const void *q, const void *k, const void *v,
+                 const float *w, void *o, float *m, float *l, void *stream);
+
+/*
+ * Backward preparation: D = rowsum(dO * O), LSE = M + log L, both fp32.  Replaces
+ * the unfused torch ops of FlashConvAttentionCUDAFunction.backward
+ * (conv_attn/conv_attention_cuda.py:130,144).  `o` is out_dtype, `d_o` in_dtype.
+ */
+int convattn_bwd_preprocess(const convattn_desc *desc, const void *o, const void *d_o,
+                            const float *m, const float *l, float *D, float *lse,
+                            void *stream);
+
+/* Bytes of the dW partial buffer convattn_bwd_dq_dw writes (0 on a bad descriptor). */
+size_t convattn_dw_partial_bytes(const convattn_desc *desc);
+
+/*
+ * dQ and the per-tile partial sums of dW.  Replaces flash_conv_attention_dq_backward
+ * (conv_attn/kernels/dq_bwd_wrapper.cu:11-93, bound as `dq_backward` in
+ * conv_attn/bindings.cpp:50-52) and dq_kernel (conv_attn/kernels/dq_bwd.cu:20-587).
+ * The reference adds dW with float atomics (dq_bwd.cu:498-501); here every tile
+ * stores its own partial and convattn_dw_reduce sums them in a fixed order.
+ */
+int convattn_bwd_dq_dw(const convattn_desc *desc, const void *q, const void *k, const void *v,
+                       const void *d_o, const float *D, const float *lse, const float *w,
+                       void *dq, float *dw_partial, void *stream);
+
+/* dW [H,c_q,c_k] fp32 = ordered sum of the partials over batch and query tiles. */
+int convattn_dw_reduce(const convattn_desc *desc, const float *dw_partial, float *dw,
+                       void *stream);
+
+/*
+ * dK and dV.  Replaces flash_conv_attention_dkdv_backward
+ * (conv_attn/kernels/dkdv_wrapper.cu:12-89, bound as `dkdv_backward` in
+ * conv_attn/bindings.cpp:54-56) and dk_dv_kernel (conv_attn/kernels/dkdv_kernel.cu:18-527).
+ */
+int convattn_bwd_dkdv(const convattn_desc *desc, const void *q, const void *k, const void *v,
+                      const void *d_o, const float *D, const float *lse, const float *w,
+                      void *dk, void *dv, void *stream);
+
+/* Bytes of o_part (fp32 [B,H,n_splits,d]); m_part and l_part are fp32 [B,H,n_splits]. */
+size_t convattn_decode_partial_bytes(const convattn_desc *desc);
+
+/*
+ * Decode step over a KV cache: un-normalised per-split partials of the last
+ * query row.  Replaces flash_conv_attention_inference
+ * (conv_attn/kernels/fwd_inference_wrapper.cu:13-120, bound as
+ * `forward_inference` in conv_attn/fwd_inference_bindings.cpp:20-23) and
+ * fwd_inference_kernel (conv_attn/kernels/fwd_inference.cu:19-283).
+ * q is [B,H,Nq,d] with Nq resident rows (no front padding needed).
+ */
+int convattn_decode(const convattn_desc *desc, const void *q, const void *k, const void *v,
+                    const float *w, float *o_part, float *m_part, float *l_part, void *stream);
+
+/*
+ * Log-sum-exp merge of the split partials into O [B,H,1,d] (out_dtype), M, L
+ * [B,H,1] fp32.  Replaces combine_splits_kernel (conv_attn/kernels/
+ * fwd_inference.cu:286-369); unlike the reference it also runs for n_splits == 1,
+ * so O is always normalised.
+ */
+int convattn_decode_combine(const convattn_desc *desc, const float *o_part, const float *m_part,
+                            const float *l_part, void *o, float *m, float *l, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CONVATTN_H */

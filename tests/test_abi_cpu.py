@@ -1,0 +1,132 @@
+"""Host-only checks of the C ABI: the library loads without a GPU, exports every
+symbol include/convattn.h declares, and rejects bad descriptors with the
+documented status codes before touching the device."""
+import ctypes as C
+import os
+import re
+
+import pytest
+import torch
+
+from flash_multi_token_attention_amd import _lib
+from flash_multi_token_attention_amd.conv_attn import ops, fwd_conv_attn_inference, ConvAttentionCUDA
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(_lib.LIB_PATH):
+        from flash_multi_token_attention_amd import build
+        build.build(verbose=False)
+    return _lib.load()
+
+
+def desc(**kw):
+    base = dict(B=2, H=4, Nq=128, Nk=128, d=64, c_q=6, c_k=11, scale=0.125, causal=1,
+                in_dtype=_lib.BF16, out_dtype=_lib.BF16, n_splits=1, flags=0)
+    base.update(kw)
+    return _lib.Desc(**base)
+
+
+def test_header_symbols_are_exported(lib):
+    text = open(os.path.join(ROOT, "include", "convattn.h")).read()
+    declared = set(re.findall(r"^(?:int|size_t|const char \*)\s*(convattn_[a-z_]+)\s*\(", text, re.M))
+    assert declared, "no declarations parsed"
+    assert declared == set(_lib.EXPORTS)
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.convattn_version() == 100
+
+
+def test_desc_layout_matches_header():
+    # 7 int32, float, 4 int32, uint32 -> 13 * 4 bytes, no padding
+    assert C.sizeof(_lib.Desc) == 52
+
+
+@pytest.mark.parametrize("kw,op,code", [
+    (dict(), _lib.OP_FWD, 0),
+    (dict(), _lib.OP_BWD, 0),
+    (dict(B=0), _lib.OP_FWD, -2),
+    (dict(Nk=-1), _lib.OP_FWD, -2),
+    (dict(d=60), _lib.OP_FWD, -3),
+    (dict(d=256), _lib.OP_FWD, -3),
+    (dict(c_k=10), _lib.OP_FWD, -4),
+    (dict(c_q=17), _lib.OP_FWD, -4),
+    (dict(c_k=35), _lib.OP_BWD, -4),
+    (dict(in_dtype=7), _lib.OP_FWD, -5),
+    (dict(out_dtype=-1), _lib.OP_BWD, -5),
+    (dict(scale=float("nan")), _lib.OP_FWD, -9),
+    (dict(Nq=64), _lib.OP_FWD, -10),
+    (dict(Nq=64, causal=0), _lib.OP_FWD, 0),
+    (dict(Nq=6, Nk=8192, causal=0, n_splits=4), _lib.OP_DECODE, 0),
+    (dict(Nq=17, Nk=8192, causal=0), _lib.OP_DECODE, -8),
+    (dict(Nq=6, Nk=8192, causal=0, n_splits=0), _lib.OP_DECODE, -7),
+    (dict(Nq=6, Nk=100, causal=0, n_splits=101), _lib.OP_DECODE, -7),
+    (dict(Nq=6, Nk=8192, causal=0, n_splits=2000), _lib.OP_DECODE, -7),
+    (dict(B=70000), _lib.OP_FWD, -12),
+])
+def test_validate_codes(lib, kw, op, code):
+    assert lib.convattn_validate(C.byref(desc(**kw)), op) == code
+
+
+def test_null_and_misaligned_pointers_rejected_before_launch(lib):
+    d = desc()
+    null = C.c_void_p(0)
+    ok = C.c_void_p(4096)
+    odd = C.c_void_p(4100)
+    assert lib.convattn_fwd(C.byref(d), null, ok, ok, ok, ok, ok, ok, null) == -1
+    assert lib.convattn_fwd(C.byref(d), ok, ok, odd, ok, ok, ok, ok, null) == -6
+    assert lib.convattn_bwd_dkdv(C.byref(d), ok, ok, ok, ok, ok, ok, ok, ok, null, null) == -1
+    assert lib.convattn_validate(None, 0) == -1
+    assert lib.convattn_dw_partial_bytes(C.byref(desc(d=3))) == 0
+    assert lib.convattn_decode_partial_bytes(C.byref(desc(Nq=6, causal=0, n_splits=8))) == 2 * 4 * 8 * 64 * 4
+
+
+def test_strerror_texts(lib):
+    assert "kernel size" in _lib.strerror(-4)
+    assert "head dimension" in _lib.strerror(-3)
+    assert "between 1 and 16" in _lib.strerror(-8)
+    assert _lib.strerror(0) == "ok"
+    assert _lib.strerror(-999) == "unknown convattn status"
+
+
+def test_dw_partial_size_matches_tiling(lib):
+    n = lib.convattn_dw_partial_bytes(C.byref(desc(in_dtype=_lib.F32)))
+    assert n > 0 and n % (2 * 4 * 66 * 4) == 0
+
+
+def test_python_shim_errors_without_gpu():
+    Q = torch.zeros(1, 2, 8, 64, dtype=torch.bfloat16)
+    W = torch.zeros(2, 3, 3)
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        ops.forward(Q, Q, Q, W, 0.125, 2, 1, True)
+    with pytest.raises(ValueError, match="<= 16"):
+        fwd_conv_attn_inference(torch.zeros(1, 2, 17, 64), Q, Q, W, 1, 0.125, 2, 1, False)
+    with pytest.raises(RuntimeError, match="k_splits must be positive"):
+        ops.forward_inference(Q, Q, Q, W, 0, 0.125, 2, 1, False, 1)
+
+
+def test_module_state_dict_and_init_modes():
+    m = ConvAttentionCUDA(4, 6, 11, init_random=False)
+    assert list(m.state_dict()) == ["conv_weight"]
+    assert m.conv_weight.shape == (4, 6, 11)
+    w = m.conv_weight.detach()
+    assert w.sum() == 4 and (w[:, 5, 5] == 1).all()
+    f = ConvAttentionCUDA(2, 3, 5, init_random=False, init_first=True).conv_weight.detach()
+    assert f.sum() == 2 and (f[:, 0, 0] == 1).all()
+    torch.manual_seed(0)
+    r = ConvAttentionCUDA(8, 7, 7).conv_weight.detach()
+    assert 0.1 < float(r.std()) < 0.3
+    m2 = ConvAttentionCUDA(4, 6, 11)
+    m2.load_state_dict(m.state_dict())
+    assert torch.equal(m2.conv_weight, m.conv_weight)
+
+
+def test_drop_in_import_path():
+    import flash_multi_token_attention as ref_name
+    import flash_multi_token_attention.conv_attn as ca
+    assert ref_name.FlashConvAttention is ConvAttentionCUDA
+    for name in ("FlashConvAttention", "FlashConvAttentionFunction", "forward", "dq_backward",
+                 "dkdv_backward", "fwd_conv_attn", "dq_bwd_conv_attn", "dkdv_bwd_conv_attn"):
+        assert hasattr(ca, name)
