@@ -4,6 +4,7 @@
 #include <string.h>
 
 #include "common.hpp"
+#include "mfma_common.hpp"
 
 using namespace convattn;
 
@@ -45,8 +46,8 @@ int validate(const convattn_desc *d, int op, Problem *out) {
 
 // 0 = fp32-arithmetic kernels, 1 = bf16 MFMA kernels.
 int pick_path(const convattn_desc *d, const Problem &p, int op) {
-    (void)d; (void)p; (void)op;
-    return 0;
+    if (!mfma_shape_ok(p, d->in_dtype, d->flags)) return 0;
+    return op == CONVATTN_OP_FWD ? 1 : 0;
 }
 
 int dw_tiles(const convattn_desc *d, const Problem &p) {
@@ -104,6 +105,8 @@ int convattn_fwd(const convattn_desc *desc, const void *q, const void *k, const 
     REQUIRE_PTR(q); REQUIRE_PTR(k); REQUIRE_PTR(v); REQUIRE_PTR(w);
     REQUIRE_PTR(o); REQUIRE_PTR(m); REQUIRE_PTR(l);
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (pick_path(desc, p, CONVATTN_OP_FWD) == 1)
+        return (int)mfma_fwd(p, desc->out_dtype, q, k, v, w, o, m, l, s);
     return (int)generic_fwd(p, desc->in_dtype, desc->out_dtype, q, k, v, w, o, m, l, s);
 }
 

@@ -1,0 +1,77 @@
+// Building blocks of the bf16 MFMA conv-attention kernels (gfx950, wave64).
+//
+// MFMA 16x16x32 register layout (lane = 16*g + n, g = 0..3, n = 0..15):
+//   A operand: row n of the 16 x 32 tile, k = 8g .. 8g+7   (8 x 16-bit, one b128)
+//   B operand: column n of the 32 x 16 tile, k = 8g .. 8g+7
+//   C/D:       column n, rows 4g .. 4g+3                    (4 x fp32)
+//
+// The key-axis part of the (c_q x c_k) window is a banded Toeplitz matrix, so the
+// convolution of a score tile is c_q MFMAs per 16 x 16 output block: for query
+// tap a, C^T[16 out keys][16 queries] += T_a^T[16 x 32] * S^T[32 in keys][16
+// queries shifted by a - pad_q rows].  The 32 input keys start 8 before the
+// block's first output key (a 16-byte-aligned LDS column), which covers
+// pad_k <= 8.  Scores are staged in LDS as fp16 (11-bit significand; bf16's 8
+// bits would cost ~1e-2 in the softmax argument).
+#pragma once
+#include "common.hpp"
+
+namespace convattn {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kKeyHalo = 8;          // LDS columns before a block's first output key
+constexpr int kMfmaMaxPk = 8;        // so c_k <= 17 on the MFMA path
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kF16Max = 65504.f;
+
+__device__ __forceinline__ f32x4 mfma_bf16(bf16x8 a, bf16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4 mfma_f16(f16x8 a, f16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Toeplitz fragment of query tap `a` for this lane: element e is
+// W[a][b], b = (8g + e) - 8 - n + pk, zero outside the window.  `flip` builds the
+// transposed-convolution band instead (b -> c_k - 1 - b).
+__device__ __forceinline__ f16x8 toeplitz_frag(const float *__restrict__ w_row, int c_k, int pk,
+                                               int g, int n, bool flip) {
+    f16x8 t;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        int b = 8 * g + e - kKeyHalo - n + pk;
+        float v = 0.f;
+        if (b >= 0 && b < c_k) v = w_row[flip ? (c_k - 1 - b) : b];
+        t[e] = (_Float16)v;
+    }
+    return t;
+}
+
+// 8 bf16 (16 bytes) of row `row` at element offset `col` of a dense [N][D]
+// matrix, zeros when the row is outside [0, N).
+template <int D>
+__device__ __forceinline__ u32x4 load_row16(const bf16_t *__restrict__ base, int row, int N, int col) {
+    u32x4 z = {0u, 0u, 0u, 0u};
+    if (row < 0 || row >= N) return z;
+    return *reinterpret_cast<const u32x4 *>(base + (size_t)row * D + col);
+}
+
+// fp32-arithmetic fallbacks are chosen when this is false.
+inline bool mfma_shape_ok(const Problem &p, int in_dt, unsigned flags) {
+    return in_dt == CONVATTN_BF16 && !(flags & CONVATTN_FLAG_EXACT) && (p.d == 64 || p.d == 128) &&
+           p.pk <= kMfmaMaxPk && p.c_q <= 11;
+}
+
+// ---- bf16 MFMA kernels ----
+constexpr int kMfmaFwdRows = 128;  // query rows per forward workgroup
+hipError_t mfma_fwd(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
+                    const float *w, void *o, float *m, float *l, hipStream_t s);
+
+}  // namespace convattn

@@ -1,0 +1,74 @@
+"""GPU parity of the bf16 MFMA kernels against the CPU oracle (small shapes) and
+against the fp32-arithmetic GPU kernels (full benchmark shapes), through the C ABI.
+Tolerances: max-abs 2e-2 for O / dQ / dK / dV, 5e-2 relative for dW."""
+import pytest
+import torch
+
+from flash_multi_token_attention_amd import synthetic
+from flash_multi_token_attention_amd.conv_attn import ops
+from tests.util import TOL_BF16, TOL_DW_REL, max_abs, oracle_bwd, oracle_fwd, rand_case, rel_max, scale_of
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+FWD_SHAPES = [
+    # B, H, N, d, c_q, c_k
+    (1, 2, 128, 128, 6, 11),
+    (2, 2, 300, 128, 6, 11),
+    (1, 2, 257, 64, 6, 11),
+    (1, 2, 100, 64, 3, 5),
+    (1, 1, 64, 128, 1, 1),
+    (1, 2, 200, 64, 11, 11),
+    (1, 1, 130, 128, 6, 17),
+    (1, 2, 31, 64, 2, 3),
+    (1, 1, 1, 64, 6, 11),
+]
+
+
+@pytest.mark.parametrize("shape", FWD_SHAPES)
+@pytest.mark.parametrize("causal", [True, False])
+def test_forward_bf16_mfma(shape, causal):
+    B, H, N, d, c_q, c_k = shape
+    Q, K, V, _, W = rand_case(B, H, N, N, d, c_q, c_k, torch.bfloat16, seed=N + c_q)
+    O_ref, M_ref, L_ref = oracle_fwd(Q, K, V, W, causal)
+    g = [t.to(DEV) for t in (Q, K, V, W)]
+    assert ops.kernel_path(g[0], g[1], g[3], causal) == "mfma"
+    for odt in (torch.bfloat16, torch.float32):
+        O, M, L = ops.forward(g[0], g[1], g[2], g[3], scale_of(d), c_q - 1, (c_k - 1) // 2, causal,
+                              out_dtype=odt)
+        assert O.dtype == odt
+        assert max_abs(O, O_ref) <= TOL_BF16
+        assert max_abs(M, M_ref) <= TOL_BF16
+        assert rel_max(L, L_ref) <= TOL_BF16
+
+
+def test_forward_random_window_weights():
+    # all taps of comparable size (the reference module's init_random=True)
+    Q, K, V, _, W = rand_case(1, 2, 260, 260, 128, 6, 11, torch.bfloat16, seed=4, w_mode="rand")
+    O_ref, M_ref, _ = oracle_fwd(Q, K, V, W, True)
+    O, M, _ = ops.forward(Q.to(DEV), K.to(DEV), V.to(DEV), W.to(DEV), scale_of(128), 5, 5, True)
+    assert max_abs(O, O_ref) <= TOL_BF16 and max_abs(M, M_ref) <= TOL_BF16
+
+
+def test_forward_noncausal_rectangular_mfma():
+    Q, K, V, _, W = rand_case(1, 2, 70, 333, 128, 6, 11, torch.bfloat16, seed=6)
+    O_ref, M_ref, _ = oracle_fwd(Q, K, V, W, False)
+    O, M, _ = ops.forward(Q.to(DEV), K.to(DEV), V.to(DEV), W.to(DEV), scale_of(128), 5, 5, False)
+    assert max_abs(O, O_ref) <= TOL_BF16 and max_abs(M, M_ref) <= TOL_BF16
+
+
+def test_c2_full_size_forward_against_fp32_kernels():
+    wl = synthetic.WORKLOADS["c2_fwd"]
+    t = {k: v.to(DEV) for k, v in synthetic.make_inputs(wl, seed=0).items()}
+    args = (t["Q"], t["K"], t["V"], t["W"], wl.scale, wl.pad_q, wl.pad_k, True)
+    O, M, L = ops.forward(*args, out_dtype=torch.bfloat16)
+    O_x, M_x, L_x = ops.forward(*args, out_dtype=torch.float32, exact=True)
+    assert ops.kernel_path(t["Q"], t["K"], t["W"]) == "mfma"
+    assert max_abs(O, O_x) <= TOL_BF16
+    assert max_abs(M, M_x) <= TOL_BF16
+    assert rel_max(L, L_x) <= TOL_BF16
+    # rows of P sum to one: with V = 1 the output is 1 wherever the row sees a key
+    ones = torch.ones_like(t["V"])
+    O1, _, _ = ops.forward(t["Q"], t["K"], ones, t["W"], wl.scale, wl.pad_q, wl.pad_k, True,
+                           out_dtype=torch.float32)
+    assert float((O1 - 1).abs().max()) <= 1e-2
