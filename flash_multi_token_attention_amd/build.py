@@ -20,7 +20,8 @@ INCLUDE = os.path.join(ROOT, "include")
 LIB_NAME = "libconvattn_hip.so"
 LIB_PATH = os.path.join(PKG_DIR, LIB_NAME)
 
-SOURCES = ["api.hip", "generic_kernels.hip", "reduce_kernels.hip", "fwd_mfma.hip"]
+SOURCES = ["api.hip", "generic_kernels.hip", "reduce_kernels.hip", "fwd_mfma.hip", "bwd_dq_mfma.hip",
+           "bwd_dkdv_mfma.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall",

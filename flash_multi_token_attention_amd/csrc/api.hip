@@ -46,13 +46,13 @@ int validate(const convattn_desc *d, int op, Problem *out) {
 
 // 0 = fp32-arithmetic kernels, 1 = bf16 MFMA kernels.
 int pick_path(const convattn_desc *d, const Problem &p, int op) {
-    if (!mfma_shape_ok(p, d->in_dtype, d->flags)) return 0;
-    return op == CONVATTN_OP_FWD ? 1 : 0;
+    if (op == CONVATTN_OP_FWD) return mfma_shape_ok(p, d->in_dtype, d->flags) ? 1 : 0;
+    if (op == CONVATTN_OP_BWD) return mfma_bwd_shape_ok(p, d->in_dtype, d->flags) ? 1 : 0;
+    return 0;
 }
 
 int dw_tiles(const convattn_desc *d, const Problem &p) {
-    (void)d;
-    return generic_q_tiles(p);
+    return pick_path(d, p, CONVATTN_OP_BWD) == 1 ? mfma_dq_tiles(p) : generic_q_tiles(p);
 }
 
 #define REQUIRE_PTR(x)                                   \
@@ -135,6 +135,8 @@ int convattn_bwd_dq_dw(const convattn_desc *desc, const void *q, const void *k, 
     REQUIRE_PTR(q); REQUIRE_PTR(k); REQUIRE_PTR(v); REQUIRE_PTR(d_o); REQUIRE_PTR(D);
     REQUIRE_PTR(lse); REQUIRE_PTR(w); REQUIRE_PTR(dq); REQUIRE_PTR(dw_partial);
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (pick_path(desc, p, CONVATTN_OP_BWD) == 1)
+        return (int)mfma_bwd_dq_dw(p, desc->out_dtype, q, k, v, d_o, D, lse, w, dq, dw_partial, s);
     return (int)generic_bwd_dq_dw(p, desc->in_dtype, desc->out_dtype, q, k, v, d_o, D, lse, w, dq,
                                   dw_partial, s);
 }
@@ -156,6 +158,8 @@ int convattn_bwd_dkdv(const convattn_desc *desc, const void *q, const void *k, c
     REQUIRE_PTR(q); REQUIRE_PTR(k); REQUIRE_PTR(v); REQUIRE_PTR(d_o); REQUIRE_PTR(D);
     REQUIRE_PTR(lse); REQUIRE_PTR(w); REQUIRE_PTR(dk); REQUIRE_PTR(dv);
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (pick_path(desc, p, CONVATTN_OP_BWD) == 1)
+        return (int)mfma_bwd_dkdv(p, desc->out_dtype, q, k, v, d_o, D, lse, w, dk, dv, s);
     return (int)generic_bwd_dkdv(p, desc->in_dtype, desc->out_dtype, q, k, v, d_o, D, lse, w, dk, dv, s);
 }
 

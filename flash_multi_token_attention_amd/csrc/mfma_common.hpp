@@ -23,6 +23,8 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+// 8 fp16 at any 2-byte boundary (gfx950 LDS reads need no natural alignment)
+struct __attribute__((packed, aligned(2))) F16x8U { f16x8 v; };
 
 constexpr int kKeyHalo = 8;          // LDS columns before a block's first output key
 constexpr int kMfmaMaxPk = 8;        // so c_k <= 17 on the MFMA path
@@ -68,10 +70,23 @@ inline bool mfma_shape_ok(const Problem &p, int in_dt, unsigned flags) {
     return in_dt == CONVATTN_BF16 && !(flags & CONVATTN_FLAG_EXACT) && (p.d == 64 || p.d == 128) &&
            p.pk <= kMfmaMaxPk && p.c_q <= 11;
 }
+// The backward kernels put the key taps on one 16-wide MFMA dimension.
+inline bool mfma_bwd_shape_ok(const Problem &p, int in_dt, unsigned flags) {
+    return mfma_shape_ok(p, in_dt, flags) && p.c_k <= 15;
+}
 
 // ---- bf16 MFMA kernels ----
 constexpr int kMfmaFwdRows = 128;  // query rows per forward workgroup
 hipError_t mfma_fwd(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
                     const float *w, void *o, float *m, float *l, hipStream_t s);
+
+constexpr int kMfmaDqRows = 128;   // query rows per dQ/dW workgroup (= one dW partial)
+inline int mfma_dq_tiles(const Problem &p) { return (p.Nq + kMfmaDqRows - 1) / kMfmaDqRows; }
+hipError_t mfma_bwd_dq_dw(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
+                          const void *d_o, const float *Dl, const float *lse, const float *w, void *dq,
+                          float *dw_part, hipStream_t s);
+hipError_t mfma_bwd_dkdv(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
+                         const void *d_o, const float *Dl, const float *lse, const float *w, void *dk,
+                         void *dv, hipStream_t s);
 
 }  // namespace convattn

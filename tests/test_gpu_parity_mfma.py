@@ -72,3 +72,92 @@ def test_c2_full_size_forward_against_fp32_kernels():
     O1, _, _ = ops.forward(t["Q"], t["K"], ones, t["W"], wl.scale, wl.pad_q, wl.pad_k, True,
                            out_dtype=torch.float32)
     assert float((O1 - 1).abs().max()) <= 1e-2
+
+
+BWD_SHAPES = [
+    # B, H, N, d, c_q, c_k
+    (1, 2, 128, 128, 6, 11),
+    (2, 2, 300, 128, 6, 11),
+    (1, 2, 257, 64, 6, 11),
+    (1, 2, 100, 64, 3, 5),
+    (1, 1, 64, 128, 1, 1),
+    (1, 2, 200, 64, 11, 11),
+    (1, 1, 130, 128, 6, 15),
+    (1, 2, 31, 64, 2, 3),
+    (1, 1, 1, 64, 6, 11),
+]
+
+
+def _run_bwd(Q, K, V, dO, W, causal, odt):
+    d = Q.shape[-1]
+    c_q, c_k = W.shape[1:]
+    sc, pq, pk = scale_of(d), c_q - 1, (c_k - 1) // 2
+    O, M, L = ops.forward(Q, K, V, W, sc, pq, pk, causal, out_dtype=odt)
+    D, LSE = ops.bwd_preprocess(O, dO, M, L)
+    dQ, dW = ops.dq_backward(Q, K, V, dO, D, LSE, W, sc, pq, pk, causal, out_dtype=odt)
+    dK, dV = ops.dkdv_backward(Q, K, V, dO, D, LSE, W, sc, pq, pk, causal, out_dtype=odt)
+    return dQ, dK, dV, dW
+
+
+@pytest.mark.parametrize("shape", BWD_SHAPES)
+@pytest.mark.parametrize("causal", [True, False])
+def test_backward_bf16_mfma(shape, causal):
+    B, H, N, d, c_q, c_k = shape
+    Q, K, V, dO, W = rand_case(B, H, N, N, d, c_q, c_k, torch.bfloat16, seed=3 * N + c_q)
+    ref = oracle_bwd(Q, K, V, W, dO, causal)
+    g = [t.to(DEV) for t in (Q, K, V, dO, W)]
+    assert ops.kernel_path(g[0], g[1], g[4], causal, op="bwd") == "mfma"
+    for odt in (torch.bfloat16, torch.float32):
+        dQ, dK, dV, dW = _run_bwd(*g, causal, odt)
+        assert dQ.dtype == odt and dW.dtype == torch.float32
+        assert max_abs(dQ, ref[0]) <= TOL_BF16
+        assert max_abs(dK, ref[1]) <= TOL_BF16
+        assert max_abs(dV, ref[2]) <= TOL_BF16
+        assert rel_max(dW, ref[3]) <= TOL_DW_REL
+
+
+def test_backward_random_window_weights_and_determinism():
+    Q, K, V, dO, W = rand_case(2, 2, 260, 260, 128, 6, 11, torch.bfloat16, seed=8, w_mode="rand")
+    ref = oracle_bwd(Q, K, V, W, dO, True)
+    g = [t.to(DEV) for t in (Q, K, V, dO, W)]
+    out = _run_bwd(*g, True, torch.bfloat16)
+    for got, want in zip(out[:3], ref[:3]):
+        assert max_abs(got, want) <= TOL_BF16
+    assert rel_max(out[3], ref[3]) <= TOL_DW_REL
+    again = _run_bwd(*g, True, torch.bfloat16)
+    for a, b in zip(out, again):
+        assert torch.equal(a, b)       # no atomics anywhere: bitwise repeatable
+
+
+def test_backward_noncausal_rectangular_mfma():
+    Q, K, V, dO, W = rand_case(1, 2, 70, 333, 128, 6, 11, torch.bfloat16, seed=10)
+    ref = oracle_bwd(Q, K, V, W, dO, False)
+    g = [t.to(DEV) for t in (Q, K, V, dO, W)]
+    out = _run_bwd(*g, False, torch.bfloat16)
+    for got, want in zip(out[:3], ref[:3]):
+        assert max_abs(got, want) <= TOL_BF16
+    assert rel_max(out[3], ref[3]) <= TOL_DW_REL
+
+
+def test_module_autograd_matches_oracle_autograd():
+    from flash_multi_token_attention_amd.conv_attn import ConvAttentionCUDA
+    B, H, N, d, c_q, c_k = 2, 4, 192, 128, 6, 11
+    Q, K, V, dO, W = rand_case(B, H, N, N, d, c_q, c_k, torch.bfloat16, seed=12)
+    mod = ConvAttentionCUDA(H, c_q, c_k, init_random=False).to(DEV)
+    with torch.no_grad():
+        mod.conv_weight.copy_(W)
+    q, k, v = (t.to(DEV).requires_grad_(True) for t in (Q, K, V))
+    O = mod(q, k, v, causal=True)
+    assert O.dtype == torch.bfloat16
+    O.backward(dO.to(DEV))
+    O_ref, _, _ = oracle_fwd(Q, K, V, W, True)
+    ref = oracle_bwd(Q, K, V, W, dO, True)
+    assert max_abs(O.detach(), O_ref) <= TOL_BF16
+    assert max_abs(q.grad, ref[0]) <= TOL_BF16 and max_abs(k.grad, ref[1]) <= TOL_BF16
+    assert max_abs(v.grad, ref[2]) <= TOL_BF16
+    assert rel_max(mod.conv_weight.grad, ref[3]) <= TOL_DW_REL
+    # identity window == plain causal attention
+    ident = ConvAttentionCUDA(H, c_q, c_k, init_random=False).to(DEV)
+    O_id = ident(q.detach(), k.detach(), v.detach())
+    sdpa = torch.nn.functional.scaled_dot_product_attention(Q.float(), K.float(), V.float(), is_causal=True)
+    assert max_abs(O_id, sdpa) <= TOL_BF16
