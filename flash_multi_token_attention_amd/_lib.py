@@ -6,7 +6,8 @@ import os
 import threading
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_PKG, "libconvattn_hip.so")
+# CONVATTN_LIB points at another build of the same C ABI (e.g. an instrumented one).
+LIB_PATH = os.environ.get("CONVATTN_LIB") or os.path.join(_PKG, "libconvattn_hip.so")
 
 BF16, F32 = 0, 1
 OP_FWD, OP_BWD, OP_DECODE = 0, 1, 2

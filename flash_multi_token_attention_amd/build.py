@@ -21,7 +21,7 @@ LIB_NAME = "libconvattn_hip.so"
 LIB_PATH = os.path.join(PKG_DIR, LIB_NAME)
 
 SOURCES = ["api.hip", "generic_kernels.hip", "reduce_kernels.hip", "fwd_mfma.hip", "bwd_dq_mfma.hip",
-           "bwd_dkdv_mfma.hip"]
+           "bwd_dkdv_mfma.hip", "decode_stream.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall",

@@ -48,6 +48,7 @@ int validate(const convattn_desc *d, int op, Problem *out) {
 int pick_path(const convattn_desc *d, const Problem &p, int op) {
     if (op == CONVATTN_OP_FWD) return mfma_shape_ok(p, d->in_dtype, d->flags) ? 1 : 0;
     if (op == CONVATTN_OP_BWD) return mfma_bwd_shape_ok(p, d->in_dtype, d->flags) ? 1 : 0;
+    if (op == CONVATTN_OP_DECODE) return decode_stream_ok(p, d->in_dtype, d->flags) ? 1 : 0;
     return 0;
 }
 
@@ -177,6 +178,8 @@ int convattn_decode(const convattn_desc *desc, const void *q, const void *k, con
     REQUIRE_PTR(q); REQUIRE_PTR(k); REQUIRE_PTR(v); REQUIRE_PTR(w);
     REQUIRE_PTR(o_part); REQUIRE_PTR(m_part); REQUIRE_PTR(l_part);
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (pick_path(desc, p, CONVATTN_OP_DECODE) == 1)
+        return (int)decode_stream(p, q, k, v, w, o_part, m_part, l_part, s);
     return (int)generic_decode(p, desc->in_dtype, q, k, v, w, o_part, m_part, l_part, s);
 }
 

@@ -79,7 +79,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
 
     const int h = blockIdx.y, b = blockIdx.z;
     const int k0 = blockIdx.x * BKW, c0 = k0 + wave * WK;
-    const int pq = p.pq, pk = p.pk, cq = p.c_q, ck = p.c_k;
+    const int pk = p.pk, cq = p.c_q, ck = p.c_k;
     const bool causal = p.causal != 0;
     const size_t bh = (size_t)b * p.H + h;
     const bf16_t *Qb = Q + bh * p.Nq * D;
@@ -90,12 +90,8 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
     const float *dl_b = Dl + bh * p.Nq;
 
     f16x8 tf[CQT], tfl[CQT];
-#pragma unroll
-    for (int a = 0; a < CQT; ++a) {
-        const float *wrow = W + ((size_t)h * cq + (a < cq ? a : 0)) * ck;
-        tf[a] = toeplitz_frag(wrow, ck, pk, g, n, false);
-        tfl[a] = toeplitz_frag(wrow, ck, pk, g, n, true);
-    }
+    load_bands<CQT>(tf, W + (size_t)h * cq * ck, cq, ck, pk, g, n, false);
+    load_bands<CQT>(tfl, W + (size_t)h * cq * ck, cq, ck, pk, g, n, true);
 
     bf16x8 kf[4][KS];  // K rows c0-16 .. c0+47
     bf16x8 vf[3][KS];  // V rows c0-8 .. c0+39
@@ -120,6 +116,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
         }
 
     const float scale = p.scale;
+    const float scale2 = p.scale * kLog2e;  // score tile in log2 units (the window is linear)
     // Causal: rows before the first key this workgroup touches (k0 - 8) see none of its keys.
     const int r_begin = causal ? (max(0, k0 - 8) / BR) * BR : 0;
     for (int r0 = r_begin; r0 < p.Nq; r0 += BR) {
@@ -163,7 +160,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                 f16x4 hv;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    float s = acc[kb][r] * scale;
+                    float s = acc[kb][r] * scale2;
                     if (causal && key0 + r > qpos) s = 0.f;
                     s = fminf(fmaxf(s, -kF16Max), kF16Max);
                     hv[r] = (_Float16)s;
@@ -179,16 +176,14 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
         for (int rb = 0; rb < 3; ++rb) {
             const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(lse_s + rb * 16 + 4 * g);
             const f32x4 dl4 = *reinterpret_cast<const f32x4 *>(dl_s + rb * 16 + 4 * g);
-            const int srow = 16 + rb * 16 + n - pq;
+            const int srow = 16 + rb * 16 + n - (CQT - 1);
 #pragma unroll
             for (int kb = 0; kb < 3; ++kb) {
                 f32x4 c = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int a = 0; a < CQT; ++a) {
-                    if (a < cq) {
-                        f16x8 sf = *reinterpret_cast<const f16x8 *>(Ss + (srow + a) * SST + (kb * 16 + 8 * g) * 2);
-                        c = mfma_f16(sf, tf[a], c);
-                    }
+                    f16x8 sf = *reinterpret_cast<const f16x8 *>(Ss + (srow + a) * SST + (kb * 16 + 8 * g) * 2);
+                    c = mfma_f16(sf, tf[a], c);
                 }
                 f32x4 dp = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -201,7 +196,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int qpos = r0 + rb * 16 + 4 * g + r;
-                    float e = fast_exp2(c[r] * kLog2e - lse4[r]);
+                    float e = fast_exp2(c[r] - lse4[r]);
                     float dc = e * (dp[r] - dl4[r]);
                     if (key < 0 || key >= p.Nk || qpos >= p.Nq || (causal && key > qpos)) { e = 0.f; dc = 0.f; }
                     dc = fminf(fmaxf(dc, -kF16Max), kF16Max);
@@ -241,10 +236,8 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                 f32x4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int a = 0; a < CQT; ++a) {
-                    if (a < cq) {
-                        f16x8 cf = *reinterpret_cast<const f16x8 *>(Cs + (ob * 16 + n + pq - a) * CST + (m * 16 + 8 * g) * 2);
-                        s = mfma_f16(cf, tfl[a], s);
-                    }
+                    f16x8 cf = *reinterpret_cast<const f16x8 *>(Cs + (ob * 16 + n + (CQT - 1) - a) * CST + (m * 16 + 8 * g) * 2);
+                    s = mfma_f16(cf, tfl[a], s);
                 }
                 if (causal) {
                     const int key = c0 + m * 16 + n;

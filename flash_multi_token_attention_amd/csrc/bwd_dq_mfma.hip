@@ -76,13 +76,9 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_mfma_kernel(
     const bf16_t *Vb = V + bh * p.Nk * D;
     const bf16_t *dOb = dO + bh * p.Nq * D;
 
-    f16x8 tf[CQT], tfl[CQT];  // forward band and flipped (transposed-window) band per tap
-#pragma unroll
-    for (int a = 0; a < CQT; ++a) {
-        const float *wrow = W + ((size_t)h * cq + (a < cq ? a : 0)) * ck;
-        tf[a] = toeplitz_frag(wrow, ck, pk, g, n, false);
-        tfl[a] = toeplitz_frag(wrow, ck, pk, g, n, true);
-    }
+    f16x8 tf[CQT], tfl[CQT];  // forward band and flipped (transposed-window) band per tap slot
+    load_bands<CQT>(tf, W + (size_t)h * cq * ck, cq, ck, pk, g, n, false);
+    load_bands<CQT>(tfl, W + (size_t)h * cq * ck, cq, ck, pk, g, n, true);
 
     bf16x8 qf[4][KS];   // Q rows r0-16 .. r0+47
     bf16x8 gf[3][KS];   // dO rows r0 .. r0+47
@@ -111,6 +107,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_mfma_kernel(
     const int bcl = n < ck ? n : ck - 1;  // lanes past the last key tap re-read a valid one
 
     const float scale = p.scale;
+    const float scale2 = p.scale * kLog2e;  // score tile in log2 units (the window is linear)
     const int k_end = causal ? min(p.Nk, i0 + BQ) : p.Nk;
     for (int c0 = 0; c0 < k_end; c0 += BK) {
         __syncthreads();
@@ -154,7 +151,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_mfma_kernel(
                 f16x4 hv;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    float s = acc[rb][r] * scale;
+                    float s = acc[rb][r] * scale2;
                     if (causal && key0 + r > qpos) s = 0.f;
                     s = fminf(fmaxf(s, -kF16Max), kF16Max);
                     hv[r] = (_Float16)s;
@@ -168,17 +165,15 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_mfma_kernel(
 #pragma unroll
         for (int rb = 0; rb < 3; ++rb) {
             const int qpos = r0 + rb * 16 + n;
-            const int srow = 16 + rb * 16 + n - pq;  // S-tile row of tap 0
+            const int srow = 16 + rb * 16 + n - (CQT - 1);  // S-tile row of tap slot 0
 #pragma unroll
             for (int kb = 0; kb < C_COLS / 16; ++kb) {
                 f32x4 c = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int a = 0; a < CQT; ++a) {
-                    if (a < cq) {
-                        // keys c0-8+16kb .. need S keys from 8 before: S-tile column 16kb
-                        f16x8 sf = *reinterpret_cast<const f16x8 *>(Ss + (srow + a) * SST + (kb * 16 + 8 * g) * 2);
-                        c = mfma_f16(tf[a], sf, c);
-                    }
+                    // keys c0-8+16kb .. need S keys from 8 before: S-tile column 16kb
+                    f16x8 sf = *reinterpret_cast<const f16x8 *>(Ss + (srow + a) * SST + (kb * 16 + 8 * g) * 2);
+                    c = mfma_f16(tf[a], sf, c);
                 }
                 f32x4 dp = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -190,7 +185,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_mfma_kernel(
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int key = c0 - 8 + kb * 16 + 4 * g + r;
-                    float pr = fast_exp2(c[r] * kLog2e - lse2[rb]);
+                    float pr = fast_exp2(c[r] - lse2[rb]);
                     float dc = pr * (dp[r] - dl[rb]);
                     if (key < 0 || key >= p.Nk || qpos >= p.Nq || (causal && key > qpos)) dc = 0.f;
                     dc = fminf(fmaxf(dc, -kF16Max), kF16Max);
@@ -211,10 +206,8 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_mfma_kernel(
                 ds[kb] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int a = 0; a < CQT; ++a) {
-                    if (a < cq) {
-                        f16x8 cf = *reinterpret_cast<const f16x8 *>(Cs + (ob * 16 + n + pq - a) * CST + (kb * 16 + 8 * g) * 2);
-                        ds[kb] = mfma_f16(tfl[a], cf, ds[kb]);
-                    }
+                    f16x8 cf = *reinterpret_cast<const f16x8 *>(Cs + (ob * 16 + n + (CQT - 1) - a) * CST + (kb * 16 + 8 * g) * 2);
+                    ds[kb] = mfma_f16(tfl[a], cf, ds[kb]);
                 }
                 if (causal) {
 #pragma unroll
@@ -291,7 +284,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_mfma_kernel(
         float s = 0.f;
 #pragma unroll
         for (int w = 0; w < NW; ++w) s += red[(w * 16 + a) * 16 + bb];
-        dW_part[(bh * gridDim.x + qt) * ntap + tid] = s;
+        dW_part[(bh * gridDim.x + qt) * ntap + tid] = s * (1.f / kLog2e);  // S tile was in log2 units
     }
 }
 

@@ -61,7 +61,7 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_mfma_kernel(
     const int h = blockIdx.y, b = blockIdx.z;
     const int qt = gridDim.x - 1 - blockIdx.x;  // longest (causal) tiles first
     const int i0 = qt * BQ, i0w = i0 + wave * WR;
-    const int pq = p.pq, pk = p.pk, cq = p.c_q;
+    const int pk = p.pk, cq = p.c_q;
     const bool causal = p.causal != 0;
     const size_t bh = (size_t)b * p.H + h;
     const bf16_t *Qb = Q + bh * p.Nq * D;
@@ -70,11 +70,7 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_mfma_kernel(
 
     // Toeplitz bands of this head, one fragment per query tap.
     f16x8 tf[CQT];
-#pragma unroll
-    for (int a = 0; a < CQT; ++a) {
-        if (a < cq) tf[a] = toeplitz_frag(W + ((size_t)h * cq + a) * p.c_k, p.c_k, pk, g, n, false);
-        else tf[a] = (f16x8)(_Float16)0.f;
-    }
+    load_bands<CQT>(tf, W + (size_t)h * cq * p.c_k, cq, p.c_k, pk, g, n, false);
 
     // Q^T fragments (B operand): rows i0w-16 .. i0w+31, resident for the whole loop.
     bf16x8 qf[3][KS];
@@ -94,7 +90,7 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_mfma_kernel(
     float m_run[2] = {kNegInf, kNegInf};  // running max, in log2 units (C * log2 e)
     float l_run[2] = {0.f, 0.f};          // this lane's share of the row sum
 
-    const float scale = p.scale;
+    const float scale = p.scale * kLog2e;  // scores are kept in log2 units: the window is linear
     const int k_end = causal ? min(p.Nk, i0 + BQ) : p.Nk;
     for (int j0 = 0; j0 < k_end; j0 += BK) {
         __syncthreads();
@@ -150,16 +146,14 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_mfma_kernel(
         for (int ob = 0; ob < 2; ++ob) {
             // ---- convolution: C^T block = sum_a T_a^T * S^T(rows shifted by a - pq) ----
             f32x4 c[BK / 16];
-            const int srow = QH + ob * 16 + n - pq;
+            const int srow = QH + ob * 16 + n - (CQT - 1);
 #pragma unroll
             for (int kb = 0; kb < BK / 16; ++kb) {
                 c[kb] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int a = 0; a < CQT; ++a) {
-                    if (a < cq) {
-                        f16x8 sf = *reinterpret_cast<const f16x8 *>(Ss + (srow + a) * SST + (kb * 16 + 8 * g) * 2);
-                        c[kb] = mfma_f16(tf[a], sf, c[kb]);
-                    }
+                    f16x8 sf = *reinterpret_cast<const f16x8 *>(Ss + (srow + a) * SST + (kb * 16 + 8 * g) * 2);
+                    c[kb] = mfma_f16(tf[a], sf, c[kb]);
                 }
             }
             // ---- post-mask and online softmax (log2 domain) ----
@@ -170,7 +164,7 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_mfma_kernel(
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int key = j0 + kb * 16 + 4 * g + r;
-                    float x = c[kb][r] * kLog2e;
+                    float x = c[kb][r];
                     if (key >= p.Nk || (causal && key > qpos)) x = kNegInf;
                     c[kb][r] = x;
                     mx = fmaxf(mx, x);

@@ -56,6 +56,21 @@ __device__ __forceinline__ f16x8 toeplitz_frag(const float *__restrict__ w_row, 
     return t;
 }
 
+// Bands for a compile-time tap count CQT >= c_q: the window is padded with zero
+// taps in FRONT (older query rows), so tap slot t stands for tap a = t - (CQT - c_q)
+// and reads score row  i + t - (CQT - 1); the padded slots read rows that exist
+// (the halo above the tile) and multiply them by zero.  No run-time tap loop.
+template <int CQT>
+__device__ __forceinline__ void load_bands(f16x8 (&tf)[CQT], const float *__restrict__ w_head, int c_q,
+                                           int c_k, int pk, int g, int n, bool flip) {
+#pragma unroll
+    for (int t = 0; t < CQT; ++t) {
+        const int a = t - (CQT - c_q);
+        if (a >= 0) tf[t] = toeplitz_frag(w_head + (size_t)a * c_k, c_k, pk, g, n, flip);
+        else tf[t] = (f16x8)(_Float16)0.f;
+    }
+}
+
 // 8 bf16 (16 bytes) of row `row` at element offset `col` of a dense [N][D]
 // matrix, zeros when the row is outside [0, N).
 template <int D>
@@ -88,5 +103,10 @@ hipError_t mfma_bwd_dq_dw(const Problem &p, int out_dt, const void *q, const voi
 hipError_t mfma_bwd_dkdv(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
                          const void *d_o, const float *Dl, const float *lse, const float *w, void *dk,
                          void *dv, hipStream_t s);
+
+// ---- decode as an HBM stream (decode_stream.hip) ----
+bool decode_stream_ok(const Problem &p, int in_dt, unsigned flags);
+hipError_t decode_stream(const Problem &p, const void *q, const void *k, const void *v, const float *w,
+                         float *o_part, float *m_part, float *l_part, hipStream_t s);
 
 }  // namespace convattn

@@ -161,3 +161,48 @@ def test_module_autograd_matches_oracle_autograd():
     O_id = ident(q.detach(), k.detach(), v.detach())
     sdpa = torch.nn.functional.scaled_dot_product_attention(Q.float(), K.float(), V.float(), is_causal=True)
     assert max_abs(O_id, sdpa) <= TOL_BF16
+
+
+@pytest.mark.parametrize("r,Nk,d,c_q,c_k,splits", [
+    (6, 500, 128, 6, 11, 3),
+    (6, 8192, 128, 6, 11, 1),
+    (16, 240, 64, 5, 5, 4),
+    (1, 77, 64, 6, 11, 1),
+    (3, 1000, 128, 3, 5, 7),
+    (6, 64, 64, 6, 11, 64),
+    (6, 130, 128, 16, 17, 2),
+])
+@pytest.mark.parametrize("causal", [False, True])
+def test_decode_bf16_stream(r, Nk, d, c_q, c_k, splits, causal):
+    from flash_multi_token_attention_amd.conv_attn import fwd_conv_attn_inference
+    from oracle import conv_attn_oracle as orc
+    Q, K, V, _, W = rand_case(2, 3, r, Nk, d, c_q, c_k, torch.bfloat16, seed=Nk + r)
+    O_ref, M_ref, L_ref = orc.decode(Q.float(), K.float(), V.float(), W, scale_of(d), causal=causal)
+    g = [t.to(DEV) for t in (Q, K, V, W)]
+    assert ops.kernel_path(g[0], g[1], g[3], causal, op="decode") == "mfma"
+    O, M, L = fwd_conv_attn_inference(g[0], g[1], g[2], g[3], splits, scale_of(d), c_q - 1,
+                                      (c_k - 1) // 2, causal)
+    assert O.shape == (2, 3, 1, d)
+    assert max_abs(O, O_ref) <= TOL_BF16
+    assert max_abs(M, M_ref) <= 1e-3
+    assert rel_max(L, L_ref) <= 1e-3
+
+
+def test_decode_full_size_properties():
+    # c4-sized cache per (batch, head) (fewer pairs): split invariance, agreement with
+    # the fp32-arithmetic kernel, and sum of probabilities == 1 (V = 1 -> O = 1).
+    from flash_multi_token_attention_amd.conv_attn.ops import decode
+    wl = synthetic.WORKLOADS["c4_decode"]
+    g = torch.Generator(device=DEV).manual_seed(1)
+    mk = lambda *s: torch.randn(*s, generator=g, device=DEV).to(torch.bfloat16)
+    Q, K, V = mk(4, 8, wl.Nq, wl.d), mk(4, 8, wl.Nk, wl.d), mk(4, 8, wl.Nk, wl.d)
+    W = synthetic.conv_weight(synthetic.Workload("x", 4, 8, 6, 8192, 128, 6, 11),
+                              torch.randn(8, 6, 11, generator=torch.Generator().manual_seed(2))).to(DEV)
+    base = decode(Q, K, V, W, 1, wl.scale)
+    exact = decode(Q, K, V, W, 4, wl.scale, exact=True)
+    assert max_abs(base[0], exact[0]) <= 2e-3 and max_abs(base[1], exact[1]) <= 1e-3
+    for s in (2, 5, 32):
+        o = decode(Q, K, V, W, s, wl.scale)
+        assert max_abs(o[0], base[0]) <= 1e-4 and rel_max(o[2], base[2]) <= 1e-4
+    ones = decode(Q, K, torch.ones_like(V), W, 3, wl.scale)
+    assert float((ones[0] - 1).abs().max()) <= 1e-4
