@@ -90,8 +90,8 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
     const float *dl_b = Dl + bh * p.Nq;
 
     f16x8 tf[CQT], tfl[CQT];
-    load_bands<CQT>(tf, W + (size_t)h * cq * ck, cq, ck, pk, g, n, false);
-    load_bands<CQT>(tfl, W + (size_t)h * cq * ck, cq, ck, pk, g, n, true);
+    load_bands<CQT>(tf, W + (size_t)h * cq * ck, cq, ck, pk, g, n, false, 1.f);
+    load_bands<CQT>(tfl, W + (size_t)h * cq * ck, cq, ck, pk, g, n, true, 1.f);
 
     bf16x8 kf[4][KS];  // K rows c0-16 .. c0+47
     bf16x8 vf[3][KS];  // V rows c0-8 .. c0+39

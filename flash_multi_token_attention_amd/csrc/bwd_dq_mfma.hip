@@ -77,8 +77,8 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_mfma_kernel(
     const bf16_t *dOb = dO + bh * p.Nq * D;
 
     f16x8 tf[CQT], tfl[CQT];  // forward band and flipped (transposed-window) band per tap slot
-    load_bands<CQT>(tf, W + (size_t)h * cq * ck, cq, ck, pk, g, n, false);
-    load_bands<CQT>(tfl, W + (size_t)h * cq * ck, cq, ck, pk, g, n, true);
+    load_bands<CQT>(tf, W + (size_t)h * cq * ck, cq, ck, pk, g, n, false, 1.f);
+    load_bands<CQT>(tfl, W + (size_t)h * cq * ck, cq, ck, pk, g, n, true, 1.f);
 
     bf16x8 qf[4][KS];   // Q rows r0-16 .. r0+47
     bf16x8 gf[3][KS];   // dO rows r0 .. r0+47

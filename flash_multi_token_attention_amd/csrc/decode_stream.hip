@@ -29,15 +29,6 @@ constexpr int IT = 64;             // keys per wave iteration
 constexpr int SW = IT + 16;        // score strip width: 16 carried + 64 new
 constexpr int SROW = SW + 4;       // floats per strip row (84)
 
-// 8 bf16 of row `row`, zeros outside [0, N); no branch, so loads can be batched.
-template <int D>
-__device__ __forceinline__ u32x4 load_row16_nb(const bf16_t *__restrict__ base, int row, int N, int col) {
-    const int rr = min(max(row, 0), N - 1);
-    u32x4 v = *reinterpret_cast<const u32x4 *>(base + (size_t)rr * D + col);
-    if (rr != row) v = (u32x4){0u, 0u, 0u, 0u};
-    return v;
-}
-
 __device__ __forceinline__ float bf16_lo(unsigned int w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float bf16_hi(unsigned int w) { return __uint_as_float(w & 0xffff0000u); }
 

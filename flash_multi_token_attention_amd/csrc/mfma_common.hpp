@@ -62,13 +62,45 @@ __device__ __forceinline__ f16x8 toeplitz_frag(const float *__restrict__ w_row, 
 // (the halo above the tile) and multiply them by zero.  No run-time tap loop.
 template <int CQT>
 __device__ __forceinline__ void load_bands(f16x8 (&tf)[CQT], const float *__restrict__ w_head, int c_q,
-                                           int c_k, int pk, int g, int n, bool flip) {
+                                           int c_k, int pk, int g, int n, bool flip, float mul) {
 #pragma unroll
     for (int t = 0; t < CQT; ++t) {
         const int a = t - (CQT - c_q);
-        if (a >= 0) tf[t] = toeplitz_frag(w_head + (size_t)a * c_k, c_k, pk, g, n, flip);
-        else tf[t] = (f16x8)(_Float16)0.f;
+        f16x8 f = (f16x8)(_Float16)0.f;
+        if (a >= 0) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                int b = 8 * g + e - kKeyHalo - n + pk;
+                float v = 0.f;
+                if (b >= 0 && b < c_k) v = w_head[a * c_k + (flip ? (c_k - 1 - b) : b)] * mul;
+                f[e] = (_Float16)v;
+            }
+        }
+        tf[t] = f;
     }
+}
+
+// 8 bf16 of row `row`, zeros outside [0, N); branch-free so a batch of loads can be in flight.
+template <int D>
+__device__ __forceinline__ u32x4 load_row16_nb(const bf16_t *__restrict__ base, int row, int N, int col) {
+    const int rr = min(max(row, 0), N - 1);
+    u32x4 v = *reinterpret_cast<const u32x4 *>(base + (size_t)rr * D + col);
+    if (rr != row) v = (u32x4){0u, 0u, 0u, 0u};
+    return v;
+}
+
+// LDS transpose read (ds_read_b64_tr_b16): the 16 lanes of a group pass the
+// addresses of a 4-row x 16-column block of 16-bit elements (lane p: row p/4,
+// columns 4(p%4) .. +3) and lane p gets column p of the 4 rows.  With
+// `row0`/`col0` the block origin inside a row-major tile of row stride `stride`
+// bytes this yields, for MFMA operands whose k index runs over the tile's rows,
+// k = row0 .. row0+3 for column col0 + (lane % 16).
+__device__ __forceinline__ bf16x4 lds_read_tr4x16(const unsigned char *tile, int stride, int row0, int col0,
+                                                  int n) {
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    const unsigned char *ptr = tile + (row0 + (n >> 2)) * stride + (col0 + 4 * (n & 3)) * 2;
+    s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(ptr));
+    return __builtin_bit_cast(bf16x4, v);
 }
 
 // 8 bf16 (16 bytes) of row `row` at element offset `col` of a dense [N][D]
