@@ -313,18 +313,32 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_mfma_kernel(
             // A: S[i + a - pq][c0 + 32jb + 8g ..]   (S-tile row 16 + i + a - pq, column 16 + ...)
             // B: dC[i][c0 + 32jb + 8g - b + pk ..]  (dC-tile column 8 + ... - b + pk)
             const unsigned char *abase = Ss + (16 + n - pq) * SST + (16 + 8 * g) * 2;
-            const unsigned char *bbase = Cs + (8 + 8 * g - bcl + pk) * 2;
+            // LDS reads at odd 2-byte offsets are slow: read 5 dwords from the even
+            // element below and funnel-shift by 0 or 16 bits per lane instead.
+            const int boff = 8 + 8 * g - bcl + pk;
+            const unsigned char *bbase = Cs + (boff & ~1) * 2;
+            const unsigned int bsh = (boff & 1) * 16;
 #pragma unroll 1
             for (int i = 0; i < WR; i += 2) {
-                f16x8 af[4], bf[4];
+                f16x8 af[4];
+                u32x4 bw[4];
+                unsigned int bx[4];
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     const int ii = i + (u >> 1), jb = u & 1;
                     af[u] = *reinterpret_cast<const f16x8 *>(abase + ii * SST + jb * 64);
-                    bf[u] = reinterpret_cast<const F16x8U *>(bbase + ii * CST + jb * 64)->v;
+                    bw[u] = reinterpret_cast<const U32x4A4 *>(bbase + ii * CST + jb * 64)->v;
+                    bx[u] = *reinterpret_cast<const unsigned int *>(bbase + ii * CST + jb * 64 + 16);
                 }
 #pragma unroll
-                for (int u = 0; u < 4; ++u) acc_w[u] = mfma_f16(af[u], bf[u], acc_w[u]);
+                for (int u = 0; u < 4; ++u) {
+                    u32x4 sh;
+                    sh[0] = __builtin_amdgcn_alignbit(bw[u][1], bw[u][0], bsh);
+                    sh[1] = __builtin_amdgcn_alignbit(bw[u][2], bw[u][1], bsh);
+                    sh[2] = __builtin_amdgcn_alignbit(bw[u][3], bw[u][2], bsh);
+                    sh[3] = __builtin_amdgcn_alignbit(bx[u], bw[u][3], bsh);
+                    acc_w[u] = mfma_f16(af[u], __builtin_bit_cast(f16x8, sh), acc_w[u]);
+                }
             }
         }
     }

@@ -23,8 +23,9 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-// 8 fp16 at any 2-byte boundary (gfx950 LDS reads need no natural alignment)
-struct __attribute__((packed, aligned(2))) F16x8U { f16x8 v; };
+// 16 bytes at a 4-byte boundary (gfx950 LDS reads need no natural alignment, and
+// dword-aligned ones run at full speed)
+struct __attribute__((packed, aligned(4))) U32x4A4 { u32x4 v; };
 
 constexpr int kKeyHalo = 8;          // LDS columns before a block's first output key
 constexpr int kMfmaMaxPk = 8;        // so c_k <= 17 on the MFMA path
