@@ -5,17 +5,17 @@
 // before the window-aligned ones, keys c0-8 .. c0+23 for dV (the shifted ranges
 // of neighbouring waves and workgroups tile the key axis just the same).  The
 // wave keeps its K and V fragments and both accumulators in registers and walks
-// the queries in 32-row tiles that the workgroup stages in LDS (Q and dO
-// row-major for the score / dP products, transposed for the dK / dV products).
-// Per tile, with r0 its first row:
-//   S^T  rows r0-16 .. r0+47, keys c0-16 .. c0+47    K Q^T, pre-masked, fp16 -> LDS
+// the queries in 32-row tiles that the workgroup stages row-major in LDS (Q
+// and dO; their transposes for the dK / dV products come from LDS transpose
+// reads).  Per tile, with r0 its first row:
+//   S^T  rows r0-16 .. r0+47, keys c0-16 .. c0+47    raw K Q^T, pre-masked, fp16 -> LDS
 //   C    rows r0 .. r0+47, keys c0-8 .. c0+39        Toeplitz MFMAs, here oriented
 //        [query][key] so that a lane holds one key and 4 query rows: that is the
 //        operand layout the dV and dK products need, no transposition in between
-//   P = exp(C - LSE), dP = dO V^T, dC = P (dP - D): fp16 -> LDS (2-byte stores)
+//   P = exp2(C - LSE), dP = dO V^T, dC = P (dP - D): fp16 -> LDS (2-byte stores)
 //   dV^T += dO^T P        (rows r0 .. r0+31, keys c0-8 .. c0+23)
 //   dS   rows r0 .. r0+31, keys c0 .. c0+31: flipped-band MFMAs over dC, causal zero
-//   dK^T += Q^T dS
+//   dK^T += Q^T dS        (the flipped bands carry the softmax scale)
 #include "mfma_common.hpp"
 
 namespace convattn {
@@ -31,28 +31,17 @@ constexpr int C_ROWS = BR + 16;        // 48
 constexpr int C_COLS = WK + 16;        // 48
 constexpr int SST = (S_COLS + 8) * 2;  // 144
 constexpr int CST = (C_COLS + 8) * 2;  // 112
-constexpr int TST = BR * 2 + 16;       // 80 bytes per row of Q^T / dO^T
+constexpr int NSB = S_COLS / 16;       // 4 key blocks of S
+constexpr int NCB = C_COLS / 16;       // 3 key blocks of C / dP / dC
 
 template <int D> struct KvLds {
     static constexpr int RST = D * 2 + 16;
     static constexpr int q_bytes = S_ROWS * RST;
     static constexpr int g_bytes = C_ROWS * RST;
-    static constexpr int qt_bytes = D * TST;
-    static constexpr int gt_bytes = D * TST;
     static constexpr int stat_bytes = 2 * C_ROWS * 4;
     static constexpr int wave_bytes = S_ROWS * SST + C_ROWS * CST;
-    static constexpr int total = q_bytes + g_bytes + qt_bytes + gt_bytes + stat_bytes + NW * wave_bytes;
+    static constexpr int total = q_bytes + g_bytes + stat_bytes + NW * wave_bytes;
 };
-
-__device__ __forceinline__ void store_transposed(unsigned char *dst_base, int tst, int col8, int row,
-                                                 u32x4 v4) {
-    unsigned short *dst = reinterpret_cast<unsigned short *>(dst_base + (col8 * 8) * tst + row * 2);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        dst[(2 * e) * (tst / 2)] = (unsigned short)(v4[e] & 0xffffu);
-        dst[(2 * e + 1) * (tst / 2)] = (unsigned short)(v4[e] >> 16);
-    }
-}
 
 template <int D, int CQT, typename TO>
 __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
@@ -63,18 +52,19 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
     using Lds = KvLds<D>;
     constexpr int RST = Lds::RST;
     constexpr int KS = D / 32, DB = D / 16, CPR = D / 8;
+    constexpr int Q_CH = S_ROWS * CPR, G_CH = C_ROWS * CPR;
+    constexpr int Q_LD = (Q_CH + NW * 64 - 1) / (NW * 64);
+    constexpr int G_LD = (G_CH + NW * 64 - 1) / (NW * 64);
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     unsigned char *Qs = smem;
     unsigned char *Gs = Qs + Lds::q_bytes;
-    unsigned char *Qt = Gs + Lds::g_bytes;
-    unsigned char *Gt = Qt + Lds::qt_bytes;
-    float *lse_s = reinterpret_cast<float *>(Gt + Lds::gt_bytes);
+    float *lse_s = reinterpret_cast<float *>(Gs + Lds::g_bytes);
     float *dl_s = lse_s + C_ROWS;
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     const int g = lane >> 4, n = lane & 15;
-    unsigned char *Ss = Gt + Lds::gt_bytes + Lds::stat_bytes + wave * Lds::wave_bytes;
+    unsigned char *Ss = Gs + Lds::g_bytes + Lds::stat_bytes + wave * Lds::wave_bytes;
     unsigned char *Cs = Ss + S_ROWS * SST;
 
     const int h = blockIdx.y, b = blockIdx.z;
@@ -90,21 +80,21 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
     const float *dl_b = Dl + bh * p.Nq;
 
     f16x8 tf[CQT], tfl[CQT];
-    load_bands<CQT>(tf, W + (size_t)h * cq * ck, cq, ck, pk, g, n, false, 1.f);
-    load_bands<CQT>(tfl, W + (size_t)h * cq * ck, cq, ck, pk, g, n, true, 1.f);
+    load_bands<CQT>(tf, W + (size_t)h * cq * ck, cq, ck, pk, g, n, false, p.scale * kLog2e);
+    load_bands<CQT>(tfl, W + (size_t)h * cq * ck, cq, ck, pk, g, n, true, p.scale);
 
-    bf16x8 kf[4][KS];  // K rows c0-16 .. c0+47
-    bf16x8 vf[3][KS];  // V rows c0-8 .. c0+39
+    bf16x8 kf[NSB][KS];  // K rows c0-16 .. c0+47
+    bf16x8 vf[NCB][KS];  // V rows c0-8 .. c0+39
 #pragma unroll
-    for (int kb = 0; kb < 4; ++kb)
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
-            kf[kb][ks] = __builtin_bit_cast(bf16x8, load_row16<D>(Kb, c0 - 16 + kb * 16 + n, p.Nk, ks * 32 + g * 8));
-#pragma unroll
-    for (int kb = 0; kb < 3; ++kb)
+    for (int kb = 0; kb < NSB; ++kb)
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks)
-            vf[kb][ks] = __builtin_bit_cast(bf16x8, load_row16<D>(Vb, c0 - 8 + kb * 16 + n, p.Nk, ks * 32 + g * 8));
+            kf[kb][ks] = __builtin_bit_cast(bf16x8, load_row16_nb<D>(Kb, c0 - 16 + kb * 16 + n, p.Nk, ks * 32 + g * 8));
+#pragma unroll
+    for (int kb = 0; kb < NCB; ++kb)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+            vf[kb][ks] = __builtin_bit_cast(bf16x8, load_row16_nb<D>(Vb, c0 - 8 + kb * 16 + n, p.Nk, ks * 32 + g * 8));
 
     f32x4 acc_k[2][DB], acc_v[2][DB];
 #pragma unroll
@@ -115,57 +105,75 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
             acc_v[m][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
         }
 
-    const float scale = p.scale;
-    const float scale2 = p.scale * kLog2e;  // score tile in log2 units (the window is linear)
     // Causal: rows before the first key this workgroup touches (k0 - 8) see none of its keys.
     const int r_begin = causal ? (max(0, k0 - 8) / BR) * BR : 0;
     for (int r0 = r_begin; r0 < p.Nq; r0 += BR) {
         __syncthreads();
-        for (int c = tid; c < S_ROWS * CPR; c += NW * 64) {
-            int row = c / CPR, cc = c - row * CPR;
-            u32x4 v4 = load_row16<D>(Qb, r0 - 16 + row, p.Nq, cc * 8);
-            *reinterpret_cast<u32x4 *>(Qs + row * RST + cc * 16) = v4;
-            if (row >= 16 && row < 16 + BR) store_transposed(Qt, TST, cc, row - 16, v4);
-        }
-        for (int c = tid; c < C_ROWS * CPR; c += NW * 64) {
-            int row = c / CPR, cc = c - row * CPR;
-            u32x4 v4 = load_row16<D>(dOb, r0 + row, p.Nq, cc * 8);
-            *reinterpret_cast<u32x4 *>(Gs + row * RST + cc * 16) = v4;
-            if (row < BR) store_transposed(Gt, TST, cc, row, v4);
-        }
-        if (tid < C_ROWS) {
-            int qr = r0 + tid;
-            lse_s[tid] = qr < p.Nq ? lse_b[qr] * kLog2e : 0.f;
-            dl_s[tid] = qr < p.Nq ? dl_b[qr] : 0.f;
+        {   // stage Q rows r0-16 .. r0+47 and dO rows r0 .. r0+47: loads first, one wait, then writes
+            u32x4 qr[Q_LD], gr[G_LD];
+#pragma unroll
+            for (int i = 0; i < Q_LD; ++i) {
+                const int c = min(tid + i * NW * 64, Q_CH - 1), row = c / CPR, cc = c % CPR;
+                qr[i] = load_row16_nb<D>(Qb, r0 - 16 + row, p.Nq, cc * 8);
+            }
+#pragma unroll
+            for (int i = 0; i < G_LD; ++i) {
+                const int c = min(tid + i * NW * 64, G_CH - 1), row = c / CPR, cc = c % CPR;
+                gr[i] = load_row16_nb<D>(dOb, r0 + row, p.Nq, cc * 8);
+            }
+            float ls = 0.f, dd = 0.f;
+            if (tid < C_ROWS && r0 + tid < p.Nq) { ls = lse_b[r0 + tid] * kLog2e; dd = dl_b[r0 + tid]; }
+#pragma unroll
+            for (int i = 0; i < Q_LD; ++i) {
+                const int c = tid + i * NW * 64, row = c / CPR, cc = c % CPR;
+                if (c < Q_CH) *reinterpret_cast<u32x4 *>(Qs + row * RST + cc * 16) = qr[i];
+            }
+#pragma unroll
+            for (int i = 0; i < G_LD; ++i) {
+                const int c = tid + i * NW * 64, row = c / CPR, cc = c % CPR;
+                if (c < G_CH) *reinterpret_cast<u32x4 *>(Gs + row * RST + cc * 16) = gr[i];
+            }
+            if (tid < C_ROWS) { lse_s[tid] = ls; dl_s[tid] = dd; }
         }
         __syncthreads();
         if (causal && r0 + BR - 1 < c0 - 8) continue;  // none of the tile's own rows sees the wave's keys
+        const bool edge = c0 == 0 || (causal && c0 + 48 > r0 - 16) || (c0 + 40 > p.Nk) || (r0 + C_ROWS > p.Nq);
 
-        // ---- S^T tile -> fp16 LDS ----
+        // ---- S^T tile (raw) -> fp16 LDS; Q fragments one row block ahead ----
+        {
+            bf16x8 qf[2][KS];
+            auto load_qf = [&](int buf, int rb) {
 #pragma unroll
-        for (int rb = 0; rb < 4; ++rb) {
-            f32x4 acc[4];
+                for (int ks = 0; ks < KS; ++ks)
+                    qf[buf][ks] = *reinterpret_cast<const bf16x8 *>(Qs + (rb * 16 + n) * RST + (ks * 32 + g * 8) * 2);
+            };
+            load_qf(0, 0);
 #pragma unroll
-            for (int kb = 0; kb < 4; ++kb) acc[kb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            for (int rb = 0; rb < 4; ++rb) {
+                const int cur = rb & 1;
+                if (rb + 1 < 4) load_qf(cur ^ 1, rb + 1);
+                f32x4 acc[NSB];
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                bf16x8 qf = *reinterpret_cast<const bf16x8 *>(Qs + (rb * 16 + n) * RST + (ks * 32 + g * 8) * 2);
+                for (int kb = 0; kb < NSB; ++kb) acc[kb] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int kb = 0; kb < 4; ++kb) acc[kb] = mfma_bf16(kf[kb][ks], qf, acc[kb]);
-            }
-            const int qpos = r0 - 16 + rb * 16 + n;
+                for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
-            for (int kb = 0; kb < 4; ++kb) {
-                const int key0 = c0 - 16 + kb * 16 + 4 * g;
-                f16x4 hv;
+                    for (int kb = 0; kb < NSB; ++kb) acc[kb] = mfma_bf16(kf[kb][ks], qf[cur][ks], acc[kb]);
+                const int qpos = r0 - 16 + rb * 16 + n;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    float s = acc[kb][r] * scale2;
-                    if (causal && key0 + r > qpos) s = 0.f;
-                    s = fminf(fmaxf(s, -kF16Max), kF16Max);
-                    hv[r] = (_Float16)s;
+                for (int kb = 0; kb < NSB; ++kb) {
+                    if (edge && causal) {
+                        const int key0 = c0 - 16 + kb * 16 + 4 * g;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            if (key0 + r > qpos) acc[kb][r] = 0.f;
+                    }
+                    f16x4 hv;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        hv[r] = (_Float16)__builtin_amdgcn_fmed3f(acc[kb][r], -kF16Max, kF16Max);
+                    *reinterpret_cast<f16x4 *>(Ss + (rb * 16 + n) * SST + (kb * 16 + 4 * g) * 2) = hv;
                 }
-                *reinterpret_cast<f16x4 *>(Ss + (rb * 16 + n) * SST + (kb * 16 + 4 * g) * 2) = hv;
             }
         }
         __builtin_amdgcn_wave_barrier();
@@ -176,92 +184,145 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
         for (int rb = 0; rb < 3; ++rb) {
             const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(lse_s + rb * 16 + 4 * g);
             const f32x4 dl4 = *reinterpret_cast<const f32x4 *>(dl_s + rb * 16 + 4 * g);
-            const int srow = 16 + rb * 16 + n - (CQT - 1);
+            f32x4 c[NCB], dp[NCB];
 #pragma unroll
-            for (int kb = 0; kb < 3; ++kb) {
-                f32x4 c = {0.f, 0.f, 0.f, 0.f};
+            for (int kb = 0; kb < NCB; ++kb) {
+                c[kb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+                dp[kb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            }
+            {
+                const unsigned char *sbase = Ss + (16 + rb * 16 + n - (CQT - 1)) * SST + (8 * g) * 2;
+                f16x8 sf[2][NCB];
+                auto load_sf = [&](int buf, int a) {
+#pragma unroll
+                    for (int kb = 0; kb < NCB; ++kb)
+                        sf[buf][kb] = *reinterpret_cast<const f16x8 *>(sbase + a * SST + kb * 32);
+                };
+                load_sf(0, 0);
 #pragma unroll
                 for (int a = 0; a < CQT; ++a) {
-                    f16x8 sf = *reinterpret_cast<const f16x8 *>(Ss + (srow + a) * SST + (kb * 16 + 8 * g) * 2);
-                    c = mfma_f16(sf, tf[a], c);
+                    if (a + 1 < CQT) load_sf((a + 1) & 1, a + 1);
+#pragma unroll
+                    for (int kb = 0; kb < NCB; ++kb) c[kb] = mfma_f16(sf[a & 1][kb], tf[a], c[kb]);
                 }
-                f32x4 dp = {0.f, 0.f, 0.f, 0.f};
+            }
+            {
+                bf16x8 gf[2];
+                auto load_gf = [&](int buf, int ks) {
+                    gf[buf] = *reinterpret_cast<const bf16x8 *>(Gs + (rb * 16 + n) * RST + (ks * 32 + g * 8) * 2);
+                };
+                load_gf(0, 0);
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
-                    bf16x8 gf = *reinterpret_cast<const bf16x8 *>(Gs + (rb * 16 + n) * RST + (ks * 32 + g * 8) * 2);
-                    dp = mfma_bf16(gf, vf[kb][ks], dp);
+                    if (ks + 1 < KS) load_gf((ks + 1) & 1, ks + 1);
+#pragma unroll
+                    for (int kb = 0; kb < NCB; ++kb) dp[kb] = mfma_bf16(gf[ks & 1], vf[kb][ks], dp[kb]);
                 }
-                const int key = c0 - 8 + kb * 16 + n;
-                f32x4 pr;
+            }
+#pragma unroll
+            for (int kb = 0; kb < NCB; ++kb) {
+                f32x4 pr, dc;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const int qpos = r0 + rb * 16 + 4 * g + r;
-                    float e = fast_exp2(c[r] - lse4[r]);
-                    float dc = e * (dp[r] - dl4[r]);
-                    if (key < 0 || key >= p.Nk || qpos >= p.Nq || (causal && key > qpos)) { e = 0.f; dc = 0.f; }
-                    dc = fminf(fmaxf(dc, -kF16Max), kF16Max);
-                    pr[r] = e;
-                    *reinterpret_cast<_Float16 *>(Cs + (rb * 16 + 4 * g + r) * CST + (kb * 16 + n) * 2) = (_Float16)dc;
+                    pr[r] = fast_exp2(c[kb][r] - lse4[r]);
+                    dc[r] = pr[r] * (dp[kb][r] - dl4[r]);
                 }
+                if (edge) {
+                    const int key = c0 - 8 + kb * 16 + n;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int qpos = r0 + rb * 16 + 4 * g + r;
+                        if (key < 0 || key >= p.Nk || qpos >= p.Nq || (causal && key > qpos)) { pr[r] = 0.f; dc[r] = 0.f; }
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    *reinterpret_cast<_Float16 *>(Cs + (rb * 16 + 4 * g + r) * CST + (kb * 16 + n) * 2) =
+                        (_Float16)__builtin_amdgcn_fmed3f(dc[r], -kF16Max, kF16Max);
                 if (rb < 2 && kb < 2) pkeep[rb][kb] = pr;
             }
         }
         __builtin_amdgcn_wave_barrier();
 
-        // ---- dV^T += dO^T P  (keys c0-8 .. c0+23) ----
+        // ---- dV^T += dO^T P  (keys c0-8 .. c0+23); dO^T by transpose reads of the dO tile ----
+        {
+            bf16x8 pf[2];
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-            bf16x8 pf;
+            for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                pf[r] = (bf16_t)pkeep[0][kb][r];
-                pf[4 + r] = (bf16_t)pkeep[1][kb][r];
-            }
+                for (int r = 0; r < 4; ++r) {
+                    pf[kb][r] = (bf16_t)pkeep[0][kb][r];
+                    pf[kb][4 + r] = (bf16_t)pkeep[1][kb][r];
+                }
+            bf16x8 gt[2];
+            auto load_gt = [&](int buf, int db) {
+                bf16x4 lo = lds_read_tr4x16(Gs, RST, 4 * g, db * 16, n);
+                bf16x4 hi = lds_read_tr4x16(Gs, RST, 16 + 4 * g, db * 16, n);
+                gt[buf] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            };
+            load_gt(0, 0);
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
-                const unsigned char *grow = Gt + (db * 16 + n) * TST + (4 * g) * 2;
-                bf16x4 lo = *reinterpret_cast<const bf16x4 *>(grow);
-                bf16x4 hi = *reinterpret_cast<const bf16x4 *>(grow + 32);
-                bf16x8 gf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                acc_v[kb][db] = mfma_bf16(gf, pf, acc_v[kb][db]);
+                if (db + 1 < DB) load_gt((db + 1) & 1, db + 1);
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb) acc_v[kb][db] = mfma_bf16(gt[db & 1], pf[kb], acc_v[kb][db]);
             }
         }
 
-        // ---- dS (keys c0 .. c0+31) and dK^T += Q^T dS ----
+        // ---- dS (keys c0 .. c0+31): 4 chains over the taps ----
         f32x4 ds[2][2];
 #pragma unroll
         for (int ob = 0; ob < 2; ++ob)
 #pragma unroll
-            for (int m = 0; m < 2; ++m) {
-                f32x4 s = {0.f, 0.f, 0.f, 0.f};
+            for (int m = 0; m < 2; ++m) ds[ob][m] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        {
+            constexpr int NST = 2 * CQT;  // stage = (tap slot, row block)
+            f16x8 cf[2][2];
+            auto load_cf = [&](int buf, int st) {
+                const int a = st >> 1, ob = st & 1;
+                const unsigned char *base = Cs + (ob * 16 + n + (CQT - 1) - a) * CST + (8 * g) * 2;
+                cf[buf][0] = *reinterpret_cast<const f16x8 *>(base);
+                cf[buf][1] = *reinterpret_cast<const f16x8 *>(base + 32);
+            };
+            load_cf(0, 0);
 #pragma unroll
-                for (int a = 0; a < CQT; ++a) {
-                    f16x8 cf = *reinterpret_cast<const f16x8 *>(Cs + (ob * 16 + n + (CQT - 1) - a) * CST + (m * 16 + 8 * g) * 2);
-                    s = mfma_f16(cf, tfl[a], s);
-                }
-                if (causal) {
-                    const int key = c0 + m * 16 + n;
+            for (int st = 0; st < NST; ++st) {
+                if (st + 1 < NST) load_cf((st + 1) & 1, st + 1);
+#pragma unroll
+                for (int m = 0; m < 2; ++m) ds[st & 1][m] = mfma_f16(cf[st & 1][m], tfl[st >> 1], ds[st & 1][m]);
+            }
+        }
+        if (edge && causal) {
+#pragma unroll
+            for (int ob = 0; ob < 2; ++ob)
+#pragma unroll
+                for (int m = 0; m < 2; ++m)
 #pragma unroll
                     for (int r = 0; r < 4; ++r)
-                        if (key > r0 + ob * 16 + 4 * g + r) s[r] = 0.f;
+                        if (c0 + m * 16 + n > r0 + ob * 16 + 4 * g + r) ds[ob][m][r] = 0.f;
+        }
+        // ---- dK^T += Q^T dS; Q^T by transpose reads (own rows start at Q-tile row 16) ----
+        {
+            bf16x8 sf[2];
+#pragma unroll
+            for (int m = 0; m < 2; ++m)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    sf[m][r] = (bf16_t)ds[0][m][r];
+                    sf[m][4 + r] = (bf16_t)ds[1][m][r];
                 }
-                ds[ob][m] = s;
-            }
-#pragma unroll
-        for (int m = 0; m < 2; ++m) {
-            bf16x8 sf;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                sf[r] = (bf16_t)ds[0][m][r];
-                sf[4 + r] = (bf16_t)ds[1][m][r];
-            }
+            bf16x8 qt[2];
+            auto load_qt = [&](int buf, int db) {
+                bf16x4 lo = lds_read_tr4x16(Qs, RST, 16 + 4 * g, db * 16, n);
+                bf16x4 hi = lds_read_tr4x16(Qs, RST, 32 + 4 * g, db * 16, n);
+                qt[buf] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            };
+            load_qt(0, 0);
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
-                const unsigned char *qrow = Qt + (db * 16 + n) * TST + (4 * g) * 2;
-                bf16x4 lo = *reinterpret_cast<const bf16x4 *>(qrow);
-                bf16x4 hi = *reinterpret_cast<const bf16x4 *>(qrow + 32);
-                bf16x8 qf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                acc_k[m][db] = mfma_bf16(qf, sf, acc_k[m][db]);
+                if (db + 1 < DB) load_qt((db + 1) & 1, db + 1);
+#pragma unroll
+                for (int m = 0; m < 2; ++m) acc_k[m][db] = mfma_bf16(qt[db & 1], sf[m], acc_k[m][db]);
             }
         }
     }
@@ -279,10 +340,10 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                 if constexpr (sizeof(TO) == 2) {
                     bf16x4 ov;
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) ov[r] = (bf16_t)(acc_k[m][db][r] * scale);
+                    for (int r = 0; r < 4; ++r) ov[r] = (bf16_t)acc_k[m][db][r];
                     *reinterpret_cast<bf16x4 *>(dst) = ov;
                 } else {
-                    *reinterpret_cast<f32x4 *>(dst) = acc_k[m][db] * scale;
+                    *reinterpret_cast<f32x4 *>(dst) = acc_k[m][db];
                 }
             }
             if (key_v >= 0 && key_v < p.Nk) {
