@@ -31,6 +31,17 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 HBM_PEAK_GBPS = 8000.0
 
 
+def measured_traffic(kernel, workload):
+    """HBM bytes per launch of `kernel` on `workload` as measured with rocprofv3
+    FETCH_SIZE / WRITE_SIZE (calibrated on a plain copy), from profiles/traffic.json;
+    None when that kernel has not been measured."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            return json.load(f).get(f"{kernel}@{workload}", {}).get("hbm_bytes_per_launch")
+    except (OSError, ValueError):
+        return None
+
+
 def _p(t):
     return C.c_void_p(t.data_ptr())
 
@@ -174,6 +185,14 @@ def main():
     wl = synthetic.WORKLOADS[args.workload]
     fl = synthetic.useful_flops(wl)
 
+    if args.only == "copy":
+        # plain device copy of known size: calibrates the HBM traffic counters
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        ms = time_events(lambda: dst.copy_(src), args.steps, args.warmup)
+        print(json.dumps({"only": "copy", "bytes_read": 1 << 30, "bytes_written": 1 << 30, "ms": ms,
+                          "GBps": 2 * (1 << 30) / ms / 1e6}))
+        return
     ts = TrainStep(wl, dev, exact=args.exact)
     if args.only:
         if args.only == "decode":
@@ -214,7 +233,7 @@ def main():
                    "useful_flop_per_step": useful, "conv_flop_per_pass": fl["conv_per_pass"]},
         "kernel_ms": k_ms,
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None},
+                     "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": measured_traffic(dom, wl.name)},
     }
     if not args.no_decode:
         dwl = synthetic.WORKLOADS["c4_decode"]
@@ -228,7 +247,8 @@ def main():
                                      f"window={dwl.c_q}x{dwl.c_k} resident_rows={dwl.Nq} splits={ds.splits}",
                          "ms": dms, "bytes": nbytes,
                          "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                                      "frac": gbps / HBM_PEAK_GBPS, "traffic": None}}
+                                      "frac": gbps / HBM_PEAK_GBPS,
+                                      "traffic": measured_traffic("decode", dwl.name)}}
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(wl)
     print(json.dumps(out))
