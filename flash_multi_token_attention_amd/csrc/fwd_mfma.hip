@@ -66,8 +66,10 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_mfma_kernel(
     const int g = lane >> 4, n = lane & 15;
     unsigned char *Ss = smem + Lds::k_bytes + Lds::v_bytes + wave * (SR * SST);
 
-    const int h = blockIdx.y, b = blockIdx.z;
-    const int qt = gridDim.x - 1 - blockIdx.x;  // longest (causal) tiles first
+    // x = head, y = batch, z = query tile: the dispatcher hands out every (batch, head) of the
+    // longest (causal) tiles first, so the tail of the launch is made of short tiles
+    const int h = blockIdx.x, b = blockIdx.y;
+    const int qt = gridDim.z - 1 - blockIdx.z;
     const int i0 = qt * BQ, i0w = i0 + wave * WR;
     const int pk = p.pk, cq = p.c_q;
     const bool causal = p.causal != 0;
@@ -97,9 +99,28 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_mfma_kernel(
     float m_run[2] = {kNegInf, kNegInf};  // running max, in log2 units
     float l_run[2] = {0.f, 0.f};          // this lane's share of the row sum
 
+    // Staging registers: every thread holds its 16-byte chunks of the next K / V tile.
+    u32x4 kr[K_LD], vr[V_LD];
+    auto load_tile = [&](int j0) {
+#pragma unroll
+        for (int i = 0; i < K_LD; ++i) {
+            const int c = min(tid + i * NW * 64, K_CH - 1), row = c / CPR, cc = c % CPR;
+            kr[i] = load_row16_nb<D>(Kb, j0 - kKeyHalo + row, p.Nk, cc * 8);
+        }
+#pragma unroll
+        for (int i = 0; i < V_LD; ++i) {
+            const int c = min(tid + i * NW * 64, V_CH - 1), row = c / CPR, cc = c % CPR;
+            vr[i] = load_row16_nb<D>(Vb, j0 + row, p.Nk, cc * 8);
+        }
+    };
+
     // One tile of the wave; `edge` = the tile touches the diagonal or the end of the keys
     // (wave-uniform), only then are the masks evaluated.
-    auto tile = [&](int j0, bool edge) {
+    auto tile = [&](int j0, bool edge, bool skip, bool more) {
+        if (skip) {
+            if (more) load_tile(j0 + BK);
+            return;
+        }
         // ---- S^T = K Q^T (raw), pre-mask, fp16 -> LDS; K fragments one block ahead ----
         {
             bf16x8 kf[2][KS];
@@ -167,6 +188,8 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_mfma_kernel(
                 c[ob][2 * kh + 1] = mfma_f16(tf[a], sf[st & 1][1], c[ob][2 * kh + 1]);
             }
         }
+        // next tile's K / V: in flight during the softmax and the P.V products
+        if (more) load_tile(j0 + BK);
         // ---- post-mask and online softmax (log2 domain) ----
         float alpha[2];
 #pragma unroll
@@ -241,36 +264,24 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_mfma_kernel(
     };
 
     const int k_end = causal ? min(p.Nk, i0 + BQ) : p.Nk;
+    load_tile(0);
     for (int j0 = 0; j0 < k_end; j0 += BK) {
         __syncthreads();
-        // ---- stage K and V row-major: all loads in flight, then one wait, then the LDS writes ----
-        {
-            u32x4 kr[K_LD], vr[V_LD];
+        // ---- K and V of this tile were loaded during the previous one: write them to LDS ----
 #pragma unroll
-            for (int i = 0; i < K_LD; ++i) {
-                const int c = min(tid + i * NW * 64, K_CH - 1), row = c / CPR, cc = c % CPR;
-                kr[i] = load_row16_nb<D>(Kb, j0 - kKeyHalo + row, p.Nk, cc * 8);
-            }
+        for (int i = 0; i < K_LD; ++i) {
+            const int c = tid + i * NW * 64, row = c / CPR, cc = c % CPR;
+            if (c < K_CH) *reinterpret_cast<u32x4 *>(Ks + row * KST + cc * 16) = kr[i];
+        }
 #pragma unroll
-            for (int i = 0; i < V_LD; ++i) {
-                const int c = min(tid + i * NW * 64, V_CH - 1), row = c / CPR, cc = c % CPR;
-                vr[i] = load_row16_nb<D>(Vb, j0 + row, p.Nk, cc * 8);
-            }
-#pragma unroll
-            for (int i = 0; i < K_LD; ++i) {
-                const int c = tid + i * NW * 64, row = c / CPR, cc = c % CPR;
-                if (c < K_CH) *reinterpret_cast<u32x4 *>(Ks + row * KST + cc * 16) = kr[i];
-            }
-#pragma unroll
-            for (int i = 0; i < V_LD; ++i) {
-                const int c = tid + i * NW * 64, row = c / CPR, cc = c % CPR;
-                if (c < V_CH) *reinterpret_cast<u32x4 *>(Vs + row * KST + cc * 16) = vr[i];
-            }
+        for (int i = 0; i < V_LD; ++i) {
+            const int c = tid + i * NW * 64, row = c / CPR, cc = c % CPR;
+            if (c < V_CH) *reinterpret_cast<u32x4 *>(Vs + row * KST + cc * 16) = vr[i];
         }
         __syncthreads();
-        if (causal && j0 > i0w + WR - 1) continue;  // every key of the tile is after this wave's rows
+        const bool skip = causal && j0 > i0w + WR - 1;  // every key of the tile is after this wave's rows
         const bool edge = (causal && j0 + BK + kKeyHalo > i0w - QH) || (j0 + BK > p.Nk);
-        tile(j0, edge);
+        tile(j0, edge, skip, j0 + BK < k_end);
     }
 
     // ---- epilogue: finish the row sums, normalise, store O, M, L ----
@@ -314,7 +325,7 @@ hipError_t launch_fwd(const Problem &p, const void *q, const void *k, const void
                                            hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (e != hipSuccess) return e;
     }
-    dim3 grid((p.Nq + BQ - 1) / BQ, p.H, p.B);
+    dim3 grid(p.H, p.B, (p.Nq + BQ - 1) / BQ);
     kern<<<grid, NW * 64, lds, s>>>(p, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, w,
                                     (TO *)o, m, l);
     return hipGetLastError();
