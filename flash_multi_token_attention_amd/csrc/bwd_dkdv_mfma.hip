@@ -67,8 +67,9 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
     unsigned char *Ss = Gs + Lds::g_bytes + Lds::stat_bytes + wave * Lds::wave_bytes;
     unsigned char *Cs = Ss + S_ROWS * SST;
 
-    const int h = blockIdx.y, b = blockIdx.z;
-    const int k0 = blockIdx.x * BKW, c0 = k0 + wave * WK;
+    // x = head, y = batch, z = key tile: the first key tiles see the most rows and go first
+    const int h = blockIdx.x, b = blockIdx.y;
+    const int k0 = blockIdx.z * BKW, c0 = k0 + wave * WK;
     const int pk = p.pk, cq = p.c_q, ck = p.c_k;
     const bool causal = p.causal != 0;
     const size_t bh = (size_t)b * p.H + h;
@@ -107,35 +108,39 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
 
     // Causal: rows before the first key this workgroup touches (k0 - 8) see none of its keys.
     const int r_begin = causal ? (max(0, k0 - 8) / BR) * BR : 0;
+    // Staging registers: this thread's 16-byte chunks of the next Q / dO tile and its LSE / D entry.
+    u32x4 qr[Q_LD], gr[G_LD];
+    float ls = 0.f, dd = 0.f;
+    auto load_tile = [&](int r0) {
+#pragma unroll
+        for (int i = 0; i < Q_LD; ++i) {
+            const int c = min(tid + i * NW * 64, Q_CH - 1), row = c / CPR, cc = c % CPR;
+            qr[i] = load_row16_nb<D>(Qb, r0 - 16 + row, p.Nq, cc * 8);
+        }
+#pragma unroll
+        for (int i = 0; i < G_LD; ++i) {
+            const int c = min(tid + i * NW * 64, G_CH - 1), row = c / CPR, cc = c % CPR;
+            gr[i] = load_row16_nb<D>(dOb, r0 + row, p.Nq, cc * 8);
+        }
+        ls = 0.f; dd = 0.f;
+        if (tid < C_ROWS && r0 + tid < p.Nq) { ls = lse_b[r0 + tid] * kLog2e; dd = dl_b[r0 + tid]; }
+    };
+    load_tile(r_begin);
     for (int r0 = r_begin; r0 < p.Nq; r0 += BR) {
         __syncthreads();
-        {   // stage Q rows r0-16 .. r0+47 and dO rows r0 .. r0+47: loads first, one wait, then writes
-            u32x4 qr[Q_LD], gr[G_LD];
 #pragma unroll
-            for (int i = 0; i < Q_LD; ++i) {
-                const int c = min(tid + i * NW * 64, Q_CH - 1), row = c / CPR, cc = c % CPR;
-                qr[i] = load_row16_nb<D>(Qb, r0 - 16 + row, p.Nq, cc * 8);
-            }
-#pragma unroll
-            for (int i = 0; i < G_LD; ++i) {
-                const int c = min(tid + i * NW * 64, G_CH - 1), row = c / CPR, cc = c % CPR;
-                gr[i] = load_row16_nb<D>(dOb, r0 + row, p.Nq, cc * 8);
-            }
-            float ls = 0.f, dd = 0.f;
-            if (tid < C_ROWS && r0 + tid < p.Nq) { ls = lse_b[r0 + tid] * kLog2e; dd = dl_b[r0 + tid]; }
-#pragma unroll
-            for (int i = 0; i < Q_LD; ++i) {
-                const int c = tid + i * NW * 64, row = c / CPR, cc = c % CPR;
-                if (c < Q_CH) *reinterpret_cast<u32x4 *>(Qs + row * RST + cc * 16) = qr[i];
-            }
-#pragma unroll
-            for (int i = 0; i < G_LD; ++i) {
-                const int c = tid + i * NW * 64, row = c / CPR, cc = c % CPR;
-                if (c < G_CH) *reinterpret_cast<u32x4 *>(Gs + row * RST + cc * 16) = gr[i];
-            }
-            if (tid < C_ROWS) { lse_s[tid] = ls; dl_s[tid] = dd; }
+        for (int i = 0; i < Q_LD; ++i) {
+            const int c = tid + i * NW * 64, row = c / CPR, cc = c % CPR;
+            if (c < Q_CH) *reinterpret_cast<u32x4 *>(Qs + row * RST + cc * 16) = qr[i];
         }
+#pragma unroll
+        for (int i = 0; i < G_LD; ++i) {
+            const int c = tid + i * NW * 64, row = c / CPR, cc = c % CPR;
+            if (c < G_CH) *reinterpret_cast<u32x4 *>(Gs + row * RST + cc * 16) = gr[i];
+        }
+        if (tid < C_ROWS) { lse_s[tid] = ls; dl_s[tid] = dd; }
         __syncthreads();
+        if (r0 + BR < p.Nq) load_tile(r0 + BR);
         if (causal && r0 + BR - 1 < c0 - 8) continue;  // none of the tile's own rows sees the wave's keys
         const bool edge = c0 == 0 || (causal && c0 + 48 > r0 - 16) || (c0 + 40 > p.Nk) || (r0 + C_ROWS > p.Nq);
 
@@ -371,7 +376,7 @@ hipError_t launch_kv(const Problem &p, const void *q, const void *k, const void 
                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return e;
     // + 8: the last workgroup's dV range starts 8 keys early, so the key axis needs 8 more
-    dim3 grid((p.Nk + 8 + BKW - 1) / BKW, p.H, p.B);
+    dim3 grid(p.H, p.B, (p.Nk + 8 + BKW - 1) / BKW);
     kern<<<grid, NW * 64, lds, s>>>(p, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v,
                                     (const bf16_t *)d_o, Dl, lse, w, (TO *)dk, (TO *)dv);
     return hipGetLastError();

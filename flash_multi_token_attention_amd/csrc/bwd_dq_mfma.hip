@@ -68,8 +68,9 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_mfma_kernel(
     unsigned char *Ss = Vs + Lds::v_bytes + wave * Lds::wave_bytes;
     unsigned char *Cs = Ss + S_ROWS * SST;
 
-    const int h = blockIdx.y, b = blockIdx.z;
-    const int qt = gridDim.x - 1 - blockIdx.x;
+    // x = head, y = batch, z = query tile: longest (causal) tiles of every (batch, head) first
+    const int h = blockIdx.x, b = blockIdx.y;
+    const int n_qt = gridDim.z, qt = n_qt - 1 - blockIdx.z;
     const int i0 = qt * BQ, r0 = i0 + wave * WR;
     const int pq = p.pq, pk = p.pk, cq = p.c_q, ck = p.c_k;
     const bool causal = p.causal != 0;
@@ -113,33 +114,38 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_mfma_kernel(
     for (int i = 0; i < 4; ++i) acc_w[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
     const int bcl = n < ck ? n : ck - 1;  // lanes past the last key tap re-read a valid one
 
+    // Staging registers: every thread holds its 16-byte chunks of the next K / V tile
+    // (K rows c0-16 .. c0+79, V rows c0-8 .. c0+71), loaded while the current tile is computed.
+    u32x4 kr[K_LD], vr[V_LD];
+    auto load_tile = [&](int c0) {
+#pragma unroll
+        for (int i = 0; i < K_LD; ++i) {
+            const int c = min(tid + i * NW * 64, K_CH - 1), row = c / CPR, cc = c % CPR;
+            kr[i] = load_row16_nb<D>(Kb, c0 - 16 + row, p.Nk, cc * 8);
+        }
+#pragma unroll
+        for (int i = 0; i < V_LD; ++i) {
+            const int c = min(tid + i * NW * 64, V_CH - 1), row = c / CPR, cc = c % CPR;
+            vr[i] = load_row16_nb<D>(Vb, c0 - 8 + row, p.Nk, cc * 8);
+        }
+    };
+
     const int k_end = causal ? min(p.Nk, i0 + BQ) : p.Nk;
+    load_tile(0);
     for (int c0 = 0; c0 < k_end; c0 += BK) {
         __syncthreads();
-        {   // stage K rows c0-16 .. c0+79 and V rows c0-8 .. c0+71: loads first, one wait, then writes
-            u32x4 kr[K_LD], vr[V_LD];
 #pragma unroll
-            for (int i = 0; i < K_LD; ++i) {
-                const int c = min(tid + i * NW * 64, K_CH - 1), row = c / CPR, cc = c % CPR;
-                kr[i] = load_row16_nb<D>(Kb, c0 - 16 + row, p.Nk, cc * 8);
-            }
+        for (int i = 0; i < K_LD; ++i) {
+            const int c = tid + i * NW * 64, row = c / CPR, cc = c % CPR;
+            if (c < K_CH) *reinterpret_cast<u32x4 *>(Ks + row * RST + cc * 16) = kr[i];
+        }
 #pragma unroll
-            for (int i = 0; i < V_LD; ++i) {
-                const int c = min(tid + i * NW * 64, V_CH - 1), row = c / CPR, cc = c % CPR;
-                vr[i] = load_row16_nb<D>(Vb, c0 - 8 + row, p.Nk, cc * 8);
-            }
-#pragma unroll
-            for (int i = 0; i < K_LD; ++i) {
-                const int c = tid + i * NW * 64, row = c / CPR, cc = c % CPR;
-                if (c < K_CH) *reinterpret_cast<u32x4 *>(Ks + row * RST + cc * 16) = kr[i];
-            }
-#pragma unroll
-            for (int i = 0; i < V_LD; ++i) {
-                const int c = tid + i * NW * 64, row = c / CPR, cc = c % CPR;
-                if (c < V_CH) *reinterpret_cast<u32x4 *>(Vs + row * RST + cc * 16) = vr[i];
-            }
+        for (int i = 0; i < V_LD; ++i) {
+            const int c = tid + i * NW * 64, row = c / CPR, cc = c % CPR;
+            if (c < V_CH) *reinterpret_cast<u32x4 *>(Vs + row * RST + cc * 16) = vr[i];
         }
         __syncthreads();
+        if (c0 + BK < k_end) load_tile(c0 + BK);
         if (causal && c0 > r0 + WR - 1) continue;
         // masks matter only where the tile can reach the diagonal or the end of the keys
         const bool edge = c0 == 0 || (causal && c0 + BK + 16 > r0 - 16) || (c0 + BK + 8 > p.Nk) ||
@@ -377,7 +383,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_mfma_kernel(
         float s = 0.f;
 #pragma unroll
         for (int w = 0; w < NW; ++w) s += red[(w * 16 + a) * 16 + bb];
-        dW_part[(bh * gridDim.x + qt) * ntap + tid] = s * p.scale;
+        dW_part[(bh * n_qt + qt) * ntap + tid] = s * p.scale;
     }
 }
 
@@ -390,7 +396,7 @@ hipError_t launch_dq(const Problem &p, const void *q, const void *k, const void 
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return e;
-    dim3 grid(mfma_dq_tiles(p), p.H, p.B);
+    dim3 grid(p.H, p.B, mfma_dq_tiles(p));
     kern<<<grid, NW * 64, lds, s>>>(p, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v,
                                     (const bf16_t *)d_o, Dl, lse, w, (TO *)dq, dw_part);
     return hipGetLastError();
