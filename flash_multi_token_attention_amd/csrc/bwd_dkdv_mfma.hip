@@ -115,12 +115,12 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
 #pragma unroll
         for (int i = 0; i < Q_LD; ++i) {
             const int c = min(tid + i * NW * 64, Q_CH - 1), row = c / CPR, cc = c % CPR;
-            qr[i] = load_row16_nb<D>(Qb, r0 - 16 + row, p.Nq, cc * 8);
+            qr[i] = load_row16_clamped<D>(Qb, r0 - 16 + row, p.Nq, cc * 8);
         }
 #pragma unroll
         for (int i = 0; i < G_LD; ++i) {
             const int c = min(tid + i * NW * 64, G_CH - 1), row = c / CPR, cc = c % CPR;
-            gr[i] = load_row16_nb<D>(dOb, r0 + row, p.Nq, cc * 8);
+            gr[i] = load_row16_clamped<D>(dOb, r0 + row, p.Nq, cc * 8);
         }
         ls = 0.f; dd = 0.f;
         if (tid < C_ROWS && r0 + tid < p.Nq) { ls = lse_b[r0 + tid] * kLog2e; dd = dl_b[r0 + tid]; }
@@ -128,6 +128,15 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
     load_tile(r_begin);
     for (int r0 = r_begin; r0 < p.Nq; r0 += BR) {
         __syncthreads();
+        if (r0 == 0 || r0 + C_ROWS > p.Nq) {  // rows outside the sequence count as zeros
+#pragma unroll
+            for (int i = 0; i < Q_LD; ++i) {
+                const int row = r0 - 16 + (tid + i * NW * 64) / CPR;
+                qr[i] = zero_unless(row >= 0 && row < p.Nq, qr[i]);
+            }
+#pragma unroll
+            for (int i = 0; i < G_LD; ++i) gr[i] = zero_unless(r0 + (tid + i * NW * 64) / CPR < p.Nq, gr[i]);
+        }
 #pragma unroll
         for (int i = 0; i < Q_LD; ++i) {
             const int c = tid + i * NW * 64, row = c / CPR, cc = c % CPR;

@@ -121,12 +121,12 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_mfma_kernel(
 #pragma unroll
         for (int i = 0; i < K_LD; ++i) {
             const int c = min(tid + i * NW * 64, K_CH - 1), row = c / CPR, cc = c % CPR;
-            kr[i] = load_row16_nb<D>(Kb, c0 - 16 + row, p.Nk, cc * 8);
+            kr[i] = load_row16_clamped<D>(Kb, c0 - 16 + row, p.Nk, cc * 8);
         }
 #pragma unroll
         for (int i = 0; i < V_LD; ++i) {
             const int c = min(tid + i * NW * 64, V_CH - 1), row = c / CPR, cc = c % CPR;
-            vr[i] = load_row16_nb<D>(Vb, c0 - 8 + row, p.Nk, cc * 8);
+            vr[i] = load_row16_clamped<D>(Vb, c0 - 8 + row, p.Nk, cc * 8);
         }
     };
 
@@ -134,6 +134,18 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_mfma_kernel(
     load_tile(0);
     for (int c0 = 0; c0 < k_end; c0 += BK) {
         __syncthreads();
+        if (c0 == 0 || c0 + BK + 16 > p.Nk) {  // rows outside the sequence count as zeros
+#pragma unroll
+            for (int i = 0; i < K_LD; ++i) {
+                const int row = c0 - 16 + (tid + i * NW * 64) / CPR;
+                kr[i] = zero_unless(row >= 0 && row < p.Nk, kr[i]);
+            }
+#pragma unroll
+            for (int i = 0; i < V_LD; ++i) {
+                const int row = c0 - 8 + (tid + i * NW * 64) / CPR;
+                vr[i] = zero_unless(row >= 0 && row < p.Nk, vr[i]);
+            }
+        }
 #pragma unroll
         for (int i = 0; i < K_LD; ++i) {
             const int c = tid + i * NW * 64, row = c / CPR, cc = c % CPR;

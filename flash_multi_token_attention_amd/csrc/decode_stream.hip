@@ -113,13 +113,13 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(
         for (int blk = 0; blk < 4; ++blk)
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks)
-                kreg[blk][ks] = load_row16_nb<D>(Kb, lo + 8 + blk * 16 + n, p.Nk, ks * 32 + g * 8);
+                kreg[blk][ks] = load_row16_clamped<D>(Kb, lo + 8 + blk * 16 + n, p.Nk, ks * 32 + g * 8);
 
         for (int j0 = lo; j0 < hi; j0 += IT) {
             // V of this iteration: keys j0 .. j0+63
             u32x4 vreg[VT];
 #pragma unroll
-            for (int t = 0; t < VT; ++t) vreg[t] = load_row16_nb<D>(Vb, j0 + RPI * t + gph, p.Nk, cc * 8);
+            for (int t = 0; t < VT; ++t) vreg[t] = load_row16_clamped<D>(Vb, j0 + RPI * t + gph, p.Nk, cc * 8);
 
             // scores of keys j0+8 .. j0+71 -> strip columns 16 .. 79
 #pragma unroll
@@ -134,6 +134,11 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(
                         const int key = j0 + 8 + blk * 16 + 4 * g + r;
                         a4[r] = (key > row_pos) ? 0.f : a4[r] * scale;
                     }
+                    if (j0 + IT + 8 > p.Nk) {  // keys past the end of the cache score zero (K rows were clamped)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            if (j0 + 8 + blk * 16 + 4 * g + r >= p.Nk) a4[r] = 0.f;
+                    }
                     *reinterpret_cast<f32x4 *>(strip + n * SROW + 16 + blk * 16 + 4 * g) = a4;
                 }
             }
@@ -143,7 +148,7 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(
                 for (int blk = 0; blk < 4; ++blk)
 #pragma unroll
                     for (int ks = 0; ks < KS; ++ks)
-                        kreg[blk][ks] = load_row16_nb<D>(Kb, j0 + IT + 8 + blk * 16 + n, p.Nk, ks * 32 + g * 8);
+                        kreg[blk][ks] = load_row16_clamped<D>(Kb, j0 + IT + 8 + blk * 16 + n, p.Nk, ks * 32 + g * 8);
             }
             __builtin_amdgcn_wave_barrier();
 

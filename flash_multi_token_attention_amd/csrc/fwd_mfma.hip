@@ -105,12 +105,12 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_mfma_kernel(
 #pragma unroll
         for (int i = 0; i < K_LD; ++i) {
             const int c = min(tid + i * NW * 64, K_CH - 1), row = c / CPR, cc = c % CPR;
-            kr[i] = load_row16_nb<D>(Kb, j0 - kKeyHalo + row, p.Nk, cc * 8);
+            kr[i] = load_row16_clamped<D>(Kb, j0 - kKeyHalo + row, p.Nk, cc * 8);
         }
 #pragma unroll
         for (int i = 0; i < V_LD; ++i) {
             const int c = min(tid + i * NW * 64, V_CH - 1), row = c / CPR, cc = c % CPR;
-            vr[i] = load_row16_nb<D>(Vb, j0 + row, p.Nk, cc * 8);
+            vr[i] = load_row16_clamped<D>(Vb, j0 + row, p.Nk, cc * 8);
         }
     };
 
@@ -268,6 +268,15 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_mfma_kernel(
     for (int j0 = 0; j0 < k_end; j0 += BK) {
         __syncthreads();
         // ---- K and V of this tile were loaded during the previous one: write them to LDS ----
+        if (j0 == 0 || j0 + BK + kKeyHalo > p.Nk) {  // rows outside the sequence count as zeros
+#pragma unroll
+            for (int i = 0; i < K_LD; ++i) {
+                const int kr_row = j0 - kKeyHalo + (tid + i * NW * 64) / CPR;
+                kr[i] = zero_unless(kr_row >= 0 && kr_row < p.Nk, kr[i]);
+            }
+#pragma unroll
+            for (int i = 0; i < V_LD; ++i) vr[i] = zero_unless(j0 + (tid + i * NW * 64) / CPR < p.Nk, vr[i]);
+        }
 #pragma unroll
         for (int i = 0; i < K_LD; ++i) {
             const int c = tid + i * NW * 64, row = c / CPR, cc = c % CPR;

@@ -90,6 +90,18 @@ __device__ __forceinline__ u32x4 load_row16_nb(const bf16_t *__restrict__ base, 
     return v;
 }
 
+// 8 bf16 of the row nearest to `row` inside [0, N): nothing depends on the loaded value, so the
+// load stays in flight until its consumer; rows outside the sequence are zeroed by the consumer
+// (only tiles at the ends of the sequence have any).
+template <int D>
+__device__ __forceinline__ u32x4 load_row16_clamped(const bf16_t *__restrict__ base, int row, int N, int col) {
+    const int rr = min(max(row, 0), N - 1);
+    return *reinterpret_cast<const u32x4 *>(base + (size_t)rr * D + col);
+}
+__device__ __forceinline__ u32x4 zero_unless(bool keep, u32x4 v) {
+    return keep ? v : (u32x4){0u, 0u, 0u, 0u};
+}
+
 // LDS transpose read (ds_read_b64_tr_b16): the 16 lanes of a group pass the
 // addresses of a 4-row x 16-column block of 16-bit elements (lane p: row p/4,
 // columns 4(p%4) .. +3) and lane p gets column p of the 4 rows.  With
