@@ -162,10 +162,14 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                     qf[buf][ks] = *reinterpret_cast<const bf16x8 *>(Qs + (rb * 16 + n) * RST + (ks * 32 + g * 8) * 2);
             };
             load_qf(0, 0);
+            SCHED_DS_READ(KS);
 #pragma unroll
             for (int rb = 0; rb < 4; ++rb) {
                 const int cur = rb & 1;
-                if (rb + 1 < 4) load_qf(cur ^ 1, rb + 1);
+                if (rb + 1 < 4) {
+                    load_qf(cur ^ 1, rb + 1);
+                    SCHED_DS_READ(KS);
+                }
                 f32x4 acc[NSB];
 #pragma unroll
                 for (int kb = 0; kb < NSB; ++kb) acc[kb] = (f32x4){0.f, 0.f, 0.f, 0.f};
@@ -173,6 +177,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                 for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
                     for (int kb = 0; kb < NSB; ++kb) acc[kb] = mfma_bf16(kf[kb][ks], qf[cur][ks], acc[kb]);
+                SCHED_MFMA(NSB * KS);
                 const int qpos = r0 - 16 + rb * 16 + n;
 #pragma unroll
                 for (int kb = 0; kb < NSB; ++kb) {
@@ -213,11 +218,16 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                         sf[buf][kb] = *reinterpret_cast<const f16x8 *>(sbase + a * SST + kb * 32);
                 };
                 load_sf(0, 0);
+                SCHED_DS_READ(NCB);
 #pragma unroll
                 for (int a = 0; a < CQT; ++a) {
-                    if (a + 1 < CQT) load_sf((a + 1) & 1, a + 1);
+                    if (a + 1 < CQT) {
+                        load_sf((a + 1) & 1, a + 1);
+                        SCHED_DS_READ(NCB);
+                    }
 #pragma unroll
                     for (int kb = 0; kb < NCB; ++kb) c[kb] = mfma_f16(sf[a & 1][kb], tf[a], c[kb]);
+                    SCHED_MFMA(NCB);
                 }
             }
             {
@@ -226,11 +236,16 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                     gf[buf] = *reinterpret_cast<const bf16x8 *>(Gs + (rb * 16 + n) * RST + (ks * 32 + g * 8) * 2);
                 };
                 load_gf(0, 0);
+                SCHED_DS_READ(1);
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
-                    if (ks + 1 < KS) load_gf((ks + 1) & 1, ks + 1);
+                    if (ks + 1 < KS) {
+                        load_gf((ks + 1) & 1, ks + 1);
+                        SCHED_DS_READ(1);
+                    }
 #pragma unroll
                     for (int kb = 0; kb < NCB; ++kb) dp[kb] = mfma_bf16(gf[ks & 1], vf[kb][ks], dp[kb]);
+                    SCHED_MFMA(NCB);
                 }
             }
 #pragma unroll
@@ -275,11 +290,16 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                 gt[buf] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
             };
             load_gt(0, 0);
+            SCHED_DS_READ(2);
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
-                if (db + 1 < DB) load_gt((db + 1) & 1, db + 1);
+                if (db + 1 < DB) {
+                    load_gt((db + 1) & 1, db + 1);
+                    SCHED_DS_READ(2);
+                }
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb) acc_v[kb][db] = mfma_bf16(gt[db & 1], pf[kb], acc_v[kb][db]);
+                SCHED_MFMA(2);
             }
         }
 
@@ -299,11 +319,16 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                 cf[buf][1] = *reinterpret_cast<const f16x8 *>(base + 32);
             };
             load_cf(0, 0);
+            SCHED_DS_READ(2);
 #pragma unroll
             for (int st = 0; st < NST; ++st) {
-                if (st + 1 < NST) load_cf((st + 1) & 1, st + 1);
+                if (st + 1 < NST) {
+                    load_cf((st + 1) & 1, st + 1);
+                    SCHED_DS_READ(2);
+                }
 #pragma unroll
                 for (int m = 0; m < 2; ++m) ds[st & 1][m] = mfma_f16(cf[st & 1][m], tfl[st >> 1], ds[st & 1][m]);
+                SCHED_MFMA(2);
             }
         }
         if (edge && causal) {
@@ -332,11 +357,16 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                 qt[buf] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
             };
             load_qt(0, 0);
+            SCHED_DS_READ(2);
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
-                if (db + 1 < DB) load_qt((db + 1) & 1, db + 1);
+                if (db + 1 < DB) {
+                    load_qt((db + 1) & 1, db + 1);
+                    SCHED_DS_READ(2);
+                }
 #pragma unroll
                 for (int m = 0; m < 2; ++m) acc_k[m][db] = mfma_bf16(qt[db & 1], sf[m], acc_k[m][db]);
+                SCHED_MFMA(2);
             }
         }
     }

@@ -172,10 +172,14 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_mfma_kernel(
                     kf[buf][ks] = *reinterpret_cast<const bf16x8 *>(Ks + (kb * 16 + n) * RST + (ks * 32 + g * 8) * 2);
             };
             load_kf(0, 0);
+            SCHED_DS_READ(KS);
 #pragma unroll
             for (int kb = 0; kb < S_COLS / 16; ++kb) {
                 const int cur = kb & 1;
-                if (kb + 1 < S_COLS / 16) load_kf(cur ^ 1, kb + 1);
+                if (kb + 1 < S_COLS / 16) {
+                    load_kf(cur ^ 1, kb + 1);
+                    SCHED_DS_READ(KS);
+                }
                 f32x4 acc[4];
 #pragma unroll
                 for (int rb = 0; rb < 4; ++rb) acc[rb] = (f32x4){0.f, 0.f, 0.f, 0.f};
@@ -183,6 +187,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_mfma_kernel(
                 for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
                     for (int rb = 0; rb < 4; ++rb) acc[rb] = mfma_bf16(kf[cur][ks], qf[rb][ks], acc[rb]);
+                SCHED_MFMA(4 * KS);
                 const int key0 = c0 - 16 + kb * 16 + 4 * g;
 #pragma unroll
                 for (int rb = 0; rb < 4; ++rb) {
@@ -222,11 +227,16 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_mfma_kernel(
                         sf[buf][kb] = *reinterpret_cast<const f16x8 *>(sbase + a * SST + kb * 32);
                 };
                 load_sf(0, 0);
+                SCHED_DS_READ(NCB);
 #pragma unroll
                 for (int a = 0; a < CQT; ++a) {
-                    if (a + 1 < CQT) load_sf((a + 1) & 1, a + 1);
+                    if (a + 1 < CQT) {
+                        load_sf((a + 1) & 1, a + 1);
+                        SCHED_DS_READ(NCB);
+                    }
 #pragma unroll
                     for (int kb = 0; kb < NCB; ++kb) c[kb] = mfma_f16(tf[a], sf[a & 1][kb], c[kb]);
+                    SCHED_MFMA(NCB);
                 }
             }
             {
@@ -237,11 +247,16 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_mfma_kernel(
                         vf[buf][kb] = *reinterpret_cast<const bf16x8 *>(Vs + (kb * 16 + n) * RST + (ks * 32 + g * 8) * 2);
                 };
                 load_vf(0, 0);
+                SCHED_DS_READ(NCB);
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
-                    if (ks + 1 < KS) load_vf((ks + 1) & 1, ks + 1);
+                    if (ks + 1 < KS) {
+                        load_vf((ks + 1) & 1, ks + 1);
+                        SCHED_DS_READ(NCB);
+                    }
 #pragma unroll
                     for (int kb = 0; kb < NCB; ++kb) dp[kb] = mfma_bf16(vf[ks & 1][kb], gf[rb][ks], dp[kb]);
+                    SCHED_MFMA(NCB);
                 }
             }
 #pragma unroll
@@ -280,12 +295,17 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_mfma_kernel(
                 for (int kb = 0; kb < BK / 16; ++kb) cf[buf][kb] = *reinterpret_cast<const f16x8 *>(base + kb * 32);
             };
             load_cf(0, 0);
+            SCHED_DS_READ(BK / 16);
 #pragma unroll
             for (int st = 0; st < NST; ++st) {
-                if (st + 1 < NST) load_cf((st + 1) & 1, st + 1);
+                if (st + 1 < NST) {
+                    load_cf((st + 1) & 1, st + 1);
+                    SCHED_DS_READ(BK / 16);
+                }
 #pragma unroll
                 for (int kb = 0; kb < BK / 16; ++kb)
                     ds[st & 1][kb] = mfma_f16(tfl[st >> 1], cf[st & 1][kb], ds[st & 1][kb]);
+                SCHED_MFMA(BK / 16);
             }
         }
         if (edge && causal) {
@@ -317,12 +337,17 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_mfma_kernel(
                 kf[buf] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
             };
             load_kt(0, 0);
+            SCHED_DS_READ(2);
 #pragma unroll
             for (int st = 0; st < (BK / 32) * DB; ++st) {
-                if (st + 1 < (BK / 32) * DB) load_kt((st + 1) & 1, st + 1);
+                if (st + 1 < (BK / 32) * DB) {
+                    load_kt((st + 1) & 1, st + 1);
+                    SCHED_DS_READ(2);
+                }
                 const int kp = st / DB, db = st % DB;
 #pragma unroll
                 for (int ob = 0; ob < 2; ++ob) acc_q[ob][db] = mfma_bf16(kf[st & 1], sf[ob][kp], acc_q[ob][db]);
+                SCHED_MFMA(2);
             }
         }
 

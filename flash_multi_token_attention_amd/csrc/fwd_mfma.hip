@@ -148,16 +148,21 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_mfma_kernel(
                 }
             };
             load_kf(0, 0);
+            SCHED_DS_READ(KS);
 #pragma unroll
             for (int kb = 0; kb < NKB; ++kb) {
                 const int cur = kb & 1;
-                if (kb + 1 < NKB) load_kf(cur ^ 1, kb + 1);
+                if (kb + 1 < NKB) {
+                    load_kf(cur ^ 1, kb + 1);
+                    SCHED_DS_READ(KS);
+                }
 #pragma unroll
                 for (int rb = 0; rb < 3; ++rb) acc[rb] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
                     for (int rb = 0; rb < 3; ++rb) acc[rb] = mfma_bf16(kf[cur][ks], qf[rb][ks], acc[rb]);
+                SCHED_MFMA(3 * KS);
                 store_s(kb);
             }
         }
@@ -180,12 +185,17 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_mfma_kernel(
                 sf[buf][1] = *reinterpret_cast<const f16x8 *>(base + 32);
             };
             load_sf(0, 0);
+            SCHED_DS_READ(2);
 #pragma unroll
             for (int st = 0; st < NST; ++st) {
-                if (st + 1 < NST) load_sf((st + 1) & 1, st + 1);
+                if (st + 1 < NST) {
+                    load_sf((st + 1) & 1, st + 1);
+                    SCHED_DS_READ(2);
+                }
                 const int a = st >> 2, ob = (st >> 1) & 1, kh = st & 1;
                 c[ob][2 * kh] = mfma_f16(tf[a], sf[st & 1][0], c[ob][2 * kh]);
                 c[ob][2 * kh + 1] = mfma_f16(tf[a], sf[st & 1][1], c[ob][2 * kh + 1]);
+                SCHED_MFMA(2);
             }
         }
         // next tile's K / V: in flight during the softmax and the P.V products
@@ -253,12 +263,17 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_mfma_kernel(
                 vf[buf] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
             };
             load_vf(0, 0);
+            SCHED_DS_READ(2);
 #pragma unroll
             for (int st = 0; st < (BK / 32) * DB; ++st) {
-                if (st + 1 < (BK / 32) * DB) load_vf((st + 1) & 1, st + 1);
+                if (st + 1 < (BK / 32) * DB) {
+                    load_vf((st + 1) & 1, st + 1);
+                    SCHED_DS_READ(2);
+                }
                 const int kp = st / DB, db = st % DB;
 #pragma unroll
                 for (int ob = 0; ob < 2; ++ob) acc_o[ob][db] = mfma_bf16(vf[st & 1], pf[ob][kp], acc_o[ob][db]);
+                SCHED_MFMA(2);
             }
         }
     };

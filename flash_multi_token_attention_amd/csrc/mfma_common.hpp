@@ -39,6 +39,12 @@ __device__ __forceinline__ f32x4 mfma_f16(f16x8 a, f16x8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
 }
 
+// Scheduling hints: the sequence of these calls in program order is the order in which the
+// backend lays out groups of LDS reads and MFMAs.  Used as "reads of stage s+1, then MFMAs
+// of stage s" so that fragment reads stay one stage ahead instead of sinking next to their use.
+#define SCHED_DS_READ(n) __builtin_amdgcn_sched_group_barrier(0x100, (n), 0)
+#define SCHED_MFMA(n) __builtin_amdgcn_sched_group_barrier(0x008, (n), 0)
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // Toeplitz fragment of query tap `a` for this lane: element e is
