@@ -5,16 +5,16 @@
 // before the window-aligned ones, keys c0-8 .. c0+23 for dV (the shifted ranges
 // of neighbouring waves and workgroups tile the key axis just the same).  The
 // wave keeps its K and V fragments and both accumulators in registers and walks
-// the queries in 32-row tiles that the workgroup stages row-major in LDS (Q
+// the queries in 64-row tiles that the workgroup stages row-major in LDS (Q
 // and dO; their transposes for the dK / dV products come from LDS transpose
 // reads).  Per tile, with r0 its first row:
-//   S^T  rows r0-16 .. r0+47, keys c0-16 .. c0+47    raw K Q^T, pre-masked, fp16 -> LDS
-//   C    rows r0 .. r0+47, keys c0-8 .. c0+39        Toeplitz MFMAs, here oriented
+//   S^T  rows r0-16 .. r0+79, keys c0-16 .. c0+47    raw K Q^T, pre-masked, fp16 -> LDS
+//   C    rows r0 .. r0+79, keys c0-8 .. c0+39        Toeplitz MFMAs, here oriented
 //        [query][key] so that a lane holds one key and 4 query rows: that is the
 //        operand layout the dV and dK products need, no transposition in between
 //   P = exp2(C - LSE), dP = dO V^T, dC = P (dP - D): fp16 -> LDS (2-byte stores)
-//   dV^T += dO^T P        (rows r0 .. r0+31, keys c0-8 .. c0+23)
-//   dS   rows r0 .. r0+31, keys c0 .. c0+31: flipped-band MFMAs over dC, causal zero
+//   dV^T += dO^T P        (rows r0 .. r0+63, keys c0-8 .. c0+23)
+//   dS   rows r0 .. r0+63, keys c0 .. c0+31: flipped-band MFMAs over dC, causal zero
 //   dK^T += Q^T dS        (the flipped bands carry the softmax scale)
 #include "mfma_common.hpp"
 
@@ -24,15 +24,16 @@ namespace {
 constexpr int NW = 4;
 constexpr int WK = 32;                 // own keys per wave
 constexpr int BKW = NW * WK;           // 128 keys per workgroup
-constexpr int BR = 32;                 // query rows per tile
-constexpr int S_ROWS = BR + 32;        // 64
+constexpr int BR = 64;                 // query rows per tile
+constexpr int S_ROWS = BR + 32;        // 96: 16 above, 16 below
 constexpr int S_COLS = WK + 32;        // 64
-constexpr int C_ROWS = BR + 16;        // 48
+constexpr int C_ROWS = BR + 16;        // 80
 constexpr int C_COLS = WK + 16;        // 48
 constexpr int SST = (S_COLS + 8) * 2;  // 144
 constexpr int CST = (C_COLS + 8) * 2;  // 112
 constexpr int NSB = S_COLS / 16;       // 4 key blocks of S
 constexpr int NCB = C_COLS / 16;       // 3 key blocks of C / dP / dC
+constexpr int NRB = BR / 16;           // 4 own row blocks per tile
 
 template <int D> struct KvLds {
     static constexpr int RST = D * 2 + 16;
@@ -164,9 +165,9 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
             load_qf(0, 0);
             SCHED_DS_READ(KS);
 #pragma unroll
-            for (int rb = 0; rb < 4; ++rb) {
+            for (int rb = 0; rb < S_ROWS / 16; ++rb) {
                 const int cur = rb & 1;
-                if (rb + 1 < 4) {
+                if (rb + 1 < S_ROWS / 16) {
                     load_qf(cur ^ 1, rb + 1);
                     SCHED_DS_READ(KS);
                 }
@@ -198,9 +199,9 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
         __builtin_amdgcn_wave_barrier();
 
         // ---- C, P, dP, dC ([query][key] orientation: lane = key, registers = 4 rows) ----
-        f32x4 pkeep[2][2];
+        f32x4 pkeep[NRB][2];
 #pragma unroll
-        for (int rb = 0; rb < 3; ++rb) {
+        for (int rb = 0; rb < C_ROWS / 16; ++rb) {
             const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(lse_s + rb * 16 + 4 * g);
             const f32x4 dl4 = *reinterpret_cast<const f32x4 *>(dl_s + rb * 16 + 4 * g);
             f32x4 c[NCB], dp[NCB];
@@ -268,52 +269,57 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                 for (int r = 0; r < 4; ++r)
                     *reinterpret_cast<_Float16 *>(Cs + (rb * 16 + 4 * g + r) * CST + (kb * 16 + n) * 2) =
                         (_Float16)__builtin_amdgcn_fmed3f(dc[r], -kF16Max, kF16Max);
-                if (rb < 2 && kb < 2) pkeep[rb][kb] = pr;
+                if (rb < NRB && kb < 2) pkeep[rb][kb] = pr;
             }
         }
         __builtin_amdgcn_wave_barrier();
 
         // ---- dV^T += dO^T P  (keys c0-8 .. c0+23); dO^T by transpose reads of the dO tile ----
         {
-            bf16x8 pf[2];
+            bf16x8 pf[NRB / 2][2];
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+            for (int kp = 0; kp < NRB / 2; ++kp)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    pf[kb][r] = (bf16_t)pkeep[0][kb][r];
-                    pf[kb][4 + r] = (bf16_t)pkeep[1][kb][r];
-                }
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        pf[kp][kb][r] = (bf16_t)pkeep[2 * kp][kb][r];
+                        pf[kp][kb][4 + r] = (bf16_t)pkeep[2 * kp + 1][kb][r];
+                    }
+            constexpr int NST = (NRB / 2) * DB;  // stage = (row pair, head-dim block)
             bf16x8 gt[2];
-            auto load_gt = [&](int buf, int db) {
-                bf16x4 lo = lds_read_tr4x16(Gs, RST, 4 * g, db * 16, n);
-                bf16x4 hi = lds_read_tr4x16(Gs, RST, 16 + 4 * g, db * 16, n);
+            auto load_gt = [&](int buf, int st) {
+                const int kp = st / DB, db = st % DB;
+                bf16x4 lo = lds_read_tr4x16(Gs, RST, kp * 32 + 4 * g, db * 16, n);
+                bf16x4 hi = lds_read_tr4x16(Gs, RST, kp * 32 + 16 + 4 * g, db * 16, n);
                 gt[buf] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
             };
             load_gt(0, 0);
             SCHED_DS_READ(2);
 #pragma unroll
-            for (int db = 0; db < DB; ++db) {
-                if (db + 1 < DB) {
-                    load_gt((db + 1) & 1, db + 1);
+            for (int st = 0; st < NST; ++st) {
+                if (st + 1 < NST) {
+                    load_gt((st + 1) & 1, st + 1);
                     SCHED_DS_READ(2);
                 }
+                const int kp = st / DB, db = st % DB;
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb) acc_v[kb][db] = mfma_bf16(gt[db & 1], pf[kb], acc_v[kb][db]);
+                for (int kb = 0; kb < 2; ++kb) acc_v[kb][db] = mfma_bf16(gt[st & 1], pf[kp][kb], acc_v[kb][db]);
                 SCHED_MFMA(2);
             }
         }
 
         // ---- dS (keys c0 .. c0+31): 4 chains over the taps ----
-        f32x4 ds[2][2];
+        f32x4 ds[NRB][2];
 #pragma unroll
-        for (int ob = 0; ob < 2; ++ob)
+        for (int ob = 0; ob < NRB; ++ob)
 #pragma unroll
             for (int m = 0; m < 2; ++m) ds[ob][m] = (f32x4){0.f, 0.f, 0.f, 0.f};
         {
-            constexpr int NST = 2 * CQT;  // stage = (tap slot, row block)
+            constexpr int NST = NRB * CQT;  // stage = (tap slot, row block)
             f16x8 cf[2][2];
             auto load_cf = [&](int buf, int st) {
-                const int a = st >> 1, ob = st & 1;
+                const int a = st / NRB, ob = st % NRB;
                 const unsigned char *base = Cs + (ob * 16 + n + (CQT - 1) - a) * CST + (8 * g) * 2;
                 cf[buf][0] = *reinterpret_cast<const f16x8 *>(base);
                 cf[buf][1] = *reinterpret_cast<const f16x8 *>(base + 32);
@@ -327,13 +333,13 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                     SCHED_DS_READ(2);
                 }
 #pragma unroll
-                for (int m = 0; m < 2; ++m) ds[st & 1][m] = mfma_f16(cf[st & 1][m], tfl[st >> 1], ds[st & 1][m]);
+                for (int m = 0; m < 2; ++m) ds[st % NRB][m] = mfma_f16(cf[st & 1][m], tfl[st / NRB], ds[st % NRB][m]);
                 SCHED_MFMA(2);
             }
         }
         if (edge && causal) {
 #pragma unroll
-            for (int ob = 0; ob < 2; ++ob)
+            for (int ob = 0; ob < NRB; ++ob)
 #pragma unroll
                 for (int m = 0; m < 2; ++m)
 #pragma unroll
@@ -342,30 +348,35 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
         }
         // ---- dK^T += Q^T dS; Q^T by transpose reads (own rows start at Q-tile row 16) ----
         {
-            bf16x8 sf[2];
+            bf16x8 sf[NRB / 2][2];
 #pragma unroll
-            for (int m = 0; m < 2; ++m)
+            for (int kp = 0; kp < NRB / 2; ++kp)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    sf[m][r] = (bf16_t)ds[0][m][r];
-                    sf[m][4 + r] = (bf16_t)ds[1][m][r];
-                }
+                for (int m = 0; m < 2; ++m)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        sf[kp][m][r] = (bf16_t)ds[2 * kp][m][r];
+                        sf[kp][m][4 + r] = (bf16_t)ds[2 * kp + 1][m][r];
+                    }
+            constexpr int NST = (NRB / 2) * DB;
             bf16x8 qt[2];
-            auto load_qt = [&](int buf, int db) {
-                bf16x4 lo = lds_read_tr4x16(Qs, RST, 16 + 4 * g, db * 16, n);
-                bf16x4 hi = lds_read_tr4x16(Qs, RST, 32 + 4 * g, db * 16, n);
+            auto load_qt = [&](int buf, int st) {
+                const int kp = st / DB, db = st % DB;
+                bf16x4 lo = lds_read_tr4x16(Qs, RST, 16 + kp * 32 + 4 * g, db * 16, n);
+                bf16x4 hi = lds_read_tr4x16(Qs, RST, 32 + kp * 32 + 4 * g, db * 16, n);
                 qt[buf] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
             };
             load_qt(0, 0);
             SCHED_DS_READ(2);
 #pragma unroll
-            for (int db = 0; db < DB; ++db) {
-                if (db + 1 < DB) {
-                    load_qt((db + 1) & 1, db + 1);
+            for (int st = 0; st < NST; ++st) {
+                if (st + 1 < NST) {
+                    load_qt((st + 1) & 1, st + 1);
                     SCHED_DS_READ(2);
                 }
+                const int kp = st / DB, db = st % DB;
 #pragma unroll
-                for (int m = 0; m < 2; ++m) acc_k[m][db] = mfma_bf16(qt[db & 1], sf[m], acc_k[m][db]);
+                for (int m = 0; m < 2; ++m) acc_k[m][db] = mfma_bf16(qt[st & 1], sf[kp][m], acc_k[m][db]);
                 SCHED_MFMA(2);
             }
         }
