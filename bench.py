@@ -141,16 +141,16 @@ def time_events(fn, iters, warmup):
     return a.elapsed_time(b) / iters
 
 
-def cpu_baseline(wl, budget_s=25.0):
+def cpu_baseline(wl, budget_s=12.0):
     """The oracle (same torch op sequence as the reference's PyTorch module plus
     autograd), fp32, on (batch, head) pairs of the workload until ``budget_s``
     of CPU time is spent; useful FLOPs of the pairs done / time."""
     from oracle import conv_attn_oracle as orc
-    t = synthetic.make_inputs(synthetic.Workload(**{**wl.__dict__, "B": 1, "H": 4}), seed=0)
+    t = synthetic.make_inputs(synthetic.Workload(**{**wl.__dict__, "B": 1, "H": 16}), seed=0)
     fl = synthetic.useful_flops(wl)
     per_pair = (fl["fwd"] + fl["bwd"]) / (wl.B * wl.H)
     done, t0 = 0, time.perf_counter()
-    while done < 4:
+    while done < 16:
         sl = slice(done, done + 1)
         Q, K, V, dO = (t[k][:, sl].float() for k in ("Q", "K", "V", "dO"))
         orc.backward_autograd(Q, K, V, t["W"][sl], dO, wl.causal, wl.scale)

@@ -206,3 +206,52 @@ def test_decode_full_size_properties():
         assert max_abs(o[0], base[0]) <= 1e-4 and rel_max(o[2], base[2]) <= 1e-4
     ones = decode(Q, K, torch.ones_like(V), W, 3, wl.scale)
     assert float((ones[0] - 1).abs().max()) <= 1e-4
+
+
+def test_c3_full_size_fwd_bwd_against_fp32_kernels():
+    # The headline workload at full size: MFMA kernels vs the fp32-arithmetic kernels on the GPU
+    # (the CPU oracle would need minutes), plus properties that do not depend on the size.
+    wl = synthetic.WORKLOADS["c3_fwd_bwd"]
+    t = {k: v.to(DEV) for k, v in synthetic.make_inputs(wl, seed=0).items()}
+    Q, K, V, dO, W = t["Q"], t["K"], t["V"], t["dO"], t["W"]
+    args = (wl.scale, wl.pad_q, wl.pad_k, True)
+    O, M, L = ops.forward(Q, K, V, W, *args, out_dtype=torch.bfloat16)
+    O_x, M_x, L_x = ops.forward(Q, K, V, W, *args, out_dtype=torch.float32, exact=True)
+    assert max_abs(O, O_x) <= TOL_BF16 and max_abs(M, M_x) <= TOL_BF16 and rel_max(L, L_x) <= TOL_BF16
+    D, LSE = ops.bwd_preprocess(O, dO, M, L)
+    D_x, LSE_x = ops.bwd_preprocess(O_x, dO, M_x, L_x)
+    dQ, dW = ops.dq_backward(Q, K, V, dO, D, LSE, W, *args, out_dtype=torch.bfloat16)
+    dK, dV = ops.dkdv_backward(Q, K, V, dO, D, LSE, W, *args, out_dtype=torch.bfloat16)
+    dQ_x, dW_x = ops.dq_backward(Q, K, V, dO, D_x, LSE_x, W, *args, exact=True)
+    dK_x, dV_x = ops.dkdv_backward(Q, K, V, dO, D_x, LSE_x, W, *args, exact=True)
+    assert max_abs(dQ, dQ_x) <= TOL_BF16
+    assert max_abs(dK, dK_x) <= TOL_BF16
+    assert max_abs(dV, dV_x) <= TOL_BF16
+    assert rel_max(dW, dW_x) <= TOL_DW_REL
+    # dV is linear in dO, dQ/dK/dW are too: doubling dO doubles them (D doubles with it)
+    dQ2, dW2 = ops.dq_backward(Q, K, V, (2 * dO.float()).to(torch.bfloat16), 2 * D, LSE, W, *args,
+                               out_dtype=torch.float32)
+    assert rel_max(dW2, 2 * dW) <= 1e-3
+    # row 0 attends to key 0 only: O[0] = V[0]
+    assert max_abs(O[:, :, 0], V[:, :, 0]) <= 1e-6
+
+
+def test_c5_long_context_one_head_forward_and_backward():
+    # N = 16384 (the long-context workload) for one (batch, head) pair with the decaying window
+    # of that workload: forward and backward against the fp32-arithmetic kernels.
+    wl = synthetic.Workload("c5_one_head", 1, 1, 16384, 16384, 128, 6, 11, sigma=0.1, key_decay=3.0,
+                            backward=True)
+    t = {k: v.to(DEV) for k, v in synthetic.make_inputs(wl, seed=0).items()}
+    Q, K, V, dO, W = t["Q"], t["K"], t["V"], t["dO"], t["W"]
+    args = (wl.scale, wl.pad_q, wl.pad_k, True)
+    O, M, L = ops.forward(Q, K, V, W, *args, out_dtype=torch.bfloat16)
+    O_x, M_x, L_x = ops.forward(Q, K, V, W, *args, out_dtype=torch.float32, exact=True)
+    assert max_abs(O, O_x) <= TOL_BF16 and max_abs(M, M_x) <= TOL_BF16
+    D, LSE = ops.bwd_preprocess(O, dO, M, L)
+    dQ, dW = ops.dq_backward(Q, K, V, dO, D, LSE, W, *args, out_dtype=torch.bfloat16)
+    dK, dV = ops.dkdv_backward(Q, K, V, dO, D, LSE, W, *args, out_dtype=torch.bfloat16)
+    D_x, LSE_x = ops.bwd_preprocess(O_x, dO, M_x, L_x)
+    dQ_x, dW_x = ops.dq_backward(Q, K, V, dO, D_x, LSE_x, W, *args, exact=True)
+    dK_x, dV_x = ops.dkdv_backward(Q, K, V, dO, D_x, LSE_x, W, *args, exact=True)
+    assert max_abs(dQ, dQ_x) <= TOL_BF16 and max_abs(dK, dK_x) <= TOL_BF16 and max_abs(dV, dV_x) <= TOL_BF16
+    assert rel_max(dW, dW_x) <= TOL_DW_REL
