@@ -20,8 +20,23 @@ INCLUDE = os.path.join(ROOT, "include")
 LIB_NAME = "libconvattn_hip.so"
 LIB_PATH = os.path.join(PKG_DIR, LIB_NAME)
 
-SOURCES = ["api.hip", "generic_kernels.hip", "reduce_kernels.hip", "fwd_mfma.hip", "bwd_dq_mfma.hip",
-           "bwd_dkdv_mfma.hip", "decode_stream.hip"]
+# MFMA results in ordinary VGPRs where the register allocator can afford it (the 512-register
+# backward kernels otherwise copy every transient accumulator out of the accumulation file).
+VGPR_FORM = ["-mllvm", "-amdgpu-mfma-vgpr-form"]
+
+# (source, object name, extra flags).  The dK/dV kernel is compiled in two halves: its 11-tap
+# instantiations crash this compiler's MFMA rewrite pass under VGPR_FORM, so they go without it.
+UNITS = [
+    ("api.hip", "api", []),
+    ("generic_kernels.hip", "generic_kernels", []),
+    ("reduce_kernels.hip", "reduce_kernels", []),
+    ("fwd_mfma.hip", "fwd_mfma", []),
+    ("bwd_dq_mfma.hip", "bwd_dq_mfma", VGPR_FORM),
+    ("bwd_dkdv_mfma.hip", "bwd_dkdv_mfma_narrow", ["-DCONVATTN_DKDV_UNIT=0", *VGPR_FORM]),
+    ("bwd_dkdv_mfma.hip", "bwd_dkdv_mfma_wide", ["-DCONVATTN_DKDV_UNIT=1"]),
+    ("decode_stream.hip", "decode_stream", []),
+]
+SOURCES = sorted({u[0] for u in UNITS})
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall",
@@ -55,14 +70,12 @@ def build(verbose: bool = True, extra_flags=()) -> str:
     obj_dir = os.path.join(ROOT, "build", "convattn_obj")
     os.makedirs(obj_dir, exist_ok=True)
     jobs = []
-    for name in SOURCES:
-        src = os.path.join(CSRC, name)
-        obj = os.path.join(obj_dir, os.path.splitext(name)[0] + ".o")
-        jobs.append((src, obj))
+    for name, obj_name, unit_flags in UNITS:
+        jobs.append((os.path.join(CSRC, name), os.path.join(obj_dir, obj_name + ".o"), unit_flags))
     with ThreadPoolExecutor(max_workers=min(8, len(jobs))) as ex:
-        list(ex.map(lambda so: _compile(cc, so[0], so[1], list(extra_flags)), jobs))
+        list(ex.map(lambda so: _compile(cc, so[0], so[1], [*so[2], *extra_flags]), jobs))
     tmp = LIB_PATH + ".tmp"
-    cmd = [cc, "--offload-arch=gfx950", "-shared", "-fPIC", *[o for _, o in jobs], "-o", tmp]
+    cmd = [cc, "--offload-arch=gfx950", "-shared", "-fPIC", *[j[1] for j in jobs], "-o", tmp]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stdout}\n{r.stderr}")

@@ -18,6 +18,10 @@
 //   dK^T += Q^T dS        (the flipped bands carry the softmax scale)
 #include "mfma_common.hpp"
 
+#ifndef CONVATTN_DKDV_UNIT
+#define CONVATTN_DKDV_UNIT 0
+#endif
+
 namespace convattn {
 namespace {
 
@@ -432,15 +436,39 @@ hipError_t launch_kv(const Problem &p, const void *q, const void *k, const void 
     return hipGetLastError();
 }
 
+}  // namespace
+
+// This file is built as two objects (CONVATTN_DKDV_UNIT = 0: windows of up to 6 query taps and
+// the public entry; 1: the 11-tap-slot instantiations), because the two sets need different
+// compiler options.
+template <int D, typename TO>
+hipError_t dkdv_wide(const Problem &p, const void *q, const void *k, const void *v, const void *d_o,
+                     const float *Dl, const float *lse, const float *w, void *dk, void *dv,
+                     hipStream_t s);
+
+#if CONVATTN_DKDV_UNIT == 1
+template <int D, typename TO>
+hipError_t dkdv_wide(const Problem &p, const void *q, const void *k, const void *v, const void *d_o,
+                     const float *Dl, const float *lse, const float *w, void *dk, void *dv,
+                     hipStream_t s) {
+    return launch_kv<D, 11, TO>(p, q, k, v, d_o, Dl, lse, w, dk, dv, s);
+}
+#define CONVATTN_INST(D, TO)                                                                          \
+    template hipError_t dkdv_wide<D, TO>(const Problem &, const void *, const void *, const void *,   \
+                                         const void *, const float *, const float *, const float *,   \
+                                         void *, void *, hipStream_t);
+CONVATTN_INST(128, bf16_t) CONVATTN_INST(128, float) CONVATTN_INST(64, bf16_t) CONVATTN_INST(64, float)
+#undef CONVATTN_INST
+#else
+namespace {
 template <int D, typename TO>
 hipError_t pick_cq(const Problem &p, const void *q, const void *k, const void *v, const void *d_o,
                    const float *Dl, const float *lse, const float *w, void *dk, void *dv,
                    hipStream_t s) {
     if (p.c_q <= 3) return launch_kv<D, 3, TO>(p, q, k, v, d_o, Dl, lse, w, dk, dv, s);
     if (p.c_q <= 6) return launch_kv<D, 6, TO>(p, q, k, v, d_o, Dl, lse, w, dk, dv, s);
-    return launch_kv<D, 11, TO>(p, q, k, v, d_o, Dl, lse, w, dk, dv, s);
+    return dkdv_wide<D, TO>(p, q, k, v, d_o, Dl, lse, w, dk, dv, s);
 }
-
 }  // namespace
 
 hipError_t mfma_bwd_dkdv(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
@@ -453,5 +481,6 @@ hipError_t mfma_bwd_dkdv(const Problem &p, int out_dt, const void *q, const void
     if (out_dt == CONVATTN_BF16) return pick_cq<64, bf16_t>(p, q, k, v, d_o, Dl, lse, w, dk, dv, s);
     return pick_cq<64, float>(p, q, k, v, d_o, Dl, lse, w, dk, dv, s);
 }
+#endif
 
 }  // namespace convattn
