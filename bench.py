@@ -2,7 +2,7 @@
 """Headline benchmark: conv-attention forward + backward on one MI355X.
 
 One step = training forward + backward (D/LSE preparation, dQ + dW partials,
-ordered dW reduction, dK/dV) of workload c3_fwd_bwd (B=4, H=16, N=4096, d=128,
+one-pass dK/dV/dW/dS kernel, dQ = dS K, ordered dW reduction) of workload c3_fwd_bwd (B=4, H=16, N=4096, d=128,
 6x11 window, bf16, causal) through the C ABI, inputs and outputs resident in
 HBM.  ``value`` is useful TFLOP/s: (4 + 10) * d * N(N+1)/2 * B * H matmul FLOPs
 per step; the convolution's work and every recomputed tile are not counted.
@@ -66,14 +66,25 @@ class TrainStep:
         nb = self.lib.convattn_dw_partial_bytes(C.byref(self.desc))
         assert nb > 0, "descriptor rejected"
         self.part = torch.empty(nb // 4, dtype=torch.float32, device=dev)
+        self.ws = torch.empty(self.lib.convattn_bwd_fused_workspace_bytes(C.byref(self.desc)), dtype=torch.uint8,
+                              device=dev)
         self.dW = torch.empty_like(self.W)
         self.stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
         d, s = C.byref(self.desc), self.stream
+        bwd_in = (_p(self.Q), _p(self.K), _p(self.V), _p(self.dO), _p(self.D), _p(self.LSE), _p(self.W))
+        # the step: forward, D/LSE, then the one-pass backward (its three launches timed one by one)
         self.kernels = {
             "fwd": lambda: self.lib.convattn_fwd(d, _p(self.Q), _p(self.K), _p(self.V), _p(self.W),
                                                  _p(self.O), _p(self.M), _p(self.L), s),
             "bwd_preprocess": lambda: self.lib.convattn_bwd_preprocess(
                 d, _p(self.O), _p(self.dO), _p(self.M), _p(self.L), _p(self.D), _p(self.LSE), s),
+            "bwd_fused_dkdv": lambda: self.lib.convattn_bwd_fused_dkdv(d, *bwd_in, _p(self.dK), _p(self.dV),
+                                                                        _p(self.ws), s),
+            "bwd_fused_dq": lambda: self.lib.convattn_bwd_fused_dq(d, *bwd_in, _p(self.dQ), _p(self.ws), s),
+            "bwd_fused_dw": lambda: self.lib.convattn_bwd_fused_dw(d, _p(self.ws), _p(self.dW), s),
+        }
+        # the two independent passes behind dq_backward / dkdv_backward (--two-pass, --only)
+        self.two_pass = {
             "bwd_dq_dw": lambda: self.lib.convattn_bwd_dq_dw(
                 d, _p(self.Q), _p(self.K), _p(self.V), _p(self.dO), _p(self.D), _p(self.LSE), _p(self.W),
                 _p(self.dQ), _p(self.part), s),
@@ -83,8 +94,12 @@ class TrainStep:
                 _p(self.dK), _p(self.dV), s),
         }
 
-    def step(self):
-        for name, fn in self.kernels.items():
+    def step(self, two_pass=False):
+        todo = dict(self.kernels)
+        if two_pass:
+            todo = {k: v for k, v in todo.items() if not k.startswith("bwd_fused")}
+            todo.update(self.two_pass)
+        for name, fn in todo.items():
             rc = fn()
             if rc:
                 raise RuntimeError(f"{name}: {_lib.strerror(rc)}")
@@ -174,6 +189,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-decode", action="store_true", help="skip the decode measurement")
     ap.add_argument("--only", default=None, help="run only this kernel of the step (for profiling)")
+    ap.add_argument("--two-pass", action="store_true",
+                    help="backward as the two independent passes (dQ+dW, dK/dV) instead of the one-pass backward")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; run with --gpus 1 "
@@ -200,11 +217,11 @@ def main():
             ms = time_events(ds.step, args.steps, args.warmup)
         else:
             ts.step()
-            ms = time_events(ts.kernels[args.only], args.steps, args.warmup)
+            ms = time_events({**ts.kernels, **ts.two_pass}[args.only], args.steps, args.warmup)
         print(json.dumps({"only": args.only, "ms": ms}))
         return
 
-    step = ts.step if wl.backward else ts.kernels["fwd"]
+    step = (lambda: ts.step(args.two_pass)) if wl.backward else ts.kernels["fwd"]
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -216,10 +233,16 @@ def main():
     useful = fl["fwd"] + (fl["bwd"] if wl.backward else 0.0)
 
     # per-kernel launch durations (HIP events, same stream)
-    names = list(ts.kernels) if wl.backward else ["fwd"]
-    k_ms = {n: time_events(ts.kernels[n], max(3, args.steps // 2), 1) for n in names}
-    # useful FLOPs a launch of each kernel is credited with (recompute not counted)
-    credit = {"fwd": fl["fwd"], "bwd_dq_dw": 0.6 * fl["bwd"], "bwd_dkdv": 0.4 * fl["bwd"]}
+    allk = {**ts.kernels, **ts.two_pass}
+    names = ["fwd"]
+    if wl.backward:
+        names = [n for n in ts.kernels if not (args.two_pass and n.startswith("bwd_fused"))]
+        names += list(ts.two_pass) if args.two_pass else []
+    k_ms = {n: time_events(allk[n], max(3, args.steps // 2), 1) for n in names}
+    # useful FLOPs a launch of each kernel is credited with (recompute not counted): the backward
+    # has five products of equal size (S, dP, dV, dK, dQ)
+    credit = {"fwd": fl["fwd"], "bwd_dq_dw": 0.6 * fl["bwd"], "bwd_dkdv": 0.4 * fl["bwd"],
+              "bwd_fused_dkdv": 0.8 * fl["bwd"], "bwd_fused_dq": 0.2 * fl["bwd"]}
     dom = max((n for n in names if n in credit), key=lambda n: k_ms[n])
     achieved = credit[dom] / (k_ms[dom] * 1e-3) / 1e12
     out = {

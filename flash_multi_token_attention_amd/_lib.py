@@ -40,6 +40,11 @@ _SIGNATURES = {
     "convattn_bwd_dq_dw": (C.c_int, [_D] + [_P] * 10),
     "convattn_dw_reduce": (C.c_int, [_D] + [_P] * 3),
     "convattn_bwd_dkdv": (C.c_int, [_D] + [_P] * 10),
+    "convattn_bwd_fused_workspace_bytes": (C.c_size_t, [_D]),
+    "convattn_bwd_fused": (C.c_int, [_D] + [_P] * 13),
+    "convattn_bwd_fused_dkdv": (C.c_int, [_D] + [_P] * 11),
+    "convattn_bwd_fused_dq": (C.c_int, [_D] + [_P] * 10),
+    "convattn_bwd_fused_dw": (C.c_int, [_D] + [_P] * 3),
     "convattn_decode_partial_bytes": (C.c_size_t, [_D]),
     "convattn_decode": (C.c_int, [_D] + [_P] * 8),
     "convattn_decode_combine": (C.c_int, [_D] + [_P] * 7),

@@ -25,7 +25,7 @@ LIB_PATH = os.path.join(PKG_DIR, LIB_NAME)
 VGPR_FORM = ["-mllvm", "-amdgpu-mfma-vgpr-form"]
 
 # (source, object name, extra flags).  The dK/dV kernel is compiled in two halves: its 11-tap
-# instantiations crash this compiler's MFMA rewrite pass under VGPR_FORM, so they go without it.
+# instantiations (plain and fused) crash this compiler's MFMA rewrite pass under VGPR_FORM, so they go without it.
 UNITS = [
     ("api.hip", "api", []),
     ("generic_kernels.hip", "generic_kernels", []),
@@ -34,6 +34,9 @@ UNITS = [
     ("bwd_dq_mfma.hip", "bwd_dq_mfma", VGPR_FORM),
     ("bwd_dkdv_mfma.hip", "bwd_dkdv_mfma_narrow", ["-DCONVATTN_DKDV_UNIT=0", *VGPR_FORM]),
     ("bwd_dkdv_mfma.hip", "bwd_dkdv_mfma_wide", ["-DCONVATTN_DKDV_UNIT=1"]),
+    ("bwd_dkdv_mfma.hip", "bwd_fused_mfma_narrow", ["-DCONVATTN_DKDV_UNIT=2", *VGPR_FORM]),
+    ("bwd_dkdv_mfma.hip", "bwd_fused_mfma_wide", ["-DCONVATTN_DKDV_UNIT=3"]),
+    ("bwd_dq_gemm.hip", "bwd_dq_gemm", []),
     ("decode_stream.hip", "decode_stream", []),
 ]
 SOURCES = sorted({u[0] for u in UNITS})

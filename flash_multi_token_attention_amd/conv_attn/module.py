@@ -38,6 +38,9 @@ class FlashConvAttentionCUDAFunction(torch.autograd.Function):
         args = (Q, K, V, dO, D, LSE, conv_kernel, ctx.scale, ctx.pad_q, ctx.pad_k, ctx.causal)
         need_q, need_k, need_v, need_w = ctx.needs_input_grad[:4]
         dQ = dW = dK = dV = None
+        if (need_q or need_w) and (need_k or need_v):
+            dQ, dK, dV, dW = ops.backward(*args, out_dtype=Q.dtype)
+            return dQ, dK, dV, dW.to(conv_kernel.dtype), None, None, None, None
         if need_q or need_w:
             dQ, dW = ops.dq_backward(*args, out_dtype=Q.dtype)
             dW = dW.to(conv_kernel.dtype)

@@ -183,6 +183,28 @@ def dkdv_backward(Q, K, V, dO, D, L, conv_kernel, scale, pad_q, pad_k, causal,
     return dK, dV
 
 
+def backward(Q, K, V, dO, D, L, conv_kernel, scale, pad_q, pad_k, causal,
+             out_dtype=torch.float32, exact=False):
+    """-> (dQ, dK, dV, dconv_kernel) from one pass over the score tiles: the results of
+    ``dq_backward`` + ``dkdv_backward`` (same arguments) without computing the scores, the
+    convolution and dC twice.  Needs a workspace the size of the bf16 dS matrix."""
+    W, D, L, desc = _bwd_common(Q, K, V, dO, D, L, conv_kernel, scale, pad_q, pad_k, causal,
+                                out_dtype, exact)
+    lib = _lib.load()
+    nbytes = lib.convattn_bwd_fused_workspace_bytes(C.byref(desc))
+    if nbytes == 0:
+        _lib.check(lib.convattn_validate(C.byref(desc), _lib.OP_BWD), "conv_attn.backward")
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=Q.device)
+    dQ = torch.empty(Q.shape, dtype=out_dtype, device=Q.device)
+    dK = torch.empty(K.shape, dtype=out_dtype, device=Q.device)
+    dV = torch.empty(V.shape, dtype=out_dtype, device=Q.device)
+    dW = torch.empty(W.shape, dtype=torch.float32, device=Q.device)
+    rc = lib.convattn_bwd_fused(C.byref(desc), _ptr(Q), _ptr(K), _ptr(V), _ptr(dO), _ptr(D), _ptr(L),
+                                _ptr(W), _ptr(dQ), _ptr(dK), _ptr(dV), _ptr(dW), _ptr(ws), _stream(Q))
+    _lib.check(rc, "conv_attn.backward")
+    return dQ, dK, dV, dW
+
+
 def default_k_splits(B: int, H: int, Nk: int) -> int:
     """Enough (batch, head, split) workgroups to fill 256 CUs a few times over."""
     want = max(1, (4 * 256 + B * H - 1) // (B * H))

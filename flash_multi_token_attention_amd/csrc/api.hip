@@ -56,6 +56,11 @@ int dw_tiles(const convattn_desc *d, const Problem &p) {
     return pick_path(d, p, CONVATTN_OP_BWD) == 1 ? mfma_dq_tiles(p) : generic_q_tiles(p);
 }
 
+size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
+size_t fused_dw_bytes(const Problem &p) {
+    return (size_t)p.B * p.H * mfma_kv_tiles(p) * p.c_q * p.c_k * sizeof(float);
+}
+
 #define REQUIRE_PTR(x)                                   \
     do {                                                 \
         if (!(x)) return CONVATTN_ERR_NULL;              \
@@ -162,6 +167,67 @@ int convattn_bwd_dkdv(const convattn_desc *desc, const void *q, const void *k, c
     if (pick_path(desc, p, CONVATTN_OP_BWD) == 1)
         return (int)mfma_bwd_dkdv(p, desc->out_dtype, q, k, v, d_o, D, lse, w, dk, dv, s);
     return (int)generic_bwd_dkdv(p, desc->in_dtype, desc->out_dtype, q, k, v, d_o, D, lse, w, dk, dv, s);
+}
+
+size_t convattn_bwd_fused_workspace_bytes(const convattn_desc *desc) {
+    Problem p;
+    if (validate(desc, CONVATTN_OP_BWD, &p)) return 0;
+    if (pick_path(desc, p, CONVATTN_OP_BWD) != 1) return align256(convattn_dw_partial_bytes(desc));
+    return align256(mfma_ds_bytes(p)) + align256(fused_dw_bytes(p));
+}
+
+int convattn_bwd_fused_dkdv(const convattn_desc *desc, const void *q, const void *k, const void *v,
+                            const void *d_o, const float *D, const float *lse, const float *w, void *dk,
+                            void *dv, void *workspace, void *stream) {
+    Problem p;
+    int rc = validate(desc, CONVATTN_OP_BWD, &p);
+    if (rc) return rc;
+    REQUIRE_PTR(q); REQUIRE_PTR(k); REQUIRE_PTR(v); REQUIRE_PTR(d_o); REQUIRE_PTR(D);
+    REQUIRE_PTR(lse); REQUIRE_PTR(w); REQUIRE_PTR(dk); REQUIRE_PTR(dv); REQUIRE_PTR(workspace);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (pick_path(desc, p, CONVATTN_OP_BWD) != 1)
+        return (int)generic_bwd_dkdv(p, desc->in_dtype, desc->out_dtype, q, k, v, d_o, D, lse, w, dk, dv, s);
+    unsigned char *ws = static_cast<unsigned char *>(workspace);
+    float *part = reinterpret_cast<float *>(ws + align256(mfma_ds_bytes(p)));
+    return (int)mfma_bwd_fused(p, desc->out_dtype, q, k, v, d_o, D, lse, w, dk, dv, ws, part, s);
+}
+
+int convattn_bwd_fused_dq(const convattn_desc *desc, const void *q, const void *k, const void *v,
+                          const void *d_o, const float *D, const float *lse, const float *w, void *dq,
+                          void *workspace, void *stream) {
+    Problem p;
+    int rc = validate(desc, CONVATTN_OP_BWD, &p);
+    if (rc) return rc;
+    REQUIRE_PTR(k); REQUIRE_PTR(dq); REQUIRE_PTR(workspace);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (pick_path(desc, p, CONVATTN_OP_BWD) != 1) {
+        // fp32-arithmetic kernels: the separate dQ pass, its dW partials go to the workspace
+        REQUIRE_PTR(q); REQUIRE_PTR(v); REQUIRE_PTR(d_o); REQUIRE_PTR(D); REQUIRE_PTR(lse); REQUIRE_PTR(w);
+        return (int)generic_bwd_dq_dw(p, desc->in_dtype, desc->out_dtype, q, k, v, d_o, D, lse, w, dq,
+                                      static_cast<float *>(workspace), s);
+    }
+    return (int)mfma_dq_from_ds(p, desc->out_dtype, k, workspace, dq, s);
+}
+
+int convattn_bwd_fused_dw(const convattn_desc *desc, const void *workspace, float *dw, void *stream) {
+    Problem p;
+    int rc = validate(desc, CONVATTN_OP_BWD, &p);
+    if (rc) return rc;
+    REQUIRE_PTR(workspace); REQUIRE_PTR(dw);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (pick_path(desc, p, CONVATTN_OP_BWD) != 1)
+        return (int)dw_reduce(p, dw_tiles(desc, p), static_cast<const float *>(workspace), dw, s);
+    const unsigned char *ws = static_cast<const unsigned char *>(workspace);
+    return (int)dw_reduce(p, mfma_kv_tiles(p), reinterpret_cast<const float *>(ws + align256(mfma_ds_bytes(p))), dw, s);
+}
+
+int convattn_bwd_fused(const convattn_desc *desc, const void *q, const void *k, const void *v,
+                       const void *d_o, const float *D, const float *lse, const float *w, void *dq,
+                       void *dk, void *dv, float *dw, void *workspace, void *stream) {
+    int rc = convattn_bwd_fused_dkdv(desc, q, k, v, d_o, D, lse, w, dk, dv, workspace, stream);
+    if (rc == 0) rc = convattn_bwd_fused_dq(desc, q, k, v, d_o, D, lse, w, dq, workspace, stream);
+    if (rc == 0) rc = convattn_bwd_fused_dw(desc, workspace, dw, stream);
+    return rc;
 }
 
 size_t convattn_decode_partial_bytes(const convattn_desc *desc) {

@@ -16,6 +16,15 @@
 //   dV^T += dO^T P        (rows r0 .. r0+63, keys c0-8 .. c0+23)
 //   dS   rows r0 .. r0+63, keys c0 .. c0+31: flipped-band MFMAs over dC, causal zero
 //   dK^T += Q^T dS        (the flipped bands carry the softmax scale)
+//
+// FUSED instantiations do the whole backward in this one pass over the score tiles: they also
+//   * store dS (bf16, the operand of dK) to a workspace as [key tile of 32][row tile of 64]
+//     blocks of [32 keys][64 rows]; dQ = dS K is then a plain batched product (bwd_dq_gemm.hip);
+//   * accumulate dW[a][b] += sum over own rows i and own keys j' of
+//     S[i+a-pq][j'] * dC[i][j'-b+pk]: an MFMA contraction with M = a, N = b and (row, 8 keys)
+//     as the k index; the dC operand is read from LDS at a 2-byte granular offset.  Every
+//     (dC row, S key) pair belongs to exactly one (wave, tile); the waves' partials are summed
+//     in a fixed order and stored per workgroup.
 #include "mfma_common.hpp"
 
 #ifndef CONVATTN_DKDV_UNIT
@@ -38,6 +47,7 @@ constexpr int CST = (C_COLS + 8) * 2;  // 112
 constexpr int NSB = S_COLS / 16;       // 4 key blocks of S
 constexpr int NCB = C_COLS / 16;       // 3 key blocks of C / dP / dC
 constexpr int NRB = BR / 16;           // 4 own row blocks per tile
+static_assert(BKW == kKvKeysPerWg && WK == kDsKeys && BR == kDsRows, "dS workspace layout");
 
 template <int D> struct KvLds {
     static constexpr int RST = D * 2 + 16;
@@ -48,12 +58,12 @@ template <int D> struct KvLds {
     static constexpr int total = q_bytes + g_bytes + stat_bytes + NW * wave_bytes;
 };
 
-template <int D, int CQT, typename TO>
+template <int D, int CQT, typename TO, bool FUSED>
 __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
     Problem p, const bf16_t *__restrict__ Q, const bf16_t *__restrict__ K,
     const bf16_t *__restrict__ V, const bf16_t *__restrict__ dO, const float *__restrict__ Dl,
     const float *__restrict__ LSE, const float *__restrict__ W, TO *__restrict__ dK,
-    TO *__restrict__ dV) {
+    TO *__restrict__ dV, bf16_t *__restrict__ dS_ws, float *__restrict__ dW_part) {
     using Lds = KvLds<D>;
     constexpr int RST = Lds::RST;
     constexpr int KS = D / 32, DB = D / 16, CPR = D / 8;
@@ -110,6 +120,16 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
             acc_k[m][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
             acc_v[m][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
         }
+
+    f32x4 acc_w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc_w[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    const int bcl = n < ck ? n : ck - 1;  // dW: lanes past the last key tap re-read a valid one
+    const int pq = p.pq;
+    // dS workspace blocks of this wave: [key tile][row tile][32 keys][64 rows]
+    const int n_rt = (p.Nq + BR - 1) / BR;
+    bf16_t *ds_wave = nullptr;
+    if constexpr (FUSED) ds_wave = dS_ws + ((bh * gridDim.z * NW + blockIdx.z * NW + wave) * n_rt) * (size_t)(WK * BR);
 
     // Causal: rows before the first key this workgroup touches (k0 - 8) see none of its keys.
     const int r_begin = causal ? (max(0, k0 - 8) / BR) * BR : 0;
@@ -362,6 +382,18 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                         sf[kp][m][r] = (bf16_t)ds[2 * kp][m][r];
                         sf[kp][m][4 + r] = (bf16_t)ds[2 * kp + 1][m][r];
                     }
+            if constexpr (FUSED) {
+                // lane = key m*16+n; elements 0..3 / 4..7 are rows 4g.. of row blocks 2kp / 2kp+1
+                bf16_t *blk = ds_wave + (size_t)(r0 / BR) * (WK * BR);
+#pragma unroll
+                for (int kp = 0; kp < NRB / 2; ++kp)
+#pragma unroll
+                    for (int m = 0; m < 2; ++m) {
+                        bf16_t *dst = blk + (m * 16 + n) * BR + kp * 32 + 4 * g;
+                        *reinterpret_cast<bf16x4 *>(dst) = __builtin_shufflevector(sf[kp][m], sf[kp][m], 0, 1, 2, 3);
+                        *reinterpret_cast<bf16x4 *>(dst + 16) = __builtin_shufflevector(sf[kp][m], sf[kp][m], 4, 5, 6, 7);
+                    }
+            }
             constexpr int NST = (NRB / 2) * DB;
             bf16x8 qt[2];
             auto load_qt = [&](int buf, int st) {
@@ -382,6 +414,39 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
 #pragma unroll
                 for (int m = 0; m < 2; ++m) acc_k[m][db] = mfma_bf16(qt[st & 1], sf[kp][m], acc_k[m][db]);
                 SCHED_MFMA(2);
+            }
+        }
+
+        // ---- dW: rows m = tap a, columns n = tap b, contraction over (own row, 8 own keys) ----
+        if constexpr (FUSED) {
+            // A: S[i + a - pq][c0 + 8g ..]        (S-tile row 16 + i + a - pq, column 16 + 8g)
+            // B: dC[i][c0 + 8g - b + pk ..]       (dC-tile column 8 + 8g - b + pk)
+            const unsigned char *abase = Ss + (16 + n - pq) * SST + (16 + 8 * g) * 2;
+            // LDS reads at odd 2-byte offsets are slow: read 5 dwords from the even
+            // element below and funnel-shift by 0 or 16 bits per lane instead.
+            const int boff = 8 + 8 * g - bcl + pk;
+            const unsigned char *bbase = Cs + (boff & ~1) * 2;
+            const unsigned int bsh = (boff & 1) * 16;
+#pragma unroll 1
+            for (int i = 0; i < BR; i += 4) {
+                f16x8 af[4];
+                u32x4 bw[4];
+                unsigned int bx[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    af[u] = *reinterpret_cast<const f16x8 *>(abase + (i + u) * SST);
+                    bw[u] = reinterpret_cast<const U32x4A4 *>(bbase + (i + u) * CST)->v;
+                    bx[u] = *reinterpret_cast<const unsigned int *>(bbase + (i + u) * CST + 16);
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    u32x4 sh;
+                    sh[0] = __builtin_amdgcn_alignbit(bw[u][1], bw[u][0], bsh);
+                    sh[1] = __builtin_amdgcn_alignbit(bw[u][2], bw[u][1], bsh);
+                    sh[2] = __builtin_amdgcn_alignbit(bw[u][3], bw[u][2], bsh);
+                    sh[3] = __builtin_amdgcn_alignbit(bx[u], bw[u][3], bsh);
+                    acc_w[u] = mfma_f16(af[u], __builtin_bit_cast(f16x8, sh), acc_w[u]);
+                }
             }
         }
     }
@@ -418,69 +483,102 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
             }
         }
     }
+
+    // ---- dW partial of this workgroup: ordered sum over the 4 waves; S was raw, so * scale ----
+    if constexpr (FUSED) {
+        __syncthreads();
+        float *red = reinterpret_cast<float *>(smem);  // [NW][16][16]
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            red[(wave * 16 + 4 * g + r) * 16 + n] = (acc_w[0][r] + acc_w[1][r]) + (acc_w[2][r] + acc_w[3][r]);
+        __syncthreads();
+        const int ntap = cq * ck;
+        if (tid < ntap) {
+            const int a = tid / ck, bb = tid - a * ck;
+            float sum = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) sum += red[(w * 16 + a) * 16 + bb];
+            dW_part[(bh * gridDim.z + blockIdx.z) * ntap + tid] = sum * p.scale;
+        }
+    }
 }
 
-template <int D, int CQT, typename TO>
+template <int D, int CQT, typename TO, bool FUSED>
 hipError_t launch_kv(const Problem &p, const void *q, const void *k, const void *v, const void *d_o,
-                     const float *Dl, const float *lse, const float *w, void *dk, void *dv,
-                     hipStream_t s) {
-    auto kern = bwd_dkdv_mfma_kernel<D, CQT, TO>;
+                     const float *Dl, const float *lse, const float *w, void *dk, void *dv, void *ds_ws,
+                     float *dw_part, hipStream_t s) {
+    auto kern = bwd_dkdv_mfma_kernel<D, CQT, TO, FUSED>;
     constexpr int lds = KvLds<D>::total;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return e;
-    // + 8: the last workgroup's dV range starts 8 keys early, so the key axis needs 8 more
-    dim3 grid(p.H, p.B, (p.Nk + 8 + BKW - 1) / BKW);
+    dim3 grid(p.H, p.B, mfma_kv_tiles(p));
     kern<<<grid, NW * 64, lds, s>>>(p, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v,
-                                    (const bf16_t *)d_o, Dl, lse, w, (TO *)dk, (TO *)dv);
+                                    (const bf16_t *)d_o, Dl, lse, w, (TO *)dk, (TO *)dv, (bf16_t *)ds_ws,
+                                    dw_part);
     return hipGetLastError();
 }
 
 }  // namespace
 
-// This file is built as two objects (CONVATTN_DKDV_UNIT = 0: windows of up to 6 query taps and
-// the public entry; 1: the 11-tap-slot instantiations), because the two sets need different
-// compiler options.
-template <int D, typename TO>
+// This file is built as four objects, CONVATTN_DKDV_UNIT = 2 * fused + wide: "wide" holds the
+// 11-tap-slot instantiations (they need different compiler options from the rest), "fused" the
+// whole-backward variants; the two narrow units also hold the entry points.
+template <int D, typename TO, bool FUSED>
 hipError_t dkdv_wide(const Problem &p, const void *q, const void *k, const void *v, const void *d_o,
-                     const float *Dl, const float *lse, const float *w, void *dk, void *dv,
-                     hipStream_t s);
+                     const float *Dl, const float *lse, const float *w, void *dk, void *dv, void *ds_ws,
+                     float *dw_part, hipStream_t s);
 
-#if CONVATTN_DKDV_UNIT == 1
-template <int D, typename TO>
+constexpr bool kFusedUnit = (CONVATTN_DKDV_UNIT & 2) != 0;
+
+#if CONVATTN_DKDV_UNIT & 1
+template <int D, typename TO, bool FUSED>
 hipError_t dkdv_wide(const Problem &p, const void *q, const void *k, const void *v, const void *d_o,
-                     const float *Dl, const float *lse, const float *w, void *dk, void *dv,
-                     hipStream_t s) {
-    return launch_kv<D, 11, TO>(p, q, k, v, d_o, Dl, lse, w, dk, dv, s);
+                     const float *Dl, const float *lse, const float *w, void *dk, void *dv, void *ds_ws,
+                     float *dw_part, hipStream_t s) {
+    return launch_kv<D, 11, TO, FUSED>(p, q, k, v, d_o, Dl, lse, w, dk, dv, ds_ws, dw_part, s);
 }
-#define CONVATTN_INST(D, TO)                                                                          \
-    template hipError_t dkdv_wide<D, TO>(const Problem &, const void *, const void *, const void *,   \
-                                         const void *, const float *, const float *, const float *,   \
-                                         void *, void *, hipStream_t);
+#define CONVATTN_INST(D, TO)                                                                             \
+    template hipError_t dkdv_wide<D, TO, kFusedUnit>(const Problem &, const void *, const void *,        \
+                                                     const void *, const void *, const float *,          \
+                                                     const float *, const float *, void *, void *,       \
+                                                     void *, float *, hipStream_t);
 CONVATTN_INST(128, bf16_t) CONVATTN_INST(128, float) CONVATTN_INST(64, bf16_t) CONVATTN_INST(64, float)
 #undef CONVATTN_INST
 #else
 namespace {
 template <int D, typename TO>
 hipError_t pick_cq(const Problem &p, const void *q, const void *k, const void *v, const void *d_o,
-                   const float *Dl, const float *lse, const float *w, void *dk, void *dv,
-                   hipStream_t s) {
-    if (p.c_q <= 3) return launch_kv<D, 3, TO>(p, q, k, v, d_o, Dl, lse, w, dk, dv, s);
-    if (p.c_q <= 6) return launch_kv<D, 6, TO>(p, q, k, v, d_o, Dl, lse, w, dk, dv, s);
-    return dkdv_wide<D, TO>(p, q, k, v, d_o, Dl, lse, w, dk, dv, s);
+                   const float *Dl, const float *lse, const float *w, void *dk, void *dv, void *ds_ws,
+                   float *dw_part, hipStream_t s) {
+    if (p.c_q <= 3) return launch_kv<D, 3, TO, kFusedUnit>(p, q, k, v, d_o, Dl, lse, w, dk, dv, ds_ws, dw_part, s);
+    if (p.c_q <= 6) return launch_kv<D, 6, TO, kFusedUnit>(p, q, k, v, d_o, Dl, lse, w, dk, dv, ds_ws, dw_part, s);
+    return dkdv_wide<D, TO, kFusedUnit>(p, q, k, v, d_o, Dl, lse, w, dk, dv, ds_ws, dw_part, s);
+}
+template <typename... A>
+hipError_t pick_d(const Problem &p, int out_dt, A... a) {
+    if (p.d == 128) {
+        if (out_dt == CONVATTN_BF16) return pick_cq<128, bf16_t>(p, a...);
+        return pick_cq<128, float>(p, a...);
+    }
+    if (out_dt == CONVATTN_BF16) return pick_cq<64, bf16_t>(p, a...);
+    return pick_cq<64, float>(p, a...);
 }
 }  // namespace
 
+#if CONVATTN_DKDV_UNIT & 2
+hipError_t mfma_bwd_fused(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
+                          const void *d_o, const float *Dl, const float *lse, const float *w, void *dk,
+                          void *dv, void *ds_ws, float *dw_part, hipStream_t s) {
+    return pick_d(p, out_dt, q, k, v, d_o, Dl, lse, w, dk, dv, ds_ws, dw_part, s);
+}
+#else
 hipError_t mfma_bwd_dkdv(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
                          const void *d_o, const float *Dl, const float *lse, const float *w, void *dk,
                          void *dv, hipStream_t s) {
-    if (p.d == 128) {
-        if (out_dt == CONVATTN_BF16) return pick_cq<128, bf16_t>(p, q, k, v, d_o, Dl, lse, w, dk, dv, s);
-        return pick_cq<128, float>(p, q, k, v, d_o, Dl, lse, w, dk, dv, s);
-    }
-    if (out_dt == CONVATTN_BF16) return pick_cq<64, bf16_t>(p, q, k, v, d_o, Dl, lse, w, dk, dv, s);
-    return pick_cq<64, float>(p, q, k, v, d_o, Dl, lse, w, dk, dv, s);
+    return pick_d(p, out_dt, q, k, v, d_o, Dl, lse, w, dk, dv, (void *)nullptr, (float *)nullptr, s);
 }
+#endif
 #endif
 
 }  // namespace convattn

@@ -149,6 +149,40 @@ int convattn_bwd_dkdv(const convattn_desc *desc, const void *q, const void *k, c
                       const void *d_o, const float *D, const float *lse, const float *w,
                       void *dk, void *dv, void *stream);
 
+/*
+ * The whole backward in one call: dQ, dK, dV and dW from one pass over the score tiles.
+ * Same results as convattn_bwd_dq_dw + convattn_dw_reduce + convattn_bwd_dkdv, which recompute
+ * the scores, the convolution and dC once each; this entry computes them once, keeps dS
+ * (bf16) in `workspace` and forms dQ = dS K from it.  It is what the autograd function of
+ * the reference (conv_attn/conv_attention_cuda.py:119-190, which calls dq_backward and then
+ * dkdv_backward) amounts to when both results are wanted.  `workspace` is device memory of
+ * convattn_bwd_fused_workspace_bytes(desc) bytes, 256-byte aligned; its contents need not be
+ * initialised and mean nothing afterwards.  dW is written (not accumulated).
+ */
+size_t convattn_bwd_fused_workspace_bytes(const convattn_desc *desc);
+int convattn_bwd_fused(const convattn_desc *desc, const void *q, const void *k, const void *v,
+                       const void *d_o, const float *D, const float *lse, const float *w,
+                       void *dq, void *dk, void *dv, float *dw, void *workspace, void *stream);
+
+/*
+ * The three steps of convattn_bwd_fused, for callers that order or time them themselves.
+ * They must run in this order on one stream (or with the caller's own dependencies) and share
+ * one workspace: _dkdv writes dK, dV and, into the workspace, dS and the dW partials; _dq
+ * forms dQ from the workspace (the arguments other than k, dq and workspace are only read
+ * for shapes the fp32-arithmetic kernels handle, where this step is the separate dQ pass);
+ * _dw sums the partials into dW.  Counterparts in the reference as for convattn_bwd_dkdv
+ * (conv_attn/kernels/dkdv_wrapper.cu:12-89), convattn_bwd_dq_dw
+ * (conv_attn/kernels/dq_bwd_wrapper.cu:11-93) and the float-atomic accumulation of dW
+ * (conv_attn/kernels/dq_bwd.cu:498-501).
+ */
+int convattn_bwd_fused_dkdv(const convattn_desc *desc, const void *q, const void *k, const void *v,
+                            const void *d_o, const float *D, const float *lse, const float *w,
+                            void *dk, void *dv, void *workspace, void *stream);
+int convattn_bwd_fused_dq(const convattn_desc *desc, const void *q, const void *k, const void *v,
+                          const void *d_o, const float *D, const float *lse, const float *w,
+                          void *dq, void *workspace, void *stream);
+int convattn_bwd_fused_dw(const convattn_desc *desc, const void *workspace, float *dw, void *stream);
+
 /* Bytes of o_part (fp32 [B,H,n_splits,d]); m_part and l_part are fp32 [B,H,n_splits]. */
 size_t convattn_decode_partial_bytes(const convattn_desc *desc);
 

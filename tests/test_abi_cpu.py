@@ -96,6 +96,19 @@ def test_dw_partial_size_matches_tiling(lib):
     assert n > 0 and n % (2 * 4 * 66 * 4) == 0
 
 
+def test_fused_backward_workspace_size(lib):
+    # bf16, N = 128, d = 64: dS blocks for ceil((128 + 8) / 128) * 4 key tiles x 2 row tiles of
+    # 32 x 64 bf16 per (batch, head), then one dW partial per 128-key workgroup; both 256-aligned
+    n = lib.convattn_bwd_fused_workspace_bytes(C.byref(desc()))
+    assert n == 2 * 4 * 8 * 2 * 32 * 64 * 2 + (2 * 4 * 2 * 66 * 4 + 255) // 256 * 256
+    # fp32 inputs run the two fp32 passes: the workspace is only the dW partial buffer
+    f32 = desc(in_dtype=_lib.F32, out_dtype=_lib.F32)
+    assert lib.convattn_bwd_fused_workspace_bytes(C.byref(f32)) == lib.convattn_dw_partial_bytes(C.byref(f32))
+    assert lib.convattn_bwd_fused_workspace_bytes(C.byref(desc(d=3))) == 0
+    ok = C.c_void_p(4096)
+    assert lib.convattn_bwd_fused(C.byref(desc()), ok, ok, ok, ok, ok, ok, ok, ok, ok, ok, ok, None, None) == -1
+
+
 def test_python_shim_errors_without_gpu():
     Q = torch.zeros(1, 2, 8, 64, dtype=torch.bfloat16)
     W = torch.zeros(2, 3, 3)

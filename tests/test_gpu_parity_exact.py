@@ -76,6 +76,9 @@ def test_backward_fp32(shape, causal):
     # fixed-order reduction: bitwise repeatable
     dQ2, dW2 = ops.dq_backward(g[0], g[1], g[2], g[3], D, LSE, g[4], sc, pq, pk, causal)
     assert torch.equal(dW, dW2) and torch.equal(dQ, dQ2)
+    # the whole-backward entry point runs the same fp32 kernels for these shapes
+    dQ3, dK3, dV3, dW3 = ops.backward(g[0], g[1], g[2], g[3], D, LSE, g[4], sc, pq, pk, causal)
+    assert torch.equal(dQ3, dQ) and torch.equal(dK3, dK) and torch.equal(dV3, dV) and torch.equal(dW3, dW)
 
 
 def test_bf16_inputs_exact_kernels_fwd_bwd():

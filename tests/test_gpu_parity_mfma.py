@@ -88,12 +88,17 @@ BWD_SHAPES = [
 ]
 
 
-def _run_bwd(Q, K, V, dO, W, causal, odt):
+def _run_bwd(Q, K, V, dO, W, causal, odt, one_pass=False):
+    """Backward through the two independent passes the reference exposes (dq_backward,
+    dkdv_backward) or, with ``one_pass``, through the single-pass backward."""
     d = Q.shape[-1]
     c_q, c_k = W.shape[1:]
     sc, pq, pk = scale_of(d), c_q - 1, (c_k - 1) // 2
     O, M, L = ops.forward(Q, K, V, W, sc, pq, pk, causal, out_dtype=odt)
     D, LSE = ops.bwd_preprocess(O, dO, M, L)
+    if one_pass:
+        dQ, dK, dV, dW = ops.backward(Q, K, V, dO, D, LSE, W, sc, pq, pk, causal, out_dtype=odt)
+        return dQ, dK, dV, dW
     dQ, dW = ops.dq_backward(Q, K, V, dO, D, LSE, W, sc, pq, pk, causal, out_dtype=odt)
     dK, dV = ops.dkdv_backward(Q, K, V, dO, D, LSE, W, sc, pq, pk, causal, out_dtype=odt)
     return dQ, dK, dV, dW
@@ -101,14 +106,15 @@ def _run_bwd(Q, K, V, dO, W, causal, odt):
 
 @pytest.mark.parametrize("shape", BWD_SHAPES)
 @pytest.mark.parametrize("causal", [True, False])
-def test_backward_bf16_mfma(shape, causal):
+@pytest.mark.parametrize("one_pass", [False, True])
+def test_backward_bf16_mfma(shape, causal, one_pass):
     B, H, N, d, c_q, c_k = shape
     Q, K, V, dO, W = rand_case(B, H, N, N, d, c_q, c_k, torch.bfloat16, seed=3 * N + c_q)
     ref = oracle_bwd(Q, K, V, W, dO, causal)
     g = [t.to(DEV) for t in (Q, K, V, dO, W)]
     assert ops.kernel_path(g[0], g[1], g[4], causal, op="bwd") == "mfma"
     for odt in (torch.bfloat16, torch.float32):
-        dQ, dK, dV, dW = _run_bwd(*g, causal, odt)
+        dQ, dK, dV, dW = _run_bwd(*g, causal, odt, one_pass)
         assert dQ.dtype == odt and dW.dtype == torch.float32
         assert max_abs(dQ, ref[0]) <= TOL_BF16
         assert max_abs(dK, ref[1]) <= TOL_BF16
@@ -116,27 +122,45 @@ def test_backward_bf16_mfma(shape, causal):
         assert rel_max(dW, ref[3]) <= TOL_DW_REL
 
 
-def test_backward_random_window_weights_and_determinism():
+@pytest.mark.parametrize("one_pass", [False, True])
+def test_backward_random_window_weights_and_determinism(one_pass):
     Q, K, V, dO, W = rand_case(2, 2, 260, 260, 128, 6, 11, torch.bfloat16, seed=8, w_mode="rand")
     ref = oracle_bwd(Q, K, V, W, dO, True)
     g = [t.to(DEV) for t in (Q, K, V, dO, W)]
-    out = _run_bwd(*g, True, torch.bfloat16)
+    out = _run_bwd(*g, True, torch.bfloat16, one_pass)
     for got, want in zip(out[:3], ref[:3]):
         assert max_abs(got, want) <= TOL_BF16
     assert rel_max(out[3], ref[3]) <= TOL_DW_REL
-    again = _run_bwd(*g, True, torch.bfloat16)
+    again = _run_bwd(*g, True, torch.bfloat16, one_pass)
     for a, b in zip(out, again):
         assert torch.equal(a, b)       # no atomics anywhere: bitwise repeatable
 
 
-def test_backward_noncausal_rectangular_mfma():
-    Q, K, V, dO, W = rand_case(1, 2, 70, 333, 128, 6, 11, torch.bfloat16, seed=10)
+@pytest.mark.parametrize("one_pass", [False, True])
+@pytest.mark.parametrize("Nq,Nk", [(70, 333), (333, 70), (200, 129)])
+def test_backward_noncausal_rectangular_mfma(Nq, Nk, one_pass):
+    Q, K, V, dO, W = rand_case(1, 2, Nq, Nk, 128, 6, 11, torch.bfloat16, seed=10)
     ref = oracle_bwd(Q, K, V, W, dO, False)
     g = [t.to(DEV) for t in (Q, K, V, dO, W)]
-    out = _run_bwd(*g, False, torch.bfloat16)
+    out = _run_bwd(*g, False, torch.bfloat16, one_pass)
     for got, want in zip(out[:3], ref[:3]):
         assert max_abs(got, want) <= TOL_BF16
     assert rel_max(out[3], ref[3]) <= TOL_DW_REL
+
+
+def test_one_pass_backward_workspace_garbage_and_tile_edges():
+    # The dS workspace is never initialised by the caller: poison the allocator's pool with
+    # NaNs first, then check sequence lengths around the 32-key / 64-row / 128-row tile edges.
+    poison = torch.full((64 << 20,), float("nan"), device=DEV)
+    del poison
+    for N in (63, 64, 65, 127, 129, 191, 193, 257, 449):
+        Q, K, V, dO, W = rand_case(1, 1, N, N, 64, 6, 11, torch.bfloat16, seed=N)
+        ref = oracle_bwd(Q, K, V, W, dO, True)
+        g = [t.to(DEV) for t in (Q, K, V, dO, W)]
+        out = _run_bwd(*g, True, torch.float32, one_pass=True)
+        for got, want in zip(out[:3], ref[:3]):
+            assert torch.isfinite(got).all() and max_abs(got, want) <= TOL_BF16, N
+        assert rel_max(out[3], ref[3]) <= TOL_DW_REL, N
 
 
 def test_module_autograd_matches_oracle_autograd():
@@ -228,6 +252,10 @@ def test_c3_full_size_fwd_bwd_against_fp32_kernels():
     assert max_abs(dK, dK_x) <= TOL_BF16
     assert max_abs(dV, dV_x) <= TOL_BF16
     assert rel_max(dW, dW_x) <= TOL_DW_REL
+    # the one-pass backward: same tiles, same arithmetic for dK / dV; dQ and dW in another order
+    dQ1, dK1, dV1, dW1 = ops.backward(Q, K, V, dO, D, LSE, W, *args, out_dtype=torch.bfloat16)
+    assert torch.equal(dK1, dK) and torch.equal(dV1, dV)
+    assert max_abs(dQ1, dQ_x) <= TOL_BF16 and rel_max(dW1, dW_x) <= TOL_DW_REL
     # dV is linear in dO, dQ/dK/dW are too: doubling dO doubles them (D doubles with it)
     dQ2, dW2 = ops.dq_backward(Q, K, V, (2 * dO.float()).to(torch.bfloat16), 2 * D, LSE, W, *args,
                                out_dtype=torch.float32)
@@ -255,3 +283,6 @@ def test_c5_long_context_one_head_forward_and_backward():
     dK_x, dV_x = ops.dkdv_backward(Q, K, V, dO, D_x, LSE_x, W, *args, exact=True)
     assert max_abs(dQ, dQ_x) <= TOL_BF16 and max_abs(dK, dK_x) <= TOL_BF16 and max_abs(dV, dV_x) <= TOL_BF16
     assert rel_max(dW, dW_x) <= TOL_DW_REL
+    dQ1, dK1, dV1, dW1 = ops.backward(Q, K, V, dO, D, LSE, W, *args, out_dtype=torch.bfloat16)
+    assert max_abs(dQ1, dQ_x) <= TOL_BF16 and max_abs(dK1, dK_x) <= TOL_BF16 and max_abs(dV1, dV_x) <= TOL_BF16
+    assert rel_max(dW1, dW_x) <= TOL_DW_REL
