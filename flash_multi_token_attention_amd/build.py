@@ -20,21 +20,22 @@ INCLUDE = os.path.join(ROOT, "include")
 LIB_NAME = "libconvattn_hip.so"
 LIB_PATH = os.path.join(PKG_DIR, LIB_NAME)
 
-# MFMA results in ordinary VGPRs where the register allocator can afford it (the 512-register
-# backward kernels otherwise copy every transient accumulator out of the accumulation file).
+# MFMA results in ordinary VGPRs (the 512-register dQ kernel otherwise copies every transient
+# accumulator out of the accumulation file).  Not for the dK/dV kernel: with its two tile loops
+# this compiler's MFMA rewrite pass crashes on it under this option.
 VGPR_FORM = ["-mllvm", "-amdgpu-mfma-vgpr-form"]
 
-# (source, object name, extra flags).  The dK/dV kernel is compiled in two halves: its 11-tap
-# instantiations (plain and fused) crash this compiler's MFMA rewrite pass under VGPR_FORM, so they go without it.
+# (source, object name, extra flags).  The dK/dV kernel is compiled as four objects (plain /
+# whole-backward variant x narrow / 11-tap windows) so that they build in parallel.
 UNITS = [
     ("api.hip", "api", []),
     ("generic_kernels.hip", "generic_kernels", []),
     ("reduce_kernels.hip", "reduce_kernels", []),
     ("fwd_mfma.hip", "fwd_mfma", []),
     ("bwd_dq_mfma.hip", "bwd_dq_mfma", VGPR_FORM),
-    ("bwd_dkdv_mfma.hip", "bwd_dkdv_mfma_narrow", ["-DCONVATTN_DKDV_UNIT=0", *VGPR_FORM]),
+    ("bwd_dkdv_mfma.hip", "bwd_dkdv_mfma_narrow", ["-DCONVATTN_DKDV_UNIT=0"]),
     ("bwd_dkdv_mfma.hip", "bwd_dkdv_mfma_wide", ["-DCONVATTN_DKDV_UNIT=1"]),
-    ("bwd_dkdv_mfma.hip", "bwd_fused_mfma_narrow", ["-DCONVATTN_DKDV_UNIT=2", *VGPR_FORM]),
+    ("bwd_dkdv_mfma.hip", "bwd_fused_mfma_narrow", ["-DCONVATTN_DKDV_UNIT=2"]),
     ("bwd_dkdv_mfma.hip", "bwd_fused_mfma_wide", ["-DCONVATTN_DKDV_UNIT=3"]),
     ("bwd_dq_gemm.hip", "bwd_dq_gemm", []),
     ("decode_stream.hip", "decode_stream", []),

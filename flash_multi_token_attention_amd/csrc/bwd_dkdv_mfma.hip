@@ -19,12 +19,15 @@
 //
 // FUSED instantiations do the whole backward in this one pass over the score tiles: they also
 //   * store dS (bf16, the operand of dK) to a workspace as [key tile of 32][row tile of 64]
-//     blocks of [32 keys][64 rows]; dQ = dS K is then a plain batched product (bwd_dq_gemm.hip);
+//     blocks of [32 keys][64 rows, permuted within groups of 32 so that a lane's 8 values are
+//     contiguous]; dQ = dS K is then a plain batched product (bwd_dq_gemm.hip);
 //   * accumulate dW[a][b] += sum over own rows i and own keys j' of
 //     S[i+a-pq][j'] * dC[i][j'-b+pk]: an MFMA contraction with M = a, N = b and (row, 8 keys)
 //     as the k index; the dC operand is read from LDS at a 2-byte granular offset.  Every
 //     (dC row, S key) pair belongs to exactly one (wave, tile); the waves' partials are summed
 //     in a fixed order and stored per workgroup.
+#include <type_traits>
+
 #include "mfma_common.hpp"
 
 #ifndef CONVATTN_DKDV_UNIT
@@ -147,11 +150,15 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
             const int c = min(tid + i * NW * 64, G_CH - 1), row = c / CPR, cc = c % CPR;
             gr[i] = load_row16_clamped<D>(dOb, r0 + row, p.Nq, cc * 8);
         }
-        ls = 0.f; dd = 0.f;
+        ls = 1e30f; dd = 0.f;  // rows past the end: exp2(C - LSE) = 0
         if (tid < C_ROWS && r0 + tid < p.Nq) { ls = lse_b[r0 + tid] * kLog2e; dd = dl_b[r0 + tid]; }
     };
     load_tile(r_begin);
-    for (int r0 = r_begin; r0 < p.Nq; r0 += BR) {
+    // One row tile.  EDGE tiles apply the causal / sequence-end masks; the others are far enough
+    // from the diagonal and from both ends of the key axis to need none (rows past the end of the
+    // sequence are dealt with by the staged values: zero Q / dO rows and a huge LSE give P = dC = 0).
+    auto tile = [&](const int r0, auto edge_tag) {
+        constexpr bool EDGE = decltype(edge_tag)::value;
         __syncthreads();
         if (r0 == 0 || r0 + C_ROWS > p.Nq) {  // rows outside the sequence count as zeros
 #pragma unroll
@@ -175,8 +182,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
         if (tid < C_ROWS) { lse_s[tid] = ls; dl_s[tid] = dd; }
         __syncthreads();
         if (r0 + BR < p.Nq) load_tile(r0 + BR);
-        if (causal && r0 + BR - 1 < c0 - 8) continue;  // none of the tile's own rows sees the wave's keys
-        const bool edge = c0 == 0 || (causal && c0 + 48 > r0 - 16) || (c0 + 40 > p.Nk) || (r0 + C_ROWS > p.Nq);
+        if (causal && r0 + BR - 1 < c0 - 8) return;  // none of the tile's own rows sees the wave's keys (only on masked tiles)
 
         // ---- S^T tile (raw) -> fp16 LDS; Q fragments one row block ahead ----
         {
@@ -206,7 +212,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                 const int qpos = r0 - 16 + rb * 16 + n;
 #pragma unroll
                 for (int kb = 0; kb < NSB; ++kb) {
-                    if (edge && causal) {
+                    if (EDGE && causal) {
                         const int key0 = c0 - 16 + kb * 16 + 4 * g;
 #pragma unroll
                         for (int r = 0; r < 4; ++r)
@@ -281,7 +287,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                     pr[r] = fast_exp2(c[kb][r] - lse4[r]);
                     dc[r] = pr[r] * (dp[kb][r] - dl4[r]);
                 }
-                if (edge) {
+                if constexpr (EDGE) {
                     const int key = c0 - 8 + kb * 16 + n;
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
@@ -361,7 +367,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                 SCHED_MFMA(2);
             }
         }
-        if (edge && causal) {
+        if (EDGE && causal) {
 #pragma unroll
             for (int ob = 0; ob < NRB; ++ob)
 #pragma unroll
@@ -383,16 +389,15 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                         sf[kp][m][4 + r] = (bf16_t)ds[2 * kp + 1][m][r];
                     }
             if constexpr (FUSED) {
-                // lane = key m*16+n; elements 0..3 / 4..7 are rows 4g.. of row blocks 2kp / 2kp+1
+                // lane = key m*16+n; elements 0..3 / 4..7 are rows 4g.. of row blocks 2kp / 2kp+1.
+                // They are stored as one 16-byte piece: within a key, row 32kp + 16h + 4g + r sits at
+                // position 32kp + 8g + 4h + r (ds_row_of_pos in mfma_common.hpp is the inverse).
                 bf16_t *blk = ds_wave + (size_t)(r0 / BR) * (WK * BR);
 #pragma unroll
                 for (int kp = 0; kp < NRB / 2; ++kp)
 #pragma unroll
-                    for (int m = 0; m < 2; ++m) {
-                        bf16_t *dst = blk + (m * 16 + n) * BR + kp * 32 + 4 * g;
-                        *reinterpret_cast<bf16x4 *>(dst) = __builtin_shufflevector(sf[kp][m], sf[kp][m], 0, 1, 2, 3);
-                        *reinterpret_cast<bf16x4 *>(dst + 16) = __builtin_shufflevector(sf[kp][m], sf[kp][m], 4, 5, 6, 7);
-                    }
+                    for (int m = 0; m < 2; ++m)
+                        *reinterpret_cast<bf16x8 *>(blk + (m * 16 + n) * BR + kp * 32 + 8 * g) = sf[kp][m];
             }
             constexpr int NST = (NRB / 2) * DB;
             bf16x8 qt[2];
@@ -427,29 +432,42 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
             const int boff = 8 + 8 * g - bcl + pk;
             const unsigned char *bbase = Cs + (boff & ~1) * 2;
             const unsigned int bsh = (boff & 1) * 16;
+            // The S operand of row i+1 is the one of row i moved down by one lane (lane n holds S row
+            // i + n - pq), so it is read from LDS once per RPL rows and shifted within the 16-lane
+            // rows in between; only lanes n < c_q matter, and (c_q - 1) + (RPL - 1) <= 15.
+            constexpr int RPL = CQT <= 6 ? 8 : 4;
+            static_assert(BR % RPL == 0 && (CQT - 1) + (RPL - 1) <= 15, "dW row groups");
 #pragma unroll 1
-            for (int i = 0; i < BR; i += 4) {
-                f16x8 af[4];
-                u32x4 bw[4];
-                unsigned int bx[4];
+            for (int i = 0; i < BR; i += RPL) {
+                u32x4 af = *reinterpret_cast<const u32x4 *>(abase + i * SST);
+                u32x4 bw[RPL];
+                unsigned int bx[RPL];
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    af[u] = *reinterpret_cast<const f16x8 *>(abase + (i + u) * SST);
+                for (int u = 0; u < RPL; ++u) {
                     bw[u] = reinterpret_cast<const U32x4A4 *>(bbase + (i + u) * CST)->v;
                     bx[u] = *reinterpret_cast<const unsigned int *>(bbase + (i + u) * CST + 16);
                 }
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
+                for (int u = 0; u < RPL; ++u) {
                     u32x4 sh;
                     sh[0] = __builtin_amdgcn_alignbit(bw[u][1], bw[u][0], bsh);
                     sh[1] = __builtin_amdgcn_alignbit(bw[u][2], bw[u][1], bsh);
                     sh[2] = __builtin_amdgcn_alignbit(bw[u][3], bw[u][2], bsh);
                     sh[3] = __builtin_amdgcn_alignbit(bx[u], bw[u][3], bsh);
-                    acc_w[u] = mfma_f16(af[u], __builtin_bit_cast(f16x8, sh), acc_w[u]);
+                    acc_w[u & 3] = mfma_f16(__builtin_bit_cast(f16x8, af), __builtin_bit_cast(f16x8, sh), acc_w[u & 3]);
+                    if (u + 1 < RPL) {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) af[r] = lane_from_next(af[r]);
+                    }
                 }
             }
         }
-    }
+    };
+    // keys before 0 or past the end in reach: every tile masks; else only the tiles near the diagonal
+    const bool always_edge = c0 == 0 || c0 + 40 > p.Nk;
+    int r0 = r_begin;
+    for (; r0 < p.Nq && (always_edge || (causal && r0 < c0 + 64)); r0 += BR) tile(r0, std::true_type{});
+    for (; r0 < p.Nq; r0 += BR) tile(r0, std::false_type{});
 
     // ---- stores: lane = key, 4 consecutive head-dim columns per block ----
 #pragma unroll
@@ -522,8 +540,8 @@ hipError_t launch_kv(const Problem &p, const void *q, const void *k, const void 
 }  // namespace
 
 // This file is built as four objects, CONVATTN_DKDV_UNIT = 2 * fused + wide: "wide" holds the
-// 11-tap-slot instantiations (they need different compiler options from the rest), "fused" the
-// whole-backward variants; the two narrow units also hold the entry points.
+// 11-tap-slot instantiations (the slowest to compile), "fused" the whole-backward variants; the
+// two narrow units also hold the entry points.
 template <int D, typename TO, bool FUSED>
 hipError_t dkdv_wide(const Problem &p, const void *q, const void *k, const void *v, const void *d_o,
                      const float *Dl, const float *lse, const float *w, void *dk, void *dv, void *ds_ws,

@@ -1,7 +1,7 @@
 // dQ = dS K on bf16 MFMA (gfx950), second step of the one-pass backward.
 //
 // dS comes from the fused dK/dV kernel as bf16 blocks [key tile of 32][row tile of 64] of
-// [32 keys][64 rows] (the softmax scale is already in it).  Workgroup = 4 waves = 128 query
+// [32 keys][64 rows in the producer's order, see ds_row_of_pos] (the softmax scale is already in it).  Workgroup = 4 waves = 128 query
 // rows of one (batch, head); wave w owns rows i0 + 32w .. +31 and all D columns.  Per step of
 // 64 keys the workgroup stages the K rows (row-major) and the four dS blocks (as [key][128
 // rows]) in LDS; both MFMA operands are LDS transpose reads with the keys as the k index:
@@ -115,10 +115,11 @@ __global__ __launch_bounds__(NW * 64) void dq_from_ds_kernel(Problem p, const bf
         }
     }
 
-    // lane = row, 4 consecutive head-dim columns per block
+    // lane = position ob*16+n of the wave's 32 rows in the dS blocks' row order;
+    // 4 consecutive head-dim columns per block
 #pragma unroll
     for (int ob = 0; ob < 2; ++ob) {
-        const int qpos = rw + ob * 16 + n;
+        const int qpos = rw + ds_row_of_pos(ob * 16 + n);
         if (qpos < p.Nq) {
             TO *orow = dQ + (bh * p.Nq + qpos) * D;
 #pragma unroll

@@ -45,6 +45,12 @@ __device__ __forceinline__ f32x4 mfma_f16(f16x8 a, f16x8 b, f32x4 c) {
 #define SCHED_DS_READ(n) __builtin_amdgcn_sched_group_barrier(0x100, (n), 0)
 #define SCHED_MFMA(n) __builtin_amdgcn_sched_group_barrier(0x008, (n), 0)
 
+// Lane n of every 16-lane row gets the value lane n+1 of that row holds (lane 15 gets 0):
+// DPP row_shl:1.
+__device__ __forceinline__ unsigned int lane_from_next(unsigned int v) {
+    return (unsigned int)__builtin_amdgcn_update_dpp(0, (int)v, 0x101, 0xf, 0xf, true);
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // Toeplitz fragment of query tap `a` for this lane: element e is
@@ -161,6 +167,11 @@ hipError_t mfma_bwd_dkdv(const Problem &p, int out_dt, const void *q, const void
 // per workgroup and dS as bf16 blocks [key tile of 32][row tile of 64][32 keys][64 rows];
 // mfma_dq_from_ds multiplies those blocks with K.
 constexpr int kKvKeysPerWg = 128, kDsKeys = 32, kDsRows = 64;
+// Inside a dS block the 64 rows of a key are stored in the order the producing lanes hold
+// them: position 32kp + 8g + 4h + r holds row 32kp + 16h + 4g + r.
+__host__ __device__ inline int ds_row_of_pos(int pos) {
+    return (pos & 32) | ((pos & 4) << 2) | ((pos >> 3 & 3) << 2) | (pos & 3);
+}
 inline int mfma_kv_tiles(const Problem &p) { return (p.Nk + 8 + kKvKeysPerWg - 1) / kKvKeysPerWg; }
 inline int mfma_ds_key_tiles(const Problem &p) { return mfma_kv_tiles(p) * (kKvKeysPerWg / kDsKeys); }
 inline int mfma_ds_row_tiles(const Problem &p) { return (p.Nq + kDsRows - 1) / kDsRows; }
