@@ -193,13 +193,13 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                     qf[buf][ks] = *reinterpret_cast<const bf16x8 *>(Qs + (rb * 16 + n) * RST + (ks * 32 + g * 8) * 2);
             };
             load_qf(0, 0);
-            SCHED_DS_READ(KS);
-#pragma unroll
-            for (int rb = 0; rb < S_ROWS / 16; ++rb) {
-                const int cur = rb & 1;
-                if (rb + 1 < S_ROWS / 16) {
+            SCHED_DS_READ_ID(KS, 10);
+            static_for<S_ROWS / 16>([&](auto rb_c) {
+                constexpr int rb = decltype(rb_c)::value;
+                constexpr int cur = rb & 1;
+                if constexpr (rb + 1 < S_ROWS / 16) {
                     load_qf(cur ^ 1, rb + 1);
-                    SCHED_DS_READ(KS);
+                    SCHED_DS_READ_ID(KS, 11 + rb);
                 }
                 f32x4 acc[NSB];
 #pragma unroll
@@ -208,7 +208,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                 for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
                     for (int kb = 0; kb < NSB; ++kb) acc[kb] = mfma_bf16(kf[kb][ks], qf[cur][ks], acc[kb]);
-                SCHED_MFMA(NSB * KS);
+                SCHED_MFMA_ID(NSB * KS, 10 + rb);
                 const int qpos = r0 - 16 + rb * 16 + n;
 #pragma unroll
                 for (int kb = 0; kb < NSB; ++kb) {
@@ -224,16 +224,18 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                         hv[r] = (_Float16)__builtin_amdgcn_fmed3f(acc[kb][r], -kF16Max, kF16Max);
                     *reinterpret_cast<f16x4 *>(Ss + (rb * 16 + n) * SST + (kb * 16 + 4 * g) * 2) = hv;
                 }
-            }
+            });
         }
         __builtin_amdgcn_wave_barrier();
 
         // ---- C, P, dP, dC ([query][key] orientation: lane = key, registers = 4 rows) ----
         f32x4 pkeep[NRB][2];
-#pragma unroll
-        for (int rb = 0; rb < C_ROWS / 16; ++rb) {
+        static_for<C_ROWS / 16>([&](auto rb_c) {
+            constexpr int rb = decltype(rb_c)::value;
+            constexpr int SID = 20 + rb;  // scheduling pipeline of this row block
             const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(lse_s + rb * 16 + 4 * g);
             const f32x4 dl4 = *reinterpret_cast<const f32x4 *>(dl_s + rb * 16 + 4 * g);
+            SCHED_DS_READ_ID(2, SID);
             f32x4 c[NCB], dp[NCB];
 #pragma unroll
             for (int kb = 0; kb < NCB; ++kb) {
@@ -249,16 +251,16 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                         sf[buf][kb] = *reinterpret_cast<const f16x8 *>(sbase + a * SST + kb * 32);
                 };
                 load_sf(0, 0);
-                SCHED_DS_READ(NCB);
+                SCHED_DS_READ_ID(NCB, SID);
 #pragma unroll
                 for (int a = 0; a < CQT; ++a) {
                     if (a + 1 < CQT) {
                         load_sf((a + 1) & 1, a + 1);
-                        SCHED_DS_READ(NCB);
+                        SCHED_DS_READ_ID(NCB, SID);
                     }
 #pragma unroll
                     for (int kb = 0; kb < NCB; ++kb) c[kb] = mfma_f16(sf[a & 1][kb], tf[a], c[kb]);
-                    SCHED_MFMA(NCB);
+                    SCHED_MFMA_ID(NCB, SID);
                 }
             }
             {
@@ -267,16 +269,16 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                     gf[buf] = *reinterpret_cast<const bf16x8 *>(Gs + (rb * 16 + n) * RST + (ks * 32 + g * 8) * 2);
                 };
                 load_gf(0, 0);
-                SCHED_DS_READ(1);
+                SCHED_DS_READ_ID(1, SID);
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
                     if (ks + 1 < KS) {
                         load_gf((ks + 1) & 1, ks + 1);
-                        SCHED_DS_READ(1);
+                        SCHED_DS_READ_ID(1, SID);
                     }
 #pragma unroll
                     for (int kb = 0; kb < NCB; ++kb) dp[kb] = mfma_bf16(gf[ks & 1], vf[kb][ks], dp[kb]);
-                    SCHED_MFMA(NCB);
+                    SCHED_MFMA_ID(NCB, SID);
                 }
             }
 #pragma unroll
@@ -299,9 +301,11 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                 for (int r = 0; r < 4; ++r)
                     *reinterpret_cast<_Float16 *>(Cs + (rb * 16 + 4 * g + r) * CST + (kb * 16 + n) * 2) =
                         (_Float16)__builtin_amdgcn_fmed3f(dc[r], -kF16Max, kF16Max);
-                if (rb < NRB && kb < 2) pkeep[rb][kb] = pr;
+                if constexpr (rb < NRB) {
+                    if (kb < 2) pkeep[rb][kb] = pr;
+                }
             }
-        }
+        });
         __builtin_amdgcn_wave_barrier();
 
         // ---- dV^T += dO^T P  (keys c0-8 .. c0+23); dO^T by transpose reads of the dO tile ----
@@ -325,17 +329,17 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                 gt[buf] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
             };
             load_gt(0, 0);
-            SCHED_DS_READ(2);
+            SCHED_DS_READ_ID(2, 30);
 #pragma unroll
             for (int st = 0; st < NST; ++st) {
                 if (st + 1 < NST) {
                     load_gt((st + 1) & 1, st + 1);
-                    SCHED_DS_READ(2);
+                    SCHED_DS_READ_ID(2, 30);
                 }
                 const int kp = st / DB, db = st % DB;
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb) acc_v[kb][db] = mfma_bf16(gt[st & 1], pf[kp][kb], acc_v[kb][db]);
-                SCHED_MFMA(2);
+                SCHED_MFMA_ID(2, 30);
             }
         }
 
@@ -355,16 +359,16 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                 cf[buf][1] = *reinterpret_cast<const f16x8 *>(base + 32);
             };
             load_cf(0, 0);
-            SCHED_DS_READ(2);
+            SCHED_DS_READ_ID(2, 31);
 #pragma unroll
             for (int st = 0; st < NST; ++st) {
                 if (st + 1 < NST) {
                     load_cf((st + 1) & 1, st + 1);
-                    SCHED_DS_READ(2);
+                    SCHED_DS_READ_ID(2, 31);
                 }
 #pragma unroll
                 for (int m = 0; m < 2; ++m) ds[st % NRB][m] = mfma_f16(cf[st & 1][m], tfl[st / NRB], ds[st % NRB][m]);
-                SCHED_MFMA(2);
+                SCHED_MFMA_ID(2, 31);
             }
         }
         if (EDGE && causal) {
@@ -408,17 +412,17 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                 qt[buf] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
             };
             load_qt(0, 0);
-            SCHED_DS_READ(2);
+            SCHED_DS_READ_ID(2, 32);
 #pragma unroll
             for (int st = 0; st < NST; ++st) {
                 if (st + 1 < NST) {
                     load_qt((st + 1) & 1, st + 1);
-                    SCHED_DS_READ(2);
+                    SCHED_DS_READ_ID(2, 32);
                 }
                 const int kp = st / DB, db = st % DB;
 #pragma unroll
                 for (int m = 0; m < 2; ++m) acc_k[m][db] = mfma_bf16(qt[st & 1], sf[kp][m], acc_k[m][db]);
-                SCHED_MFMA(2);
+                SCHED_MFMA_ID(2, 32);
             }
         }
 

@@ -13,6 +13,8 @@
 // pad_k <= 8.  Scores are staged in LDS as fp16 (11-bit significand; bf16's 8
 // bits would cost ~1e-2 in the softmax argument).
 #pragma once
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace convattn {
@@ -44,6 +46,22 @@ __device__ __forceinline__ f32x4 mfma_f16(f16x8 a, f16x8 b, f32x4 c) {
 // of stage s" so that fragment reads stay one stage ahead instead of sinking next to their use.
 #define SCHED_DS_READ(n) __builtin_amdgcn_sched_group_barrier(0x100, (n), 0)
 #define SCHED_MFMA(n) __builtin_amdgcn_sched_group_barrier(0x008, (n), 0)
+#define SCHED_VALU(n) __builtin_amdgcn_sched_group_barrier(0x002, (n), 0)
+// The same with an explicit pipeline id: groups are only ordered against groups of their own id,
+// and the backend places long pipelines badly, so every row block of a phase gets its own.
+#define SCHED_DS_READ_ID(n, id) __builtin_amdgcn_sched_group_barrier(0x100, (n), (id))
+#define SCHED_MFMA_ID(n, id) __builtin_amdgcn_sched_group_barrier(0x008, (n), (id))
+#define SCHED_VALU_ID(n, id) __builtin_amdgcn_sched_group_barrier(0x002, (n), (id))
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>): a loop whose index is a
+// constant expression in the body (the scheduling-group builtins need one).
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (N > 0) {
+        static_for<N - 1>(f);
+        f(std::integral_constant<int, N - 1>{});
+    }
+}
 
 // Lane n of every 16-lane row gets the value lane n+1 of that row holds (lane 15 gets 0):
 // DPP row_shl:1.
