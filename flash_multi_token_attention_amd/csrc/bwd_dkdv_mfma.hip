@@ -8,8 +8,11 @@
 // the queries in 64-row tiles that the workgroup stages row-major in LDS (Q
 // and dO; their transposes for the dK / dV products come from LDS transpose
 // reads).  Per tile, with r0 its first row:
-//   S^T  rows r0-16 .. r0+79, keys c0-16 .. c0+47    raw K Q^T, pre-masked, fp16 -> LDS
-//   C    rows r0 .. r0+79, keys c0-8 .. c0+39        Toeplitz MFMAs, here oriented
+//   S^T  rows r0-8 .. r0+71 (up to 6 taps; r0-16 .. r0+79 beyond), keys c0-16 .. c0+47:
+//        raw K Q^T, pre-masked, fp16 -> LDS
+//   C    rows r0 .. r0+79 (only rows up to r0+63+c_q-1 are used; with the short S tile the last
+//        ones are computed from whatever follows it in LDS and never read), keys c0-8 .. c0+39:
+//        Toeplitz MFMAs, here oriented
 //        [query][key] so that a lane holds one key and 4 query rows: that is the
 //        operand layout the dV and dK products need, no transposition in between
 //   P = exp2(C - LSE), dP = dO V^T, dC = P (dP - D): fp16 -> LDS (2-byte stores)
@@ -41,7 +44,9 @@ constexpr int NW = 4;
 constexpr int WK = 32;                 // own keys per wave
 constexpr int BKW = NW * WK;           // 128 keys per workgroup
 constexpr int BR = 64;                 // query rows per tile
-constexpr int S_ROWS = BR + 32;        // 96: 16 above, 16 below
+// Score rows staged above / below a tile's own rows: the window reaches c_q - 1 rows up (and dC
+// the same number of rows down), so 8 do for up to 6 taps; wider windows take 16.
+template <int CQT> constexpr int kHaloRows = CQT <= 6 ? 8 : 16;
 constexpr int S_COLS = WK + 32;        // 64
 constexpr int C_ROWS = BR + 16;        // 80
 constexpr int C_COLS = WK + 16;        // 48
@@ -52,7 +57,8 @@ constexpr int NCB = C_COLS / 16;       // 3 key blocks of C / dP / dC
 constexpr int NRB = BR / 16;           // 4 own row blocks per tile
 static_assert(BKW == kKvKeysPerWg && WK == kDsKeys && BR == kDsRows, "dS workspace layout");
 
-template <int D> struct KvLds {
+template <int D, int CQT> struct KvLds {
+    static constexpr int S_ROWS = BR + 2 * kHaloRows<CQT>;
     static constexpr int RST = D * 2 + 16;
     static constexpr int q_bytes = S_ROWS * RST;
     static constexpr int g_bytes = C_ROWS * RST;
@@ -67,8 +73,8 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
     const bf16_t *__restrict__ V, const bf16_t *__restrict__ dO, const float *__restrict__ Dl,
     const float *__restrict__ LSE, const float *__restrict__ W, TO *__restrict__ dK,
     TO *__restrict__ dV, bf16_t *__restrict__ dS_ws, float *__restrict__ dW_part) {
-    using Lds = KvLds<D>;
-    constexpr int RST = Lds::RST;
+    using Lds = KvLds<D, CQT>;
+    constexpr int RST = Lds::RST, S_ROWS = Lds::S_ROWS, HT = kHaloRows<CQT>;
     constexpr int KS = D / 32, DB = D / 16, CPR = D / 8;
     constexpr int Q_CH = S_ROWS * CPR, G_CH = C_ROWS * CPR;
     constexpr int Q_LD = (Q_CH + NW * 64 - 1) / (NW * 64);
@@ -143,7 +149,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
 #pragma unroll
         for (int i = 0; i < Q_LD; ++i) {
             const int c = min(tid + i * NW * 64, Q_CH - 1), row = c / CPR, cc = c % CPR;
-            qr[i] = load_row16_clamped<D>(Qb, r0 - 16 + row, p.Nq, cc * 8);
+            qr[i] = load_row16_clamped<D>(Qb, r0 - HT + row, p.Nq, cc * 8);
         }
 #pragma unroll
         for (int i = 0; i < G_LD; ++i) {
@@ -163,7 +169,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
         if (r0 == 0 || r0 + C_ROWS > p.Nq) {  // rows outside the sequence count as zeros
 #pragma unroll
             for (int i = 0; i < Q_LD; ++i) {
-                const int row = r0 - 16 + (tid + i * NW * 64) / CPR;
+                const int row = r0 - HT + (tid + i * NW * 64) / CPR;
                 qr[i] = zero_unless(row >= 0 && row < p.Nq, qr[i]);
             }
 #pragma unroll
@@ -209,7 +215,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
 #pragma unroll
                     for (int kb = 0; kb < NSB; ++kb) acc[kb] = mfma_bf16(kf[kb][ks], qf[cur][ks], acc[kb]);
                 SCHED_MFMA_ID(NSB * KS, 10 + rb);
-                const int qpos = r0 - 16 + rb * 16 + n;
+                const int qpos = r0 - HT + rb * 16 + n;
 #pragma unroll
                 for (int kb = 0; kb < NSB; ++kb) {
                     if (EDGE && causal) {
@@ -243,7 +249,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                 dp[kb] = (f32x4){0.f, 0.f, 0.f, 0.f};
             }
             {
-                const unsigned char *sbase = Ss + (16 + rb * 16 + n - (CQT - 1)) * SST + (8 * g) * 2;
+                const unsigned char *sbase = Ss + (HT + rb * 16 + n - (CQT - 1)) * SST + (8 * g) * 2;
                 f16x8 sf[2][NCB];
                 auto load_sf = [&](int buf, int a) {
 #pragma unroll
@@ -380,7 +386,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                     for (int r = 0; r < 4; ++r)
                         if (c0 + m * 16 + n > r0 + ob * 16 + 4 * g + r) ds[ob][m][r] = 0.f;
         }
-        // ---- dK^T += Q^T dS; Q^T by transpose reads (own rows start at Q-tile row 16) ----
+        // ---- dK^T += Q^T dS; Q^T by transpose reads (own rows start at Q-tile row HT) ----
         {
             bf16x8 sf[NRB / 2][2];
 #pragma unroll
@@ -407,8 +413,8 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
             bf16x8 qt[2];
             auto load_qt = [&](int buf, int st) {
                 const int kp = st / DB, db = st % DB;
-                bf16x4 lo = lds_read_tr4x16(Qs, RST, 16 + kp * 32 + 4 * g, db * 16, n);
-                bf16x4 hi = lds_read_tr4x16(Qs, RST, 32 + kp * 32 + 4 * g, db * 16, n);
+                bf16x4 lo = lds_read_tr4x16(Qs, RST, HT + kp * 32 + 4 * g, db * 16, n);
+                bf16x4 hi = lds_read_tr4x16(Qs, RST, HT + 16 + kp * 32 + 4 * g, db * 16, n);
                 qt[buf] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
             };
             load_qt(0, 0);
@@ -428,9 +434,9 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
 
         // ---- dW: rows m = tap a, columns n = tap b, contraction over (own row, 8 own keys) ----
         if constexpr (FUSED) {
-            // A: S[i + a - pq][c0 + 8g ..]        (S-tile row 16 + i + a - pq, column 16 + 8g)
+            // A: S[i + a - pq][c0 + 8g ..]        (S-tile row HT + i + a - pq, column 16 + 8g)
             // B: dC[i][c0 + 8g - b + pk ..]       (dC-tile column 8 + 8g - b + pk)
-            const unsigned char *abase = Ss + (16 + n - pq) * SST + (16 + 8 * g) * 2;
+            const unsigned char *abase = Ss + (HT + n - pq) * SST + (16 + 8 * g) * 2;
             // LDS reads at odd 2-byte offsets are slow: read 5 dwords from the even
             // element below and funnel-shift by 0 or 16 bits per lane instead.
             const int boff = 8 + 8 * g - bcl + pk;
@@ -530,7 +536,7 @@ hipError_t launch_kv(const Problem &p, const void *q, const void *k, const void 
                      const float *Dl, const float *lse, const float *w, void *dk, void *dv, void *ds_ws,
                      float *dw_part, hipStream_t s) {
     auto kern = bwd_dkdv_mfma_kernel<D, CQT, TO, FUSED>;
-    constexpr int lds = KvLds<D>::total;
+    constexpr int lds = KvLds<D, CQT>::total;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return e;
