@@ -8,16 +8,17 @@
 // the queries in 64-row tiles that the workgroup stages row-major in LDS (Q
 // and dO; their transposes for the dK / dV products come from LDS transpose
 // reads).  Per tile, with r0 its first row:
-//   S^T  rows r0-8 .. r0+71 (up to 6 taps; r0-16 .. r0+79 beyond), keys c0-16 .. c0+47:
-//        raw K Q^T, pre-masked, fp16 -> LDS
-//   C    rows r0 .. r0+79 (only rows up to r0+63+c_q-1 are used; with the short S tile the last
-//        ones are computed from whatever follows it in LDS and never read), keys c0-8 .. c0+39:
-//        Toeplitz MFMAs, here oriented
+//   S^T  rows r0-16 .. r0+63, keys c0-16 .. c0+47    raw K Q^T, pre-masked, fp16 -> LDS
+//   C    rows r0 .. r0+63, keys c0-8 .. c0+39        Toeplitz MFMAs, here oriented
 //        [query][key] so that a lane holds one key and 4 query rows: that is the
 //        operand layout the dV and dK products need, no transposition in between
-//   P = exp2(C - LSE), dP = dO V^T, dC = P (dP - D): fp16 -> LDS (2-byte stores)
+//   P = exp2(C - LSE), dP = dO V^T, dC = P (dP - D): fp16 -> LDS (2-byte stores), below the
+//        16 dC rows kept from the previous tile
 //   dV^T += dO^T P        (rows r0 .. r0+63, keys c0-8 .. c0+23)
-//   dS   rows r0 .. r0+63, keys c0 .. c0+31: flipped-band MFMAs over dC, causal zero
+//   dS   rows r0-16 .. r0+47, keys c0 .. c0+31: flipped-band MFMAs over dC, causal zero.  dS of
+//        a row needs the dC rows up to c_q-1 below it, so this product trails the tile by 16
+//        rows instead of recomputing C / dP / dC for a 16-row halo below every tile; one short
+//        tile after the last row finishes the last 16 rows
 //   dK^T += Q^T dS        (the flipped bands carry the softmax scale)
 //
 // FUSED instantiations do the whole backward in this one pass over the score tiles: they also
@@ -44,11 +45,10 @@ constexpr int NW = 4;
 constexpr int WK = 32;                 // own keys per wave
 constexpr int BKW = NW * WK;           // 128 keys per workgroup
 constexpr int BR = 64;                 // query rows per tile
-// Score rows staged above / below a tile's own rows: the window reaches c_q - 1 rows up (and dC
-// the same number of rows down), so 8 do for up to 6 taps; wider windows take 16.
-template <int CQT> constexpr int kHaloRows = CQT <= 6 ? 8 : 16;
+constexpr int HT = 16;                 // rows staged above a tile's own rows (>= c_q - 1)
+constexpr int S_ROWS = BR + HT;        // 80 score rows: r0-16 .. r0+63
 constexpr int S_COLS = WK + 32;        // 64
-constexpr int C_ROWS = BR + 16;        // 80
+constexpr int C_ROWS = BR + HT;        // 80 dC rows: 16 carried over from the previous tile + 64 new
 constexpr int C_COLS = WK + 16;        // 48
 constexpr int SST = (S_COLS + 8) * 2;  // 144
 constexpr int CST = (C_COLS + 8) * 2;  // 112
@@ -58,11 +58,10 @@ constexpr int NRB = BR / 16;           // 4 own row blocks per tile
 static_assert(BKW == kKvKeysPerWg && WK == kDsKeys && BR == kDsRows, "dS workspace layout");
 
 template <int D, int CQT> struct KvLds {
-    static constexpr int S_ROWS = BR + 2 * kHaloRows<CQT>;
     static constexpr int RST = D * 2 + 16;
     static constexpr int q_bytes = S_ROWS * RST;
-    static constexpr int g_bytes = C_ROWS * RST;
-    static constexpr int stat_bytes = 2 * C_ROWS * 4;
+    static constexpr int g_bytes = BR * RST;
+    static constexpr int stat_bytes = 2 * BR * 4;
     static constexpr int wave_bytes = S_ROWS * SST + C_ROWS * CST;
     static constexpr int total = q_bytes + g_bytes + stat_bytes + NW * wave_bytes;
 };
@@ -74,16 +73,16 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
     const float *__restrict__ LSE, const float *__restrict__ W, TO *__restrict__ dK,
     TO *__restrict__ dV, bf16_t *__restrict__ dS_ws, float *__restrict__ dW_part) {
     using Lds = KvLds<D, CQT>;
-    constexpr int RST = Lds::RST, S_ROWS = Lds::S_ROWS, HT = kHaloRows<CQT>;
+    constexpr int RST = Lds::RST;
     constexpr int KS = D / 32, DB = D / 16, CPR = D / 8;
-    constexpr int Q_CH = S_ROWS * CPR, G_CH = C_ROWS * CPR;
+    constexpr int Q_CH = S_ROWS * CPR, G_CH = BR * CPR;
     constexpr int Q_LD = (Q_CH + NW * 64 - 1) / (NW * 64);
     constexpr int G_LD = (G_CH + NW * 64 - 1) / (NW * 64);
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     unsigned char *Qs = smem;
     unsigned char *Gs = Qs + Lds::q_bytes;
     float *lse_s = reinterpret_cast<float *>(Gs + Lds::g_bytes);
-    float *dl_s = lse_s + C_ROWS;
+    float *dl_s = lse_s + BR;
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
@@ -142,6 +141,11 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
 
     // Causal: rows before the first key this workgroup touches (k0 - 8) see none of its keys.
     const int r_begin = causal ? (max(0, k0 - 8) / BR) * BR : 0;
+    // dS / dK of a row need the dC rows below it, so they trail the tiles by 16 rows: one more
+    // (short) tile when the last 16 rows of the sequence are not covered otherwise.
+    const int r_end = p.Nq + HT;
+    for (int c = lane; c < HT * (CST / 16); c += 64)  // no dC before the first tile
+        *reinterpret_cast<u32x4 *>(Cs + (c / (CST / 16)) * CST + (c % (CST / 16)) * 16) = (u32x4){0u, 0u, 0u, 0u};
     // Staging registers: this thread's 16-byte chunks of the next Q / dO tile and its LSE / D entry.
     u32x4 qr[Q_LD], gr[G_LD];
     float ls = 0.f, dd = 0.f;
@@ -157,7 +161,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
             gr[i] = load_row16_clamped<D>(dOb, r0 + row, p.Nq, cc * 8);
         }
         ls = 1e30f; dd = 0.f;  // rows past the end: exp2(C - LSE) = 0
-        if (tid < C_ROWS && r0 + tid < p.Nq) { ls = lse_b[r0 + tid] * kLog2e; dd = dl_b[r0 + tid]; }
+        if (tid < BR && r0 + tid < p.Nq) { ls = lse_b[r0 + tid] * kLog2e; dd = dl_b[r0 + tid]; }
     };
     load_tile(r_begin);
     // One row tile.  EDGE tiles apply the causal / sequence-end masks; the others are far enough
@@ -166,7 +170,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
     auto tile = [&](const int r0, auto edge_tag) {
         constexpr bool EDGE = decltype(edge_tag)::value;
         __syncthreads();
-        if (r0 == 0 || r0 + C_ROWS > p.Nq) {  // rows outside the sequence count as zeros
+        if (r0 == 0 || r0 + BR > p.Nq) {  // rows outside the sequence count as zeros
 #pragma unroll
             for (int i = 0; i < Q_LD; ++i) {
                 const int row = r0 - HT + (tid + i * NW * 64) / CPR;
@@ -185,12 +189,21 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
             const int c = tid + i * NW * 64, row = c / CPR, cc = c % CPR;
             if (c < G_CH) *reinterpret_cast<u32x4 *>(Gs + row * RST + cc * 16) = gr[i];
         }
-        if (tid < C_ROWS) { lse_s[tid] = ls; dl_s[tid] = dd; }
+        if (tid < BR) { lse_s[tid] = ls; dl_s[tid] = dd; }
         __syncthreads();
-        if (r0 + BR < p.Nq) load_tile(r0 + BR);
-        if (causal && r0 + BR - 1 < c0 - 8) return;  // none of the tile's own rows sees the wave's keys (only on masked tiles)
+        if (r0 + BR < r_end) load_tile(r0 + BR);
+        if (causal && r0 + BR - 1 < c0 - 8) return;  // none of the tile's rows sees the wave's keys (only on masked tiles)
+        // Past the last row only the dS / dK work of the 16 carried rows is left.
+        const bool tail = EDGE && r0 >= p.Nq;
+        f32x4 pkeep[NRB][2];
+        if (tail) {
+            // the tile has no dC rows of its own: zeros below the carried ones
+            for (int c = lane; c < 16 * (CST / 16); c += 64)
+                *reinterpret_cast<u32x4 *>(Cs + (HT + c / (CST / 16)) * CST + (c % (CST / 16)) * 16) = (u32x4){0u, 0u, 0u, 0u};
+        } else {
 
-        // ---- S^T tile (raw) -> fp16 LDS; Q fragments one row block ahead ----
+        // ---- S^T tile (raw) -> fp16 LDS; Q fragments one row block ahead.  (Taking the first 16 rows
+        // over from the previous tile instead of recomputing them was measured: no gain.) ----
         {
             bf16x8 qf[2][KS];
             auto load_qf = [&](int buf, int rb) {
@@ -235,8 +248,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
         __builtin_amdgcn_wave_barrier();
 
         // ---- C, P, dP, dC ([query][key] orientation: lane = key, registers = 4 rows) ----
-        f32x4 pkeep[NRB][2];
-        static_for<C_ROWS / 16>([&](auto rb_c) {
+        static_for<NRB>([&](auto rb_c) {
             constexpr int rb = decltype(rb_c)::value;
             constexpr int SID = 20 + rb;  // scheduling pipeline of this row block
             const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(lse_s + rb * 16 + 4 * g);
@@ -305,11 +317,9 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                 }
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
-                    *reinterpret_cast<_Float16 *>(Cs + (rb * 16 + 4 * g + r) * CST + (kb * 16 + n) * 2) =
+                    *reinterpret_cast<_Float16 *>(Cs + (HT + rb * 16 + 4 * g + r) * CST + (kb * 16 + n) * 2) =
                         (_Float16)__builtin_amdgcn_fmed3f(dc[r], -kF16Max, kF16Max);
-                if constexpr (rb < NRB) {
-                    if (kb < 2) pkeep[rb][kb] = pr;
-                }
+                if (kb < 2) pkeep[rb][kb] = pr;
             }
         });
         __builtin_amdgcn_wave_barrier();
@@ -348,8 +358,12 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                 SCHED_MFMA_ID(2, 30);
             }
         }
+        }  // !tail
+        __builtin_amdgcn_wave_barrier();
 
-        // ---- dS (keys c0 .. c0+31): 4 chains over the taps ----
+        // ---- dS, rows r0-16 .. r0+47 (keys c0 .. c0+31): 4 chains over the taps.  The rows are the
+        // ones whose window (c_q - 1 rows down) is complete with this tile's dC; the dC tile starts
+        // at row r0-16 with the 16 rows carried over from the previous tile. ----
         f32x4 ds[NRB][2];
 #pragma unroll
         for (int ob = 0; ob < NRB; ++ob)
@@ -384,9 +398,9 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                 for (int m = 0; m < 2; ++m)
 #pragma unroll
                     for (int r = 0; r < 4; ++r)
-                        if (c0 + m * 16 + n > r0 + ob * 16 + 4 * g + r) ds[ob][m][r] = 0.f;
+                        if (c0 + m * 16 + n > r0 - HT + ob * 16 + 4 * g + r) ds[ob][m][r] = 0.f;
         }
-        // ---- dK^T += Q^T dS; Q^T by transpose reads (own rows start at Q-tile row HT) ----
+        // ---- dK^T += Q^T dS; Q^T by transpose reads (the Q tile starts at row r0-16 as well) ----
         {
             bf16x8 sf[NRB / 2][2];
 #pragma unroll
@@ -399,22 +413,29 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                         sf[kp][m][4 + r] = (bf16_t)ds[2 * kp + 1][m][r];
                     }
             if constexpr (FUSED) {
-                // lane = key m*16+n; elements 0..3 / 4..7 are rows 4g.. of row blocks 2kp / 2kp+1.
-                // They are stored as one 16-byte piece: within a key, row 32kp + 16h + 4g + r sits at
-                // position 32kp + 8g + 4h + r (ds_row_of_pos in mfma_common.hpp is the inverse).
+                // lane = key m*16+n holds rows 4g.. of each 16-row block.  Within a key the workspace
+                // keeps row 32k + 16h + 4g + r at position 32k + 8g + 4h + r (ds_row_of_pos in
+                // mfma_common.hpp is the inverse), so the blocks at rows r0 .. r0+31 make one 16-byte
+                // piece; the block at r0-16 completes the previous row tile, the one at r0+32 starts
+                // the second half of this one.
                 bf16_t *blk = ds_wave + (size_t)(r0 / BR) * (WK * BR);
 #pragma unroll
-                for (int kp = 0; kp < NRB / 2; ++kp)
-#pragma unroll
-                    for (int m = 0; m < 2; ++m)
-                        *reinterpret_cast<bf16x8 *>(blk + (m * 16 + n) * BR + kp * 32 + 8 * g) = sf[kp][m];
+                for (int m = 0; m < 2; ++m) {
+                    bf16_t *key = blk + (m * 16 + n) * BR + 8 * g;
+                    if (!EDGE || r0 > 0)  // (unmasked tiles never start at row 0)
+                        *reinterpret_cast<bf16x4 *>(key - WK * BR + 32 + 4) = __builtin_shufflevector(sf[0][m], sf[0][m], 0, 1, 2, 3);
+                    if (!tail) {
+                        *reinterpret_cast<bf16x8 *>(key) = __builtin_shufflevector(sf[0][m], sf[1][m], 4, 5, 6, 7, 8, 9, 10, 11);
+                        *reinterpret_cast<bf16x4 *>(key + 32) = __builtin_shufflevector(sf[1][m], sf[1][m], 4, 5, 6, 7);
+                    }
+                }
             }
             constexpr int NST = (NRB / 2) * DB;
             bf16x8 qt[2];
             auto load_qt = [&](int buf, int st) {
                 const int kp = st / DB, db = st % DB;
-                bf16x4 lo = lds_read_tr4x16(Qs, RST, HT + kp * 32 + 4 * g, db * 16, n);
-                bf16x4 hi = lds_read_tr4x16(Qs, RST, HT + 16 + kp * 32 + 4 * g, db * 16, n);
+                bf16x4 lo = lds_read_tr4x16(Qs, RST, kp * 32 + 4 * g, db * 16, n);
+                bf16x4 hi = lds_read_tr4x16(Qs, RST, 16 + kp * 32 + 4 * g, db * 16, n);
                 qt[buf] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
             };
             load_qt(0, 0);
@@ -433,14 +454,14 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
         }
 
         // ---- dW: rows m = tap a, columns n = tap b, contraction over (own row, 8 own keys) ----
-        if constexpr (FUSED) {
+        if (FUSED && !tail) {
             // A: S[i + a - pq][c0 + 8g ..]        (S-tile row HT + i + a - pq, column 16 + 8g)
-            // B: dC[i][c0 + 8g - b + pk ..]       (dC-tile column 8 + 8g - b + pk)
+            // B: dC[i][c0 + 8g - b + pk ..]       (dC-tile row HT + i, column 8 + 8g - b + pk)
             const unsigned char *abase = Ss + (HT + n - pq) * SST + (16 + 8 * g) * 2;
             // LDS reads at odd 2-byte offsets are slow: read 5 dwords from the even
             // element below and funnel-shift by 0 or 16 bits per lane instead.
             const int boff = 8 + 8 * g - bcl + pk;
-            const unsigned char *bbase = Cs + (boff & ~1) * 2;
+            const unsigned char *bbase = Cs + HT * CST + (boff & ~1) * 2;
             const unsigned int bsh = (boff & 1) * 16;
             // The S operand of row i+1 is the one of row i moved down by one lane (lane n holds S row
             // i + n - pq), so it is read from LDS once per RPL rows and shifted within the 16-lane
@@ -472,12 +493,21 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                 }
             }
         }
+        // ---- the last 16 dC rows become the first 16 of the next tile ----
+        __builtin_amdgcn_wave_barrier();
+        for (int c = lane; c < HT * (CST / 16); c += 64) {
+            const int off = (c / (CST / 16)) * CST + (c % (CST / 16)) * 16;
+            *reinterpret_cast<u32x4 *>(Cs + off) = *reinterpret_cast<const u32x4 *>(Cs + BR * CST + off);
+        }
+        __builtin_amdgcn_wave_barrier();
     };
     // keys before 0 or past the end in reach: every tile masks; else only the tiles near the diagonal
+    // and the last, partial ones
     const bool always_edge = c0 == 0 || c0 + 40 > p.Nk;
     int r0 = r_begin;
-    for (; r0 < p.Nq && (always_edge || (causal && r0 < c0 + 64)); r0 += BR) tile(r0, std::true_type{});
-    for (; r0 < p.Nq; r0 += BR) tile(r0, std::false_type{});
+    for (; r0 < r_end && (always_edge || r0 == 0 || (causal && r0 < c0 + 64)); r0 += BR) tile(r0, std::true_type{});
+    for (; r0 + BR <= p.Nq; r0 += BR) tile(r0, std::false_type{});
+    for (; r0 < r_end; r0 += BR) tile(r0, std::true_type{});
 
     // ---- stores: lane = key, 4 consecutive head-dim columns per block ----
 #pragma unroll
