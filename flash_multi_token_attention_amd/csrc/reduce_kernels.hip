@@ -6,20 +6,45 @@
 namespace convattn {
 namespace {
 
-// One wave per query row: D = <dO, O>, LSE = M + log L.
+// D = <dO, O>, LSE = M + log L.  16 lanes per query row, 8 elements (16 or 32 bytes) per lane:
+// a wave reads 4 rows at a time with full-width loads; d is a multiple of 8 and at most 128.
+template <typename T>
+__device__ __forceinline__ void load8(const T *__restrict__ ptr, float (&v)[8]) {
+    if constexpr (sizeof(T) == 2) {
+        const uint4 raw = *reinterpret_cast<const uint4 *>(ptr);
+        const unsigned int w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = __uint_as_float(w[i] << 16);
+            v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+        }
+    } else {
+        const float4 a = *reinterpret_cast<const float4 *>(ptr);
+        const float4 b = *reinterpret_cast<const float4 *>(ptr + 4);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+        v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    }
+}
+
 template <typename TI, typename TO>
 __global__ __launch_bounds__(256) void preprocess_kernel(size_t rows, int d, const TO *__restrict__ O,
                                                          const TI *__restrict__ dO,
                                                          const float *__restrict__ M,
                                                          const float *__restrict__ L,
                                                          float *__restrict__ D, float *__restrict__ LSE) {
-    const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int lane = threadIdx.x & 63;
-    if (row >= rows) return;
+    const size_t row = (size_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+    const int sub = threadIdx.x & 15;
     float s = 0.f;
-    for (int c = lane; c < d; c += kWave) s = fmaf(to_f32(O[row * d + c]), to_f32(dO[row * d + c]), s);
-    s = wave_sum(s);
-    if (lane == 0) {
+    if (row < rows && sub * 8 < d) {
+        float o[8], g[8];
+        load8(O + row * d + sub * 8, o);
+        load8(dO + row * d + sub * 8, g);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) s = fmaf(o[i], g[i], s);
+    }
+#pragma unroll
+    for (int m = 8; m >= 1; m >>= 1) s += __shfl_xor(s, m, 16);
+    if (row < rows && sub == 0) {
         D[row] = s;
         LSE[row] = M[row] + __logf(L[row]);
     }
@@ -66,7 +91,7 @@ __global__ void combine_kernel(int n_splits, int d, const float *__restrict__ O_
 hipError_t bwd_preprocess(const Problem &p, int in_dt, int out_dt, const void *o, const void *d_o,
                           const float *m, const float *l, float *D, float *lse, hipStream_t s) {
     const size_t rows = (size_t)p.B * p.H * p.Nq;
-    const unsigned grid = (unsigned)((rows + 3) / 4);
+    const unsigned grid = (unsigned)((rows + 15) / 16);
 #define CALL(TI, TO) \
     preprocess_kernel<TI, TO><<<grid, 256, 0, s>>>(rows, p.d, (const TO *)o, (const TI *)d_o, m, l, D, lse)
     if (in_dt == CONVATTN_BF16 && out_dt == CONVATTN_BF16) CALL(bf16_t, bf16_t);
