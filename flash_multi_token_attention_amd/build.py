@@ -25,8 +25,8 @@ LIB_PATH = os.path.join(PKG_DIR, LIB_NAME)
 # this compiler's MFMA rewrite pass crashes on it under this option.
 VGPR_FORM = ["-mllvm", "-amdgpu-mfma-vgpr-form"]
 
-# (source, object name, extra flags).  The dK/dV kernel is compiled as four objects (plain /
-# whole-backward variant x narrow / 11-tap windows) so that they build in parallel.
+# (source, object name, extra flags).  The dK/dV kernel is compiled as two objects (narrow /
+# 11-tap windows) so that they build in parallel.
 UNITS = [
     ("api.hip", "api", []),
     ("generic_kernels.hip", "generic_kernels", []),
@@ -35,8 +35,7 @@ UNITS = [
     ("bwd_dq_mfma.hip", "bwd_dq_mfma", VGPR_FORM),
     ("bwd_dkdv_mfma.hip", "bwd_dkdv_mfma_narrow", ["-DCONVATTN_DKDV_UNIT=0"]),
     ("bwd_dkdv_mfma.hip", "bwd_dkdv_mfma_wide", ["-DCONVATTN_DKDV_UNIT=1"]),
-    ("bwd_dkdv_mfma.hip", "bwd_fused_mfma_narrow", ["-DCONVATTN_DKDV_UNIT=2"]),
-    ("bwd_dkdv_mfma.hip", "bwd_fused_mfma_wide", ["-DCONVATTN_DKDV_UNIT=3"]),
+    ("bwd_ws_mfma.hip", "bwd_ws_mfma", []),
     ("bwd_dq_gemm.hip", "bwd_dq_gemm", []),
     ("decode_stream.hip", "decode_stream", []),
 ]

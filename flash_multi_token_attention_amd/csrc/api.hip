@@ -189,7 +189,7 @@ int convattn_bwd_fused_dkdv(const convattn_desc *desc, const void *q, const void
         return (int)generic_bwd_dkdv(p, desc->in_dtype, desc->out_dtype, q, k, v, d_o, D, lse, w, dk, dv, s);
     unsigned char *ws = static_cast<unsigned char *>(workspace);
     float *part = reinterpret_cast<float *>(ws + align256(mfma_ds_bytes(p)));
-    return (int)mfma_bwd_fused(p, desc->out_dtype, q, k, v, d_o, D, lse, w, dk, dv, ws, part, s);
+    return (int)mfma_bwd_fused_ws(p, desc->out_dtype, q, k, v, d_o, D, lse, w, dk, dv, ws, part, s);
 }
 
 int convattn_bwd_fused_dq(const convattn_desc *desc, const void *q, const void *k, const void *v,

@@ -21,15 +21,7 @@
 //        tile after the last row finishes the last 16 rows
 //   dK^T += Q^T dS        (the flipped bands carry the softmax scale)
 //
-// FUSED instantiations do the whole backward in this one pass over the score tiles: they also
-//   * store dS (bf16, the operand of dK) to a workspace as [key tile of 32][row tile of 64]
-//     blocks of [32 keys][64 rows, permuted within groups of 32 so that a lane's 8 values are
-//     contiguous]; dQ = dS K is then a plain batched product (bwd_dq_gemm.hip);
-//   * accumulate dW[a][b] += sum over own rows i and own keys j' of
-//     S[i+a-pq][j'] * dC[i][j'-b+pk]: an MFMA contraction with M = a, N = b and (row, 8 keys)
-//     as the k index; the dC operand is read from LDS at a 2-byte granular offset.  Every
-//     (dC row, S key) pair belongs to exactly one (wave, tile); the waves' partials are summed
-//     in a fixed order and stored per workgroup.
+// (bwd_ws_mfma.hip is the whole-backward relative of this kernel: same tiles, two waves per SIMD.)
 #include <type_traits>
 
 #include "mfma_common.hpp"
@@ -55,7 +47,7 @@ constexpr int CST = (C_COLS + 8) * 2;  // 112
 constexpr int NSB = S_COLS / 16;       // 4 key blocks of S
 constexpr int NCB = C_COLS / 16;       // 3 key blocks of C / dP / dC
 constexpr int NRB = BR / 16;           // 4 own row blocks per tile
-static_assert(BKW == kKvKeysPerWg && WK == kDsKeys && BR == kDsRows, "dS workspace layout");
+static_assert(BKW == kKvKeysPerWg, "grid size");
 
 template <int D, int CQT> struct KvLds {
     static constexpr int RST = D * 2 + 16;
@@ -66,12 +58,12 @@ template <int D, int CQT> struct KvLds {
     static constexpr int total = q_bytes + g_bytes + stat_bytes + NW * wave_bytes;
 };
 
-template <int D, int CQT, typename TO, bool FUSED>
+template <int D, int CQT, typename TO>
 __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
     Problem p, const bf16_t *__restrict__ Q, const bf16_t *__restrict__ K,
     const bf16_t *__restrict__ V, const bf16_t *__restrict__ dO, const float *__restrict__ Dl,
     const float *__restrict__ LSE, const float *__restrict__ W, TO *__restrict__ dK,
-    TO *__restrict__ dV, bf16_t *__restrict__ dS_ws, float *__restrict__ dW_part) {
+    TO *__restrict__ dV) {
     using Lds = KvLds<D, CQT>;
     constexpr int RST = Lds::RST;
     constexpr int KS = D / 32, DB = D / 16, CPR = D / 8;
@@ -128,16 +120,6 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
             acc_k[m][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
             acc_v[m][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
         }
-
-    f32x4 acc_w[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) acc_w[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    const int bcl = n < ck ? n : ck - 1;  // dW: lanes past the last key tap re-read a valid one
-    const int pq = p.pq;
-    // dS workspace blocks of this wave: [key tile][row tile][32 keys][64 rows]
-    const int n_rt = (p.Nq + BR - 1) / BR;
-    bf16_t *ds_wave = nullptr;
-    if constexpr (FUSED) ds_wave = dS_ws + ((bh * gridDim.z * NW + blockIdx.z * NW + wave) * n_rt) * (size_t)(WK * BR);
 
     // Causal: rows before the first key this workgroup touches (k0 - 8) see none of its keys.
     const int r_begin = causal ? (max(0, k0 - 8) / BR) * BR : 0;
@@ -412,24 +394,6 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                         sf[kp][m][r] = (bf16_t)ds[2 * kp][m][r];
                         sf[kp][m][4 + r] = (bf16_t)ds[2 * kp + 1][m][r];
                     }
-            if constexpr (FUSED) {
-                // lane = key m*16+n holds rows 4g.. of each 16-row block.  Within a key the workspace
-                // keeps row 32k + 16h + 4g + r at position 32k + 8g + 4h + r (ds_row_of_pos in
-                // mfma_common.hpp is the inverse), so the blocks at rows r0 .. r0+31 make one 16-byte
-                // piece; the block at r0-16 completes the previous row tile, the one at r0+32 starts
-                // the second half of this one.
-                bf16_t *blk = ds_wave + (size_t)(r0 / BR) * (WK * BR);
-#pragma unroll
-                for (int m = 0; m < 2; ++m) {
-                    bf16_t *key = blk + (m * 16 + n) * BR + 8 * g;
-                    if (!EDGE || r0 > 0)  // (unmasked tiles never start at row 0)
-                        *reinterpret_cast<bf16x4 *>(key - WK * BR + 32 + 4) = __builtin_shufflevector(sf[0][m], sf[0][m], 0, 1, 2, 3);
-                    if (!tail) {
-                        *reinterpret_cast<bf16x8 *>(key) = __builtin_shufflevector(sf[0][m], sf[1][m], 4, 5, 6, 7, 8, 9, 10, 11);
-                        *reinterpret_cast<bf16x4 *>(key + 32) = __builtin_shufflevector(sf[1][m], sf[1][m], 4, 5, 6, 7);
-                    }
-                }
-            }
             constexpr int NST = (NRB / 2) * DB;
             bf16x8 qt[2];
             auto load_qt = [&](int buf, int st) {
@@ -453,46 +417,6 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
             }
         }
 
-        // ---- dW: rows m = tap a, columns n = tap b, contraction over (own row, 8 own keys) ----
-        if (FUSED && !tail) {
-            // A: S[i + a - pq][c0 + 8g ..]        (S-tile row HT + i + a - pq, column 16 + 8g)
-            // B: dC[i][c0 + 8g - b + pk ..]       (dC-tile row HT + i, column 8 + 8g - b + pk)
-            const unsigned char *abase = Ss + (HT + n - pq) * SST + (16 + 8 * g) * 2;
-            // LDS reads at odd 2-byte offsets are slow: read 5 dwords from the even
-            // element below and funnel-shift by 0 or 16 bits per lane instead.
-            const int boff = 8 + 8 * g - bcl + pk;
-            const unsigned char *bbase = Cs + HT * CST + (boff & ~1) * 2;
-            const unsigned int bsh = (boff & 1) * 16;
-            // The S operand of row i+1 is the one of row i moved down by one lane (lane n holds S row
-            // i + n - pq), so it is read from LDS once per RPL rows and shifted within the 16-lane
-            // rows in between; only lanes n < c_q matter, and (c_q - 1) + (RPL - 1) <= 15.
-            constexpr int RPL = CQT <= 6 ? 8 : 4;
-            static_assert(BR % RPL == 0 && (CQT - 1) + (RPL - 1) <= 15, "dW row groups");
-#pragma unroll 1
-            for (int i = 0; i < BR; i += RPL) {
-                u32x4 af = *reinterpret_cast<const u32x4 *>(abase + i * SST);
-                u32x4 bw[RPL];
-                unsigned int bx[RPL];
-#pragma unroll
-                for (int u = 0; u < RPL; ++u) {
-                    bw[u] = reinterpret_cast<const U32x4A4 *>(bbase + (i + u) * CST)->v;
-                    bx[u] = *reinterpret_cast<const unsigned int *>(bbase + (i + u) * CST + 16);
-                }
-#pragma unroll
-                for (int u = 0; u < RPL; ++u) {
-                    u32x4 sh;
-                    sh[0] = __builtin_amdgcn_alignbit(bw[u][1], bw[u][0], bsh);
-                    sh[1] = __builtin_amdgcn_alignbit(bw[u][2], bw[u][1], bsh);
-                    sh[2] = __builtin_amdgcn_alignbit(bw[u][3], bw[u][2], bsh);
-                    sh[3] = __builtin_amdgcn_alignbit(bx[u], bw[u][3], bsh);
-                    acc_w[u & 3] = mfma_f16(__builtin_bit_cast(f16x8, af), __builtin_bit_cast(f16x8, sh), acc_w[u & 3]);
-                    if (u + 1 < RPL) {
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) af[r] = lane_from_next(af[r]);
-                    }
-                }
-            }
-        }
         // ---- the last 16 dC rows become the first 16 of the next tile ----
         __builtin_amdgcn_wave_barrier();
         for (int c = lane; c < HT * (CST / 16); c += 64) {
@@ -542,101 +466,67 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
         }
     }
 
-    // ---- dW partial of this workgroup: ordered sum over the 4 waves; S was raw, so * scale ----
-    if constexpr (FUSED) {
-        __syncthreads();
-        float *red = reinterpret_cast<float *>(smem);  // [NW][16][16]
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-            red[(wave * 16 + 4 * g + r) * 16 + n] = (acc_w[0][r] + acc_w[1][r]) + (acc_w[2][r] + acc_w[3][r]);
-        __syncthreads();
-        const int ntap = cq * ck;
-        if (tid < ntap) {
-            const int a = tid / ck, bb = tid - a * ck;
-            float sum = 0.f;
-#pragma unroll
-            for (int w = 0; w < NW; ++w) sum += red[(w * 16 + a) * 16 + bb];
-            dW_part[(bh * gridDim.z + blockIdx.z) * ntap + tid] = sum * p.scale;
-        }
-    }
 }
 
-template <int D, int CQT, typename TO, bool FUSED>
+template <int D, int CQT, typename TO>
 hipError_t launch_kv(const Problem &p, const void *q, const void *k, const void *v, const void *d_o,
-                     const float *Dl, const float *lse, const float *w, void *dk, void *dv, void *ds_ws,
-                     float *dw_part, hipStream_t s) {
-    auto kern = bwd_dkdv_mfma_kernel<D, CQT, TO, FUSED>;
+                     const float *Dl, const float *lse, const float *w, void *dk, void *dv,
+                     hipStream_t s) {
+    auto kern = bwd_dkdv_mfma_kernel<D, CQT, TO>;
     constexpr int lds = KvLds<D, CQT>::total;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return e;
     dim3 grid(p.H, p.B, mfma_kv_tiles(p));
     kern<<<grid, NW * 64, lds, s>>>(p, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v,
-                                    (const bf16_t *)d_o, Dl, lse, w, (TO *)dk, (TO *)dv, (bf16_t *)ds_ws,
-                                    dw_part);
+                                    (const bf16_t *)d_o, Dl, lse, w, (TO *)dk, (TO *)dv);
     return hipGetLastError();
 }
 
 }  // namespace
 
-// This file is built as four objects, CONVATTN_DKDV_UNIT = 2 * fused + wide: "wide" holds the
-// 11-tap-slot instantiations (the slowest to compile), "fused" the whole-backward variants; the
-// two narrow units also hold the entry points.
-template <int D, typename TO, bool FUSED>
+// This file is built as two objects so that they compile in parallel: CONVATTN_DKDV_UNIT = 1
+// holds the 11-tap-slot instantiations (the slowest), 0 the others and the entry point.
+template <int D, typename TO>
 hipError_t dkdv_wide(const Problem &p, const void *q, const void *k, const void *v, const void *d_o,
-                     const float *Dl, const float *lse, const float *w, void *dk, void *dv, void *ds_ws,
-                     float *dw_part, hipStream_t s);
+                     const float *Dl, const float *lse, const float *w, void *dk, void *dv,
+                     hipStream_t s);
 
-constexpr bool kFusedUnit = (CONVATTN_DKDV_UNIT & 2) != 0;
-
-#if CONVATTN_DKDV_UNIT & 1
-template <int D, typename TO, bool FUSED>
+#if CONVATTN_DKDV_UNIT == 1
+template <int D, typename TO>
 hipError_t dkdv_wide(const Problem &p, const void *q, const void *k, const void *v, const void *d_o,
-                     const float *Dl, const float *lse, const float *w, void *dk, void *dv, void *ds_ws,
-                     float *dw_part, hipStream_t s) {
-    return launch_kv<D, 11, TO, FUSED>(p, q, k, v, d_o, Dl, lse, w, dk, dv, ds_ws, dw_part, s);
+                     const float *Dl, const float *lse, const float *w, void *dk, void *dv,
+                     hipStream_t s) {
+    return launch_kv<D, 11, TO>(p, q, k, v, d_o, Dl, lse, w, dk, dv, s);
 }
-#define CONVATTN_INST(D, TO)                                                                             \
-    template hipError_t dkdv_wide<D, TO, kFusedUnit>(const Problem &, const void *, const void *,        \
-                                                     const void *, const void *, const float *,          \
-                                                     const float *, const float *, void *, void *,       \
-                                                     void *, float *, hipStream_t);
+#define CONVATTN_INST(D, TO)                                                                          \
+    template hipError_t dkdv_wide<D, TO>(const Problem &, const void *, const void *, const void *,   \
+                                         const void *, const float *, const float *, const float *,   \
+                                         void *, void *, hipStream_t);
 CONVATTN_INST(128, bf16_t) CONVATTN_INST(128, float) CONVATTN_INST(64, bf16_t) CONVATTN_INST(64, float)
 #undef CONVATTN_INST
 #else
 namespace {
 template <int D, typename TO>
 hipError_t pick_cq(const Problem &p, const void *q, const void *k, const void *v, const void *d_o,
-                   const float *Dl, const float *lse, const float *w, void *dk, void *dv, void *ds_ws,
-                   float *dw_part, hipStream_t s) {
-    if (p.c_q <= 3) return launch_kv<D, 3, TO, kFusedUnit>(p, q, k, v, d_o, Dl, lse, w, dk, dv, ds_ws, dw_part, s);
-    if (p.c_q <= 6) return launch_kv<D, 6, TO, kFusedUnit>(p, q, k, v, d_o, Dl, lse, w, dk, dv, ds_ws, dw_part, s);
-    return dkdv_wide<D, TO, kFusedUnit>(p, q, k, v, d_o, Dl, lse, w, dk, dv, ds_ws, dw_part, s);
-}
-template <typename... A>
-hipError_t pick_d(const Problem &p, int out_dt, A... a) {
-    if (p.d == 128) {
-        if (out_dt == CONVATTN_BF16) return pick_cq<128, bf16_t>(p, a...);
-        return pick_cq<128, float>(p, a...);
-    }
-    if (out_dt == CONVATTN_BF16) return pick_cq<64, bf16_t>(p, a...);
-    return pick_cq<64, float>(p, a...);
+                   const float *Dl, const float *lse, const float *w, void *dk, void *dv,
+                   hipStream_t s) {
+    if (p.c_q <= 3) return launch_kv<D, 3, TO>(p, q, k, v, d_o, Dl, lse, w, dk, dv, s);
+    if (p.c_q <= 6) return launch_kv<D, 6, TO>(p, q, k, v, d_o, Dl, lse, w, dk, dv, s);
+    return dkdv_wide<D, TO>(p, q, k, v, d_o, Dl, lse, w, dk, dv, s);
 }
 }  // namespace
 
-#if CONVATTN_DKDV_UNIT & 2
-hipError_t mfma_bwd_fused(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
-                          const void *d_o, const float *Dl, const float *lse, const float *w, void *dk,
-                          void *dv, void *ds_ws, float *dw_part, hipStream_t s) {
-    return pick_d(p, out_dt, q, k, v, d_o, Dl, lse, w, dk, dv, ds_ws, dw_part, s);
-}
-#else
 hipError_t mfma_bwd_dkdv(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
                          const void *d_o, const float *Dl, const float *lse, const float *w, void *dk,
                          void *dv, hipStream_t s) {
-    return pick_d(p, out_dt, q, k, v, d_o, Dl, lse, w, dk, dv, (void *)nullptr, (float *)nullptr, s);
+    if (p.d == 128) {
+        if (out_dt == CONVATTN_BF16) return pick_cq<128, bf16_t>(p, q, k, v, d_o, Dl, lse, w, dk, dv, s);
+        return pick_cq<128, float>(p, q, k, v, d_o, Dl, lse, w, dk, dv, s);
+    }
+    if (out_dt == CONVATTN_BF16) return pick_cq<64, bf16_t>(p, q, k, v, d_o, Dl, lse, w, dk, dv, s);
+    return pick_cq<64, float>(p, q, k, v, d_o, Dl, lse, w, dk, dv, s);
 }
-#endif
 #endif
 
 }  // namespace convattn

@@ -44,7 +44,7 @@ __global__ __launch_bounds__(NW * 64) void dq_from_ds_kernel(Problem p, const bf
     const int g = lane >> 4, n = lane & 15;
     const int h = blockIdx.x, b = blockIdx.y;
     const int qt = gridDim.z - 1 - blockIdx.z;  // longest (causal) row tiles first
-    const int i0 = qt * BQ, rw = i0 + wave * 32;
+    const int i0 = qt * BQ - kDsRowShift, rw = i0 + wave * 32;  // the dS row tiles start 16 rows early
     const bool causal = p.causal != 0;
     const size_t bh = (size_t)b * p.H + h;
     const bf16_t *Kb = K + bh * p.Nk * D;
@@ -72,7 +72,8 @@ __global__ __launch_bounds__(NW * 64) void dq_from_ds_kernel(Problem p, const bf
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int kt = s * 2 + (i >> 1), rt = qt * 2 + (i & 1);
-            tv[i] = kt * kDsKeys < p.Nk && rt < n_rt && (!causal || kt * kDsKeys < (rt + 1) * kDsRows);
+            tv[i] = kt * kDsKeys < p.Nk && rt < n_rt &&
+                    (!causal || kt * kDsKeys < (rt + 1) * kDsRows - kDsRowShift);  // first key <= last row of the block
             const size_t blk = (size_t)min(kt, n_kt - 1) * n_rt + min(rt, n_rt - 1);
             tr[i] = *reinterpret_cast<const u32x4 *>(ws + blk * BLK + t_key * kDsRows + t_ch * 8);
         }
@@ -120,7 +121,7 @@ __global__ __launch_bounds__(NW * 64) void dq_from_ds_kernel(Problem p, const bf
 #pragma unroll
     for (int ob = 0; ob < 2; ++ob) {
         const int qpos = rw + ds_row_of_pos(ob * 16 + n);
-        if (qpos < p.Nq) {
+        if (qpos >= 0 && qpos < p.Nq) {
             TO *orow = dQ + (bh * p.Nq + qpos) * D;
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
@@ -145,7 +146,7 @@ hipError_t launch(const Problem &p, const void *k, const void *ds_ws, void *dq, 
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return e;
-    dim3 grid(p.H, p.B, (p.Nq + BQ - 1) / BQ);
+    dim3 grid(p.H, p.B, (p.Nq + kDsRowShift + BQ - 1) / BQ);
     kern<<<grid, NW * 64, lds, s>>>(p, (const bf16_t *)k, (const bf16_t *)ds_ws, mfma_ds_key_tiles(p),
                                     mfma_ds_row_tiles(p), (TO *)dq);
     return hipGetLastError();

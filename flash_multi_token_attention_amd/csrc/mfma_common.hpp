@@ -180,25 +180,27 @@ hipError_t mfma_bwd_dkdv(const Problem &p, int out_dt, const void *q, const void
                          void *dv, hipStream_t s);
 
 // ---- whole backward in one pass over the score tiles ----
-// The dK/dV kernel's workgroups cover 128 keys each (+ 8: the dV ranges start 8 keys early); its
-// waves own 32 keys and walk the rows in tiles of 64.  The fused variant leaves one dW partial
-// per workgroup and dS as bf16 blocks [key tile of 32][row tile of 64][32 keys][64 rows];
-// mfma_dq_from_ds multiplies those blocks with K.
-constexpr int kKvKeysPerWg = 128, kDsKeys = 32, kDsRows = 64;
+// The key-stationary kernel's workgroups cover 128 keys each (+ 8: the dV ranges start 8 keys
+// early).  Besides dK and dV it leaves one dW partial per workgroup and dS as bf16 blocks
+// [key tile of 32][row tile of 64][32 keys][64 rows]; mfma_dq_from_ds multiplies those blocks
+// with K.  dS of a row is finished 16 rows after the row itself, so the row tiles are shifted:
+// row tile rt holds rows 64 rt - 16 .. 64 rt + 47.
+constexpr int kKvKeysPerWg = 128, kDsKeys = 32, kDsRows = 64, kDsRowShift = 16;
 // Inside a dS block the 64 rows of a key are stored in the order the producing lanes hold
-// them: position 32kp + 8g + 4h + r holds row 32kp + 16h + 4g + r.
+// them: position 32k + 8g + 4h + r holds the block's row 32k + 16h + 4g + r.
 __host__ __device__ inline int ds_row_of_pos(int pos) {
     return (pos & 32) | ((pos & 4) << 2) | ((pos >> 3 & 3) << 2) | (pos & 3);
 }
 inline int mfma_kv_tiles(const Problem &p) { return (p.Nk + 8 + kKvKeysPerWg - 1) / kKvKeysPerWg; }
 inline int mfma_ds_key_tiles(const Problem &p) { return mfma_kv_tiles(p) * (kKvKeysPerWg / kDsKeys); }
-inline int mfma_ds_row_tiles(const Problem &p) { return (p.Nq + kDsRows - 1) / kDsRows; }
+__host__ __device__ inline int mfma_ds_row_tiles(const Problem &p) { return (p.Nq + kDsRowShift + kDsRows - 1) / kDsRows; }
 inline size_t mfma_ds_bytes(const Problem &p) {
     return (size_t)p.B * p.H * mfma_ds_key_tiles(p) * mfma_ds_row_tiles(p) * kDsKeys * kDsRows * 2;
 }
-hipError_t mfma_bwd_fused(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
-                          const void *d_o, const float *Dl, const float *lse, const float *w, void *dk,
-                          void *dv, void *ds_ws, float *dw_part, hipStream_t s);
+// bwd_ws_mfma.hip: 8-wave workgroups, producer / consumer wave pairs, two waves per SIMD.
+hipError_t mfma_bwd_fused_ws(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
+                             const void *d_o, const float *Dl, const float *lse, const float *w, void *dk,
+                             void *dv, void *ds_ws, float *dw_part, hipStream_t s);
 hipError_t mfma_dq_from_ds(const Problem &p, int out_dt, const void *k, const void *ds_ws, void *dq,
                            hipStream_t s);
 
