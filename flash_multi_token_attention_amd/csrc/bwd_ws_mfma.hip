@@ -6,10 +6,10 @@
 // the whole instruction, so a wave alone on a SIMD cannot overlap its MFMAs with its own VALU or
 // LDS work, and the one-wave kernel needs all 512 registers.  Here a workgroup is 8 waves = 4
 // pairs; pair p owns keys c0 = k0 + 32p .. c0+31 (dV: c0-8 .. c0+23), and the work of a
-// 32-row tile is split between the two waves of the pair, which sit on the same SIMD:
-//   producer (waves 0..3): keeps the K / V fragments; S^T = K Q^T (rows r0-16 .. r0+31) -> LDS,
+// 32-row tile is split between the two waves of the pair:
+//   producer (even waves): keeps the K / V fragments; S^T = K Q^T (rows r0-16 .. r0+31) -> LDS,
 //       C by Toeplitz MFMAs, P = exp2(C - LSE), dP = dO V^T, dC = P (dP - D) -> LDS, P -> LDS
-//   consumer (waves 4..7): keeps the dK / dV / dW accumulators; one tile behind the producer:
+//   consumer (odd waves):  keeps the dK / dV / dW accumulators; one tile behind the producer:
 //       dV^T += dO^T P, dS (rows r0-16 .. r0+15, flipped-band MFMAs over dC) -> workspace,
 //       dK^T += Q^T dS, dW += S (x) dC
 // Everything the consumer reads (Q, dO, S, dC, P of the previous tile) is double-buffered in
@@ -67,8 +67,8 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     const int g = lane >> 4, n = lane & 15;
-    const bool producer = wave < NP;   // waves w and w+4 land on the same SIMD
-    const int pr = wave & (NP - 1);
+    const bool producer = (wave & 1) == 0;   // (measured: this assignment beats waves 0-3 / 4-7)
+    const int pr = wave >> 1;
     auto stage_q = [&](int buf) { return smem + buf * Lds::stage_bytes; };
     auto stage_g = [&](int buf) { return smem + buf * Lds::stage_bytes + Lds::q_bytes; };
     auto stage_lse = [&](int buf) {
