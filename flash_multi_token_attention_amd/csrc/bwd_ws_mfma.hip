@@ -190,8 +190,18 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
                 }
             }
 
-            // ---- S^T tile (raw) -> fp16 LDS; Q fragments one row block ahead ----
+            // ---- S^T tile (raw) -> fp16 LDS; Q fragments one row block ahead.  The first 16 rows
+            // are the last 16 of the previous tile (masks depend on positions only): taken over from
+            // the other buffer when that tile was computed. ----
             {
+                const bool carry_s = it > 0 && !is_skipped(r0 - BR);
+                if (carry_s) {
+                    const unsigned char *prev = pair_s((it & 1) ^ 1) + BR * SST;
+                    for (int c = lane; c < HT * (S_COLS / 8); c += 64) {
+                        const int off = (c / (S_COLS / 8)) * SST + (c % (S_COLS / 8)) * 16;
+                        *reinterpret_cast<u32x4 *>(Ss + off) = *reinterpret_cast<const u32x4 *>(prev + off);
+                    }
+                }
                 bf16x8 qf[2][KS];
                 auto load_qf = [&](int buf, int rb) {
 #pragma unroll
@@ -207,6 +217,7 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
                         load_qf(cur ^ 1, rb + 1);
                         SCHED_DS_READ_ID(KS, 11 + rb);
                     }
+                    if (rb == 0 && carry_s) return;
                     f32x4 acc[NSB];
 #pragma unroll
                     for (int kb = 0; kb < NSB; ++kb) acc[kb] = (f32x4){0.f, 0.f, 0.f, 0.f};
