@@ -368,31 +368,6 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
         const unsigned char *Qs = stage_q(buf), *Gs = stage_g(buf);
         const unsigned char *Ss = pair_s(buf), *Cs = pair_c(buf), *Ps = pair_p(buf);
 
-        // ---- dV^T += dO^T P  (keys c0-8 .. c0+23); dO^T by transpose reads of the dO tile ----
-        {
-            bf16x8 pf[2];
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb) pf[kb] = *reinterpret_cast<const bf16x8 *>(Ps + (kb * 64 + lane) * 16);
-            bf16x8 gt[2];
-            auto load_gt = [&](int b2, int db) {
-                bf16x4 lo = lds_read_tr4x16(Gs, RST, 4 * g, db * 16, n);
-                bf16x4 hi = lds_read_tr4x16(Gs, RST, 16 + 4 * g, db * 16, n);
-                gt[b2] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-            };
-            load_gt(0, 0);
-            SCHED_DS_READ_ID(2, 30);
-#pragma unroll
-            for (int db = 0; db < DB; ++db) {
-                if (db + 1 < DB) {
-                    load_gt((db + 1) & 1, db + 1);
-                    SCHED_DS_READ_ID(2, 30);
-                }
-#pragma unroll
-                for (int kb = 0; kb < 2; ++kb) acc_v[kb][db] = mfma_bf16(gt[db & 1], pf[kb], acc_v[kb][db]);
-                SCHED_MFMA_ID(2, 30);
-            }
-        }
-
         // ---- dS, rows r0-16 .. r0+15 (keys c0 .. c0+31): chains over the taps; the dC buffer
         // starts at row r0-16 ----
         f32x4 ds[NRB][2];
@@ -431,7 +406,7 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
                     for (int r = 0; r < 4; ++r)
                         if (c0 + m * 16 + n > r0 - HT + ob * 16 + 4 * g + r) ds[ob][m][r] = 0.f;
         }
-        // ---- dK^T += Q^T dS; Q^T by transpose reads (the Q tile starts at row r0-16 as well) ----
+        // ---- dK^T += Q^T dS (the Q tile starts at row r0-16 as well) and dV ----
         {
             bf16x8 sf[2];
 #pragma unroll
@@ -448,23 +423,34 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
             for (int m = 0; m < 2; ++m)
                 *reinterpret_cast<bf16x8 *>(ds_pair + (size_t)(r0 / kDsRows) * (WK * kDsRows) +
                                             (m * 16 + n) * kDsRows + (r0 % kDsRows) + 8 * g) = sf[m];
-            bf16x8 qt[2];
-            auto load_qt = [&](int b2, int db) {
+            // dV^T += dO^T P (keys c0-8 .. c0+23) shares the loop: dO^T and Q^T by transpose reads of
+            // the row-major tiles, four independent MFMAs per head-dim block
+            bf16x8 pf[2];
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) pf[kb] = *reinterpret_cast<const bf16x8 *>(Ps + (kb * 64 + lane) * 16);
+            bf16x8 qt[2], gt[2];
+            auto load_qg = [&](int b2, int db) {
                 bf16x4 lo = lds_read_tr4x16(Qs, RST, 4 * g, db * 16, n);
                 bf16x4 hi = lds_read_tr4x16(Qs, RST, 16 + 4 * g, db * 16, n);
                 qt[b2] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                lo = lds_read_tr4x16(Gs, RST, 4 * g, db * 16, n);
+                hi = lds_read_tr4x16(Gs, RST, 16 + 4 * g, db * 16, n);
+                gt[b2] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
             };
-            load_qt(0, 0);
-            SCHED_DS_READ_ID(2, 32);
+            load_qg(0, 0);
+            SCHED_DS_READ_ID(6, 32);
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
                 if (db + 1 < DB) {
-                    load_qt((db + 1) & 1, db + 1);
-                    SCHED_DS_READ_ID(2, 32);
+                    load_qg((db + 1) & 1, db + 1);
+                    SCHED_DS_READ_ID(4, 32);
                 }
 #pragma unroll
-                for (int m = 0; m < 2; ++m) acc_k[m][db] = mfma_bf16(qt[db & 1], sf[m], acc_k[m][db]);
-                SCHED_MFMA_ID(2, 32);
+                for (int m = 0; m < 2; ++m) {
+                    acc_k[m][db] = mfma_bf16(qt[db & 1], sf[m], acc_k[m][db]);
+                    acc_v[m][db] = mfma_bf16(gt[db & 1], pf[m], acc_v[m][db]);
+                }
+                SCHED_MFMA_ID(4, 32);
             }
         }
 
