@@ -286,3 +286,36 @@ def test_c5_long_context_one_head_forward_and_backward():
     dQ1, dK1, dV1, dW1 = ops.backward(Q, K, V, dO, D, LSE, W, *args, out_dtype=torch.bfloat16)
     assert max_abs(dQ1, dQ_x) <= TOL_BF16 and max_abs(dK1, dK_x) <= TOL_BF16 and max_abs(dV1, dV_x) <= TOL_BF16
     assert rel_max(dW1, dW_x) <= TOL_DW_REL
+
+
+def test_one_pass_backward_steps_through_the_c_abi():
+    # The three steps of convattn_bwd_fused called one by one on raw pointers (what bench.py
+    # times) give exactly what the single call gives, and what the Python op returns.
+    import ctypes as C
+
+    from flash_multi_token_attention_amd import _lib
+    lib = _lib.load()
+    B, H, N, d, c_q, c_k = 2, 2, 300, 128, 6, 11
+    Q, K, V, dO, W = (t.to(DEV) for t in rand_case(B, H, N, N, d, c_q, c_k, torch.bfloat16, seed=21))
+    sc = scale_of(d)
+    O, M, L = ops.forward(Q, K, V, W, sc, c_q - 1, (c_k - 1) // 2, True, out_dtype=torch.bfloat16)
+    D, LSE = ops.bwd_preprocess(O, dO, M, L)
+    ref = ops.backward(Q, K, V, dO, D, LSE, W, sc, c_q - 1, (c_k - 1) // 2, True, out_dtype=torch.bfloat16)
+    desc = _lib.Desc(B, H, N, N, d, c_q, c_k, sc, 1, _lib.BF16, _lib.BF16, 1, 0)
+    ws = torch.empty(lib.convattn_bwd_fused_workspace_bytes(C.byref(desc)), dtype=torch.uint8, device=DEV)
+    p = lambda t: C.c_void_p(t.data_ptr())
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ins = (p(Q), p(K), p(V), p(dO), p(D), p(LSE), p(W))
+    for whole in (True, False):
+        dQ, dK, dV = (torch.empty_like(Q) for _ in range(3))
+        dW = torch.empty_like(W)
+        ws.fill_(0xFF)   # NaN patterns: nothing may depend on the workspace's previous contents
+        if whole:
+            assert lib.convattn_bwd_fused(C.byref(desc), *ins, p(dQ), p(dK), p(dV), p(dW), p(ws), st) == 0
+        else:
+            assert lib.convattn_bwd_fused_dkdv(C.byref(desc), *ins, p(dK), p(dV), p(ws), st) == 0
+            assert lib.convattn_bwd_fused_dq(C.byref(desc), *ins, p(dQ), p(ws), st) == 0
+            assert lib.convattn_bwd_fused_dw(C.byref(desc), p(ws), p(dW), st) == 0
+        torch.cuda.synchronize()
+        for got, want in zip((dQ, dK, dV, dW), ref):
+            assert torch.equal(got, want)
