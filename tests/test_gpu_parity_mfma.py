@@ -319,3 +319,33 @@ def test_one_pass_backward_steps_through_the_c_abi():
         torch.cuda.synchronize()
         for got, want in zip((dQ, dK, dV, dW), ref):
             assert torch.equal(got, want)
+
+
+def test_seeded_random_shapes_forward_and_both_backward_paths():
+    # Lengths on and around the 32/64/128-row tile borders, both head dims, every tap-slot
+    # class of the kernels (<=3, <=6, <=11 query taps), odd key windows up to 15 taps.
+    import random
+    rng = random.Random(7)
+    lengths = [1, 2, 17, 31, 32, 33, 63, 64, 65, 95, 96, 97, 127, 128, 129, 160, 191, 192, 255, 257, 300,
+               383, 385, 450]
+    for t in range(24):
+        d = rng.choice([64, 128])
+        c_q, c_k = rng.randint(1, 11), rng.choice([1, 3, 5, 7, 9, 11, 13, 15])
+        causal = rng.random() < 0.6
+        Nq = rng.choice(lengths)
+        Nk = Nq if causal else rng.choice([Nq, max(1, Nq // 2), Nq + 37, 129])
+        B, H = rng.choice([(1, 1), (1, 2), (2, 1)])
+        Q, K, V, dO, W = rand_case(B, H, Nq, Nk, d, c_q, c_k, torch.bfloat16, seed=100 + t,
+                                   w_mode=rng.choice(["rand", "delta"]))
+        O_ref, _, _ = oracle_fwd(Q, K, V, W, causal)
+        ref = oracle_bwd(Q, K, V, W, dO, causal)
+        g = [x.to(DEV) for x in (Q, K, V, dO, W)]
+        case = f"B{B} H{H} Nq{Nq} Nk{Nk} d{d} {c_q}x{c_k} causal={causal}"
+        O, _, _ = ops.forward(g[0], g[1], g[2], g[4], scale_of(d), c_q - 1, (c_k - 1) // 2, causal)
+        assert max_abs(O, O_ref) <= TOL_BF16, case
+        for one_pass in (False, True):
+            dQ, dK, dV, dW = _run_bwd(*g, causal, torch.bfloat16, one_pass)
+            assert max_abs(dQ, ref[0]) <= TOL_BF16, case
+            assert max_abs(dK, ref[1]) <= TOL_BF16, case
+            assert max_abs(dV, ref[2]) <= TOL_BF16, case
+            assert rel_max(dW, ref[3]) <= TOL_DW_REL, case
