@@ -1,4 +1,5 @@
-// Training forward of conv-attention on bf16 MFMA (gfx950).
+// Training forward of conv-attention on bf16 MFMA (gfx950), scores staged in LDS: the kernel for
+// windows of 7 to 11 query taps (narrower ones: fwd_reg_mfma.hip).
 //
 // Workgroup = 4 waves = 128 query rows of one (batch, head); wave w owns rows
 // i0 + 32w .. +31 and keeps their O^T accumulators, running max and partial row
@@ -358,8 +359,6 @@ hipError_t launch_fwd(const Problem &p, const void *q, const void *k, const void
 template <int D, typename TO>
 hipError_t pick_cq(const Problem &p, const void *q, const void *k, const void *v, const float *w,
                    void *o, float *m, float *l, hipStream_t s) {
-    if (p.c_q <= 3) return launch_fwd<D, 3, TO>(p, q, k, v, w, o, m, l, s);
-    if (p.c_q <= 6) return launch_fwd<D, 6, TO>(p, q, k, v, w, o, m, l, s);
     return launch_fwd<D, 11, TO>(p, q, k, v, w, o, m, l, s);
 }
 
@@ -367,6 +366,7 @@ hipError_t pick_cq(const Problem &p, const void *q, const void *k, const void *v
 
 hipError_t mfma_fwd(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
                     const float *w, void *o, float *m, float *l, hipStream_t s) {
+    if (p.c_q <= kMfmaFwdRegMaxCq) return mfma_fwd_reg(p, out_dt, q, k, v, w, o, m, l, s);
     if (p.d == 128) {
         if (out_dt == CONVATTN_BF16) return pick_cq<128, bf16_t>(p, q, k, v, w, o, m, l, s);
         return pick_cq<128, float>(p, q, k, v, w, o, m, l, s);

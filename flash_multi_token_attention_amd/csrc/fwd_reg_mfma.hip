@@ -1,0 +1,415 @@
+// Training forward of conv-attention on bf16 MFMA (gfx950) for windows of up to 6 query taps:
+// the scores never leave the registers.
+//
+// Workgroup = 4 waves of one (batch, head); a wave computes scores for 32 consecutive query rows
+// (the first CQT-1 of them only as the window's halo above its 33-CQT output rows) and keeps
+// O^T, the row sums and the softmax bases of its rows in registers for the whole key loop.
+// Lane n of score fragment f holds row base + 2n + f.  Per 32-key step:
+//   1. all waves write the K / V rows they loaded two steps ago to the LDS buffer of the next
+//      step and issue the loads for the step after it (one barrier per step);
+//   2. S^T = K Q^T for two 16-key blocks; the accumulator layout (lane = query row, 4 keys per
+//      lane group) is, packed to fp16 after the causal pre-mask, already the B operand layout of
+//      the convolution MFMA: k slots 0..3 of a lane group come from one block, 4..7 from the next
+//      (the Toeplitz bands are built for that order), so a window of 32 input keys is two packed
+//      blocks and the output block sits 8 keys into it.  The last block of a step is carried to
+//      the next step; no score is computed twice along the keys;
+//   3. convolution: C^T += T_a^T S^T(rows shifted by the tap).  A shift by an even number of
+//      rows is a DPP row shift of the packed registers, by an odd number the other fragment
+//      shifted; rows shifted in from above the wave's first row are zeros and only reach halo rows;
+//   4. post-mask (-inf) and softmax numerators against a per-row base that is only raised (with
+//      a rescale of O and the row sums) when a score exceeds it by more than 2^6: no cross-lane
+//      traffic otherwise.  The true row maximum is kept per lane for the M output;
+//   5. O^T += V^T P^T: V^T fragments through the LDS transpose read, P^T straight from the
+//      softmax registers.
+#include "mfma_common.hpp"
+
+namespace convattn {
+namespace {
+
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+
+// DPP move (CTRL 0x110+s: row_shr:s, lane n of a row of 16 gets lane n-s); lanes without a
+// source lane get 0.
+template <int CTRL>
+__device__ __forceinline__ unsigned int dpp_zero(unsigned int src) {
+    return (unsigned int)__builtin_amdgcn_update_dpp(0, (int)src, CTRL, 0xf, 0xf, true);
+}
+
+constexpr int NW = 4;             // waves per workgroup
+constexpr int BK = 32;            // keys per step
+constexpr float kMaxSlack = 6.f;  // log2 units a score may exceed its row's exponent base by
+// A wave computes scores for 32 consecutive rows; the first CQT-1 of them are only the
+// window's halo, the other 33-CQT are its output rows.
+constexpr int wave_rows(int cqt) { return 33 - cqt; }
+
+template <int D> struct FwdLds {
+    static constexpr int KST = D * 2 + 16;  // bytes per K / V row (== 16 mod 256 for D = 128)
+    static constexpr int k_bytes = BK * KST;
+    static constexpr int buf_bytes = 2 * k_bytes;  // K rows, then V rows
+    static constexpr int total = 2 * buf_bytes;    // double-buffered
+};
+
+template <int D, int CQT, typename TO>
+__global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
+    Problem p, const bf16_t *__restrict__ Q, const bf16_t *__restrict__ K,
+    const bf16_t *__restrict__ V, const float *__restrict__ W, TO *__restrict__ O,
+    float *__restrict__ M, float *__restrict__ L) {
+    using Lds = FwdLds<D>;
+    constexpr int KST = Lds::KST;
+    constexpr int KS = D / 32;   // MFMA k-steps over the head dimension
+    constexpr int DB = D / 16;   // 16-wide blocks of the head dimension
+    constexpr int CPR = D / 8;   // 16-byte chunks per row
+    constexpr int WR = wave_rows(CQT), BQ = NW * WR;
+    constexpr int N_LD = BK * CPR / (NW * 64);  // 16-byte chunks per thread and matrix
+    static_assert(BK * CPR % (NW * 64) == 0, "whole chunks per thread");
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int g = lane >> 4, n = lane & 15;
+
+    // x = head, y = batch, z = query tile: the dispatcher hands out every (batch, head) of the
+    // longest (causal) tiles first, so the tail of the launch is made of short tiles
+    const int h = blockIdx.x, b = blockIdx.y;
+    const int qt = gridDim.z - 1 - blockIdx.z;
+    const int i0 = qt * BQ, i0w = i0 + wave * WR;
+    const int base = i0w - (CQT - 1);  // first score row of the wave
+    const int pk = p.pk, cq = p.c_q;
+    const bool causal = p.causal != 0;
+    const size_t bh = (size_t)b * p.H + h;
+    const bf16_t *Qb = Q + bh * p.Nq * D;
+    const bf16_t *Kb = K + bh * p.Nk * D;
+    const bf16_t *Vb = V + bh * p.Nk * D;
+
+    // Toeplitz bands of this head, one fragment per tap slot, pre-multiplied by
+    // scale * log2(e): the convolved scores come out in log2 units.  k slot 8g+e of a window
+    // is key 4g+e of its first 16-key block for e < 4, key 4g+e-4 of its second for e >= 4.
+    f16x8 tf[CQT];
+    {
+        const float *w_head = W + (size_t)h * cq * p.c_k;
+#pragma unroll
+        for (int t = 0; t < CQT; ++t) {
+            const int a = t - (CQT - cq);
+            f16x8 f = (f16x8)(_Float16)0.f;
+            if (a >= 0) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const int kappa = e < 4 ? 4 * g + e : 16 + 4 * g + e - 4;
+                    const int bb = kappa - kKeyHalo - n + pk;
+                    float v = 0.f;
+                    if (bb >= 0 && bb < p.c_k) v = w_head[a * p.c_k + bb] * (p.scale * kLog2e);
+                    f[e] = (_Float16)v;
+                }
+            }
+            tf[t] = f;
+        }
+    }
+
+    // Q^T fragments (B operand), resident for the whole loop: lane n of fragment f holds row
+    // base + 2n + f, so a shift of the score rows by an even number of rows is a shift of
+    // lanes and by an odd number a change of fragment as well.
+    bf16x8 qf[2][KS];
+#pragma unroll
+    for (int f = 0; f < 2; ++f)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+            qf[f][ks] = __builtin_bit_cast(bf16x8, load_row16_nb<D>(Qb, base + 2 * n + f, p.Nq, ks * 32 + g * 8));
+
+    f32x4 acc_o[2][DB];
+#pragma unroll
+    for (int ob = 0; ob < 2; ++ob)
+#pragma unroll
+        for (int db = 0; db < DB; ++db) acc_o[ob][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    float m_ref[2] = {kNegInf, kNegInf};   // exponent base of the row, in log2 units (same in the row's 4 lanes)
+    float m_true[2] = {kNegInf, kNegInf};  // maximum of the scores this lane has seen
+    float l_run[2] = {0.f, 0.f};           // this lane's share of the row sum, relative to m_ref
+
+    // Step u: score blocks 2u, 2u+1 (keys 32u-8 .. 32u+23, K rows of the step) and output blocks
+    // 2u-1, 2u (keys 32u-16 .. 32u+15, V rows of the step); an output block needs the score
+    // block 8 keys before it and the one 8 keys after it, so the packed scores of block 2u-1
+    // are carried from the previous step.
+    // Staging registers: every thread holds its 16-byte chunks of K / V rows two steps ahead.
+    // The rows are clamped into the sequence, so loads past the last step are harmless.
+    u32x4 kr[N_LD], vr[N_LD];
+    auto load_step = [&](int u) {
+#pragma unroll
+        for (int i = 0; i < N_LD; ++i) {
+            const int c = tid + i * NW * 64, row = c / CPR, cc = c % CPR;
+            kr[i] = load_row16_clamped<D>(Kb, 32 * u - 8 + row, p.Nk, cc * 8);
+            vr[i] = load_row16_clamped<D>(Vb, 32 * u - 16 + row, p.Nk, cc * 8);
+        }
+    };
+    auto stage_step = [&](int u) {  // rows outside the sequence count as zeros
+        unsigned char *Ks = smem + (u & 1) * Lds::buf_bytes, *Vs = Ks + Lds::k_bytes;
+        if (u == 0 || 32 * u + 24 > p.Nk) {
+#pragma unroll
+            for (int i = 0; i < N_LD; ++i) {
+                const int row = (tid + i * NW * 64) / CPR;
+                const int krow = 32 * u - 8 + row, vrow = 32 * u - 16 + row;
+                kr[i] = zero_unless(krow >= 0 && krow < p.Nk, kr[i]);
+                vr[i] = zero_unless(vrow >= 0 && vrow < p.Nk, vr[i]);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < N_LD; ++i) {
+            const int c = tid + i * NW * 64, row = c / CPR, cc = c % CPR;
+            *reinterpret_cast<u32x4 *>(Ks + row * KST + cc * 16) = kr[i];
+            *reinterpret_cast<u32x4 *>(Vs + row * KST + cc * 16) = vr[i];
+        }
+    };
+
+    // packed fp16 scores of the last score block of the previous step:
+    // carry[f][dword] = row base + 2n + f, keys 4g .. 4g+3 of the block
+    unsigned int carry[2][2] = {{0u, 0u}, {0u, 0u}};
+
+    // One step of the wave; EDGE = the step touches the diagonal or an end of the keys
+    // (wave-uniform), only then are the masks evaluated.
+    auto step = [&](int u, auto edge_tag) {
+        constexpr bool EDGE = decltype(edge_tag)::value;
+        const unsigned char *Ks = smem + (u & 1) * Lds::buf_bytes, *Vs = Ks + Lds::k_bytes;
+        const int jk = 32 * u - 8, jv = 32 * u - 16;
+        f32x4 c[2][2];
+        bf16x8 kf[2][KS];
+        unsigned int pd[2][2][2];  // [score block of the step][f][dword]
+        auto load_kf = [&](int blk) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+                kf[blk][ks] = *reinterpret_cast<const bf16x8 *>(Ks + (blk * 16 + n) * KST + (ks * 32 + g * 8) * 2);
+        };
+        load_kf(0);
+        load_kf(1);
+        static_for<2>([&](auto BL) {
+            constexpr int blk = decltype(BL)::value;
+            // ---- S^T = K Q^T (raw), pre-mask, clamp, pack two keys per dword ----
+            f32x4 acc[2];
+#pragma unroll
+            for (int f = 0; f < 2; ++f) acc[f] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                for (int f = 0; f < 2; ++f) acc[f] = mfma_bf16(kf[blk][ks], qf[f][ks], acc[f]);
+            const int key0 = jk + blk * 16 + 4 * g;
+#pragma unroll
+            for (int f = 0; f < 2; ++f) {
+                if constexpr (EDGE) {
+                    if (causal) {
+                        const int qpos = base + 2 * n + f;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            if (key0 + r > qpos) acc[f][r] = 0.f;
+                    }
+                }
+                f16x4 hv;
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    hv[r] = (_Float16)__builtin_amdgcn_fmed3f(acc[f][r], -kF16Max, kF16Max);
+                const auto two = __builtin_bit_cast(u32x2, hv);
+                pd[blk][f][0] = two[0];
+                pd[blk][f][1] = two[1];
+            }
+            // ---- convolution of output block blk: one B operand per row offset
+            //      delta = (output row parity) + (tap slot) - (CQT-1): rows base + 2n + delta =
+            //      fragment f shifted s lanes down (zeros shifted in: those lanes are halo rows,
+            //      whose outputs are not used); k slots 0..3 of a lane group from the score block
+            //      before, 4..7 from this one ----
+#pragma unroll
+            for (int ob = 0; ob < 2; ++ob) c[ob][blk] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            static_for<CQT + 1>([&](auto DL) {
+                constexpr int delta = decltype(DL)::value - (CQT - 1);
+                constexpr int f = delta & 1, s = (f - delta) / 2;
+                u32x4 bv;
+#pragma unroll
+                for (int half = 0; half < 2; ++half)
+#pragma unroll
+                    for (int dw = 0; dw < 2; ++dw) {
+                        const unsigned int own = half ? pd[blk][f][dw] : (blk ? pd[0][f][dw] : carry[f][dw]);
+                        if constexpr (s == 0) bv[2 * half + dw] = own;
+                        else bv[2 * half + dw] = dpp_zero<0x110 + s>(own);
+                    }
+                constexpr int t0 = delta + (CQT - 1);  // tap slot of output parity 0
+                if constexpr (t0 < CQT) c[0][blk] = mfma_f16(tf[t0], __builtin_bit_cast(f16x8, bv), c[0][blk]);
+                if constexpr (t0 >= 1) c[1][blk] = mfma_f16(tf[t0 - 1], __builtin_bit_cast(f16x8, bv), c[1][blk]);
+            });
+        });
+#pragma unroll
+        for (int f = 0; f < 2; ++f)
+#pragma unroll
+            for (int dw = 0; dw < 2; ++dw) carry[f][dw] = pd[1][f][dw];
+
+        // ---- post-mask and softmax numerators (log2 domain).  The exponent base m_ref of a row
+        //      only follows the row's maximum when some score exceeds it by more than kMaxSlack
+        //      (then every lane group of the wave exchanges its maxima and rescales); otherwise no
+        //      lane talks to another.  The true maximum is tracked per lane for the M output. ----
+        float mloc[2];
+#pragma unroll
+        for (int ob = 0; ob < 2; ++ob) {
+            if constexpr (EDGE) {
+                const int qpos = base + 2 * n + ob;
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int key = jv + kb * 16 + 4 * g + r;
+                        if (key < 0 || key >= p.Nk || (causal && key > qpos)) c[ob][kb][r] = kNegInf;
+                    }
+            }
+            float mx = kNegInf;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) mx = fmaxf(mx, c[ob][kb][r]);
+            mloc[ob] = mx;
+            m_true[ob] = fmaxf(m_true[ob], mx);
+        }
+        if (__builtin_amdgcn_ballot_w64(mloc[0] > m_ref[0] + kMaxSlack || mloc[1] > m_ref[1] + kMaxSlack) != 0) {
+#pragma unroll
+            for (int ob = 0; ob < 2; ++ob) {
+                float mx = mloc[ob];
+                mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+                mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+                const float m_new = fmaxf(m_ref[ob], mx);
+                // rows with nothing visible yet keep m = -inf; 0 is the exponent base there
+                const float alpha = fast_exp2(m_ref[ob] - ((m_new == kNegInf) ? 0.f : m_new));
+                m_ref[ob] = m_new;
+                l_run[ob] *= alpha;
+#pragma unroll
+                for (int db = 0; db < DB; ++db) acc_o[ob][db] *= alpha;
+            }
+        }
+#pragma unroll
+        for (int ob = 0; ob < 2; ++ob) {
+            const float m_use = (m_ref[ob] == kNegInf) ? 0.f : m_ref[ob];
+            float psum = 0.f;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    float e = fast_exp2(c[ob][kb][r] - m_use);
+                    c[ob][kb][r] = e;
+                    psum += e;
+                }
+            l_run[ob] += psum;
+        }
+        // ---- O^T += V^T P^T: V^T fragments through the LDS transpose read, P^T straight from
+        //      the softmax registers (k slot 8g+e <-> key 4g+e of output block 0 for e < 4, of
+        //      output block 1 for e >= 4) ----
+        bf16x8 pf[2];
+#pragma unroll
+        for (int ob = 0; ob < 2; ++ob)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                pf[ob][r] = (bf16_t)c[ob][0][r];
+                pf[ob][4 + r] = (bf16_t)c[ob][1][r];
+            }
+        bf16x8 vf[2];
+        auto load_vf = [&](int buf, int db) {
+            bf16x4 lo = lds_read_tr4x16(Vs, KST, 4 * g, db * 16, n);
+            bf16x4 hi = lds_read_tr4x16(Vs, KST, 16 + 4 * g, db * 16, n);
+            vf[buf] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        };
+        load_vf(0, 0);
+        SCHED_DS_READ(2);
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+            if (db + 1 < DB) {
+                load_vf((db + 1) & 1, db + 1);
+                SCHED_DS_READ(2);
+            }
+#pragma unroll
+            for (int ob = 0; ob < 2; ++ob) acc_o[ob][db] = mfma_bf16(vf[db & 1], pf[ob], acc_o[ob][db]);
+            SCHED_MFMA(2);
+        }
+    };
+
+    const int k_end = causal ? min(p.Nk, i0 + BQ) : p.Nk;
+    const int n_steps = (k_end + 16 + BK - 1) / BK;
+    load_step(0);
+    stage_step(0);
+    load_step(1);
+#pragma unroll 1
+    for (int u = 0; u < n_steps; ++u) {
+        __syncthreads();  // step u-1 is done everywhere: its buffer is free, and step u's is written
+        stage_step(u + 1);
+        load_step(u + 2);
+        const int jk = 32 * u - 8, jv = 32 * u - 16;
+        if (causal && jv > i0w + WR - 1) {
+            // every output key of the step is after this wave's rows
+        } else if (u == 0 || (causal && jk + 31 > base) || jk + 32 > p.Nk) {
+            step(u, std::true_type{});
+        } else {
+            step(u, std::false_type{});
+        }
+    }
+
+    // ---- epilogue: finish the row sums and maxima, normalise, store O, M, L ----
+#pragma unroll
+    for (int ob = 0; ob < 2; ++ob) {
+        float l = l_run[ob];
+        l += __shfl_xor(l, 16, kWave);
+        l += __shfl_xor(l, 32, kWave);
+        float mt = m_true[ob];
+        mt = fmaxf(mt, __shfl_xor(mt, 16, kWave));
+        mt = fmaxf(mt, __shfl_xor(mt, 32, kWave));
+        const int qpos = base + 2 * n + ob;
+        if (qpos >= i0w && qpos < p.Nq) {
+            const float inv = 1.f / l;
+            TO *orow = O + (bh * p.Nq + qpos) * D;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                const int col = db * 16 + 4 * g;
+                if constexpr (sizeof(TO) == 2) {
+                    bf16x4 ov;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) ov[r] = (bf16_t)(acc_o[ob][db][r] * inv);
+                    *reinterpret_cast<bf16x4 *>(orow + col) = ov;
+                } else {
+                    f32x4 ov = acc_o[ob][db] * inv;
+                    *reinterpret_cast<f32x4 *>(orow + col) = ov;
+                }
+            }
+            if (g == 0) {
+                M[bh * p.Nq + qpos] = mt * (1.f / kLog2e);
+                L[bh * p.Nq + qpos] = l * fast_exp2(m_ref[ob] - mt);
+            }
+        }
+    }
+}
+
+template <int D, int CQT, typename TO>
+hipError_t launch_fwd(const Problem &p, const void *q, const void *k, const void *v, const float *w,
+                      void *o, float *m, float *l, hipStream_t s) {
+    auto kern = fwd_reg_mfma_kernel<D, CQT, TO>;
+    constexpr int lds = FwdLds<D>::total;
+    if (lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) return e;
+    }
+    constexpr int BQ = NW * wave_rows(CQT);
+    dim3 grid(p.H, p.B, (p.Nq + BQ - 1) / BQ);
+    kern<<<grid, NW * 64, lds, s>>>(p, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, w,
+                                    (TO *)o, m, l);
+    return hipGetLastError();
+}
+
+template <int D, typename TO>
+hipError_t pick_cq(const Problem &p, const void *q, const void *k, const void *v, const float *w,
+                   void *o, float *m, float *l, hipStream_t s) {
+    if (p.c_q <= 3) return launch_fwd<D, 3, TO>(p, q, k, v, w, o, m, l, s);
+    if (p.c_q <= kMfmaFwdRegMaxCq) return launch_fwd<D, 6, TO>(p, q, k, v, w, o, m, l, s);
+    return hipErrorInvalidValue;
+}
+
+}  // namespace
+
+hipError_t mfma_fwd_reg(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
+                    const float *w, void *o, float *m, float *l, hipStream_t s) {
+    if (p.d == 128) {
+        if (out_dt == CONVATTN_BF16) return pick_cq<128, bf16_t>(p, q, k, v, w, o, m, l, s);
+        return pick_cq<128, float>(p, q, k, v, w, o, m, l, s);
+    }
+    if (out_dt == CONVATTN_BF16) return pick_cq<64, bf16_t>(p, q, k, v, w, o, m, l, s);
+    return pick_cq<64, float>(p, q, k, v, w, o, m, l, s);
+}
+
+}  // namespace convattn

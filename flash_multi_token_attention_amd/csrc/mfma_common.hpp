@@ -166,7 +166,10 @@ inline bool mfma_bwd_shape_ok(const Problem &p, int in_dt, unsigned flags) {
 }
 
 // ---- bf16 MFMA kernels ----
-constexpr int kMfmaFwdRows = 128;  // query rows per forward workgroup
+// mfma_fwd runs the register-resident kernel (fwd_reg_mfma.hip) up to this many query taps
+constexpr int kMfmaFwdRegMaxCq = 6;
+hipError_t mfma_fwd_reg(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
+                        const float *w, void *o, float *m, float *l, hipStream_t s);
 hipError_t mfma_fwd(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
                     const float *w, void *o, float *m, float *l, hipStream_t s);
 
