@@ -366,7 +366,9 @@ hipError_t pick_cq(const Problem &p, const void *q, const void *k, const void *v
 
 hipError_t mfma_fwd(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
                     const float *w, void *o, float *m, float *l, hipStream_t s) {
-    if (p.c_q <= kMfmaFwdRegMaxCq) return mfma_fwd_reg(p, out_dt, q, k, v, w, o, m, l, s);
+    // (its buffer descriptors count bytes in 32 bits)
+    if (p.c_q <= kMfmaFwdRegMaxCq && (size_t)p.Nk * p.d * 2 < (1ull << 31))
+        return mfma_fwd_reg(p, out_dt, q, k, v, w, o, m, l, s);
     if (p.d == 128) {
         if (out_dt == CONVATTN_BF16) return pick_cq<128, bf16_t>(p, q, k, v, w, o, m, l, s);
         return pick_cq<128, float>(p, q, k, v, w, o, m, l, s);

@@ -61,7 +61,7 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
     constexpr int CPR = D / 8;   // 16-byte chunks per row
     constexpr int WR = wave_rows(CQT), BQ = NW * WR;
     constexpr int N_LD = BK * CPR / (NW * 64);  // 16-byte chunks per thread and matrix
-    static_assert(BK * CPR % (NW * 64) == 0, "whole chunks per thread");
+    static_assert(BK * CPR % (NW * 64) == 0 && (NW * 64) % CPR == 0, "whole chunks per thread, whole rows per pass");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
     const int tid = threadIdx.x;
@@ -129,27 +129,23 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
     // block 8 keys before it and the one 8 keys after it, so the packed scores of block 2u-1
     // are carried from the previous step.
     // Staging registers: every thread holds its 16-byte chunks of K / V rows two steps ahead.
-    // The rows are clamped into the sequence, so loads past the last step are harmless.
     u32x4 kr[N_LD], vr[N_LD];
+    // Buffer loads: rows before the first or after the last key are outside the descriptor's
+    // range and read as zeros, which is what the window's zero padding asks for.
+    const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)Kb, 0, p.Nk * D * 2, 0x00020000);
+    const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)Vb, 0, p.Nk * D * 2, 0x00020000);
+    const int ld_off = ((tid / CPR) * D + (tid % CPR) * 8) * 2;  // byte offset of this thread's first chunk in a step
+    constexpr int kChunkStep = (NW * 64 / CPR) * D * 2;         // and from one of its chunks to the next
     auto load_step = [&](int u) {
+        const int k0 = (32 * u - 8) * D * 2 + ld_off, v0 = (32 * u - 16) * D * 2 + ld_off;
 #pragma unroll
         for (int i = 0; i < N_LD; ++i) {
-            const int c = tid + i * NW * 64, row = c / CPR, cc = c % CPR;
-            kr[i] = load_row16_clamped<D>(Kb, 32 * u - 8 + row, p.Nk, cc * 8);
-            vr[i] = load_row16_clamped<D>(Vb, 32 * u - 16 + row, p.Nk, cc * 8);
+            kr[i] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, k0 + i * kChunkStep, 0, 0);
+            vr[i] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, v0 + i * kChunkStep, 0, 0);
         }
     };
-    auto stage_step = [&](int u) {  // rows outside the sequence count as zeros
+    auto stage_step = [&](int u) {
         unsigned char *Ks = smem + (u & 1) * Lds::buf_bytes, *Vs = Ks + Lds::k_bytes;
-        if (u == 0 || 32 * u + 24 > p.Nk) {
-#pragma unroll
-            for (int i = 0; i < N_LD; ++i) {
-                const int row = (tid + i * NW * 64) / CPR;
-                const int krow = 32 * u - 8 + row, vrow = 32 * u - 16 + row;
-                kr[i] = zero_unless(krow >= 0 && krow < p.Nk, kr[i]);
-                vr[i] = zero_unless(vrow >= 0 && vrow < p.Nk, vr[i]);
-            }
-        }
 #pragma unroll
         for (int i = 0; i < N_LD; ++i) {
             const int c = tid + i * NW * 64, row = c / CPR, cc = c % CPR;
@@ -169,15 +165,14 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
         const unsigned char *Ks = smem + (u & 1) * Lds::buf_bytes, *Vs = Ks + Lds::k_bytes;
         const int jk = 32 * u - 8, jv = 32 * u - 16;
         f32x4 c[2][2];
-        bf16x8 kf[2][KS];
+        bf16x8 kf[KS];  // K fragments of one score block; the second block's are read during the first's convolution
         unsigned int pd[2][2][2];  // [score block of the step][f][dword]
         auto load_kf = [&](int blk) {
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks)
-                kf[blk][ks] = *reinterpret_cast<const bf16x8 *>(Ks + (blk * 16 + n) * KST + (ks * 32 + g * 8) * 2);
+                kf[ks] = *reinterpret_cast<const bf16x8 *>(Ks + (blk * 16 + n) * KST + (ks * 32 + g * 8) * 2);
         };
         load_kf(0);
-        load_kf(1);
         static_for<2>([&](auto BL) {
             constexpr int blk = decltype(BL)::value;
             // ---- S^T = K Q^T (raw), pre-mask, clamp, pack two keys per dword ----
@@ -187,7 +182,12 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
-                for (int f = 0; f < 2; ++f) acc[f] = mfma_bf16(kf[blk][ks], qf[f][ks], acc[f]);
+                for (int f = 0; f < 2; ++f) acc[f] = mfma_bf16(kf[ks], qf[f][ks], acc[f]);
+            if constexpr (blk == 0) {
+                load_kf(1);
+                SCHED_DS_READ(KS);
+                SCHED_MFMA(2 * CQT);
+            }
             const int key0 = jk + blk * 16 + 4 * g;
 #pragma unroll
             for (int f = 0; f < 2; ++f) {
