@@ -65,7 +65,7 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
     const int tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;  // wave-uniform for the compiler too
     const int g = lane >> 4, n = lane & 15;
 
     // x = head, y = batch, z = query tile: the dispatcher hands out every (batch, head) of the
@@ -326,20 +326,28 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
     load_step(0);
     stage_step(0);
     load_step(1);
+    // Along the keys a wave's steps are: step 0 (keys before the first one to mask), steps whose
+    // keys all lie at or before its first score row (no masks), steps on the diagonal or at the
+    // end of the keys (masks), and steps entirely after its rows (it only takes part in the
+    // staging).  One loop per kind, so that each loop body has the accumulators in place.
+    auto run = [&](int ua, int ub, auto kind) {
+        constexpr int KIND = decltype(kind)::value;
 #pragma unroll 1
-    for (int u = 0; u < n_steps; ++u) {
-        __syncthreads();  // step u-1 is done everywhere: its buffer is free, and step u's is written
-        stage_step(u + 1);
-        load_step(u + 2);
-        const int jk = 32 * u - 8, jv = 32 * u - 16;
-        if (causal && jv > i0w + WR - 1) {
-            // every output key of the step is after this wave's rows
-        } else if (u == 0 || (causal && jk + 31 > base) || jk + 32 > p.Nk) {
-            step(u, std::true_type{});
-        } else {
-            step(u, std::false_type{});
+        for (int u = ua; u < ub; ++u) {
+            __syncthreads();  // step u-1 is done everywhere: its buffer is free, and step u's is written
+            stage_step(u + 1);
+            load_step(u + 2);
+            if constexpr (KIND != 2) step(u, std::integral_constant<bool, KIND == 1>{});
         }
-    }
+    };
+    const int u_diag = base < 23 ? 1 : (base - 23) / 32 + 1;    // first u >= 1 with 32u + 23 > base
+    const int u_tail = p.Nk < 24 ? 1 : (p.Nk - 24) / 32 + 1;    // first u >= 1 with 32u + 24 > Nk
+    const int u1 = min(causal ? min(u_diag, u_tail) : u_tail, n_steps);
+    const int u2 = max(u1, causal ? min((i0w + WR + 15) / 32 + 1, n_steps) : n_steps);  // 32u - 16 > i0w + WR - 1
+    run(0, 1, std::integral_constant<int, 1>{});
+    run(1, u1, std::integral_constant<int, 0>{});
+    run(u1, u2, std::integral_constant<int, 1>{});
+    run(u2, n_steps, std::integral_constant<int, 2>{});
 
     // ---- epilogue: finish the row sums and maxima, normalise, store O, M, L ----
 #pragma unroll
