@@ -122,6 +122,11 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
         for (int db = 0; db < DB; ++db) acc_o[ob][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
     float m_ref[2] = {kNegInf, kNegInf};   // exponent base of the row, in log2 units (same in the row's 4 lanes)
     float m_true[2] = {kNegInf, kNegInf};  // maximum of the scores this lane has seen
+    // The convolution accumulates on top of minus the exponent base (0 while the row has none),
+    // so its result is already the exponent; slack[ob]: how far it may go above 0 before the base
+    // is raised (-inf while the row has no base: any visible score sets one).
+    f32x4 neg_base[2] = {(f32x4){0.f, 0.f, 0.f, 0.f}, (f32x4){0.f, 0.f, 0.f, 0.f}};
+    float slack[2] = {kNegInf, kNegInf};
     float l_run[2] = {0.f, 0.f};           // this lane's share of the row sum, relative to m_ref
 
     // Step u: score blocks 2u, 2u+1 (keys 32u-8 .. 32u+23, K rows of the step) and output blocks
@@ -213,7 +218,7 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
             //      whose outputs are not used); k slots 0..3 of a lane group from the score block
             //      before, 4..7 from this one ----
 #pragma unroll
-            for (int ob = 0; ob < 2; ++ob) c[ob][blk] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            for (int ob = 0; ob < 2; ++ob) c[ob][blk] = neg_base[ob];
             static_for<CQT + 1>([&](auto DL) {
                 constexpr int delta = decltype(DL)::value - (CQT - 1);
                 constexpr int f = delta & 1, s = (f - delta) / 2;
@@ -236,6 +241,15 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
 #pragma unroll
             for (int dw = 0; dw < 2; ++dw) carry[f][dw] = pd[1][f][dw];
 
+        // V^T fragments of the first two head-dim blocks: in flight during the softmax
+        bf16x8 vf[3];
+        auto load_vf = [&](int buf, int db) {
+            bf16x4 lo = lds_read_tr4x16(Vs, KST, 4 * g, db * 16, n);
+            bf16x4 hi = lds_read_tr4x16(Vs, KST, 16 + 4 * g, db * 16, n);
+            vf[buf] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        };
+        load_vf(0, 0);
+        load_vf(1, 1);
         // ---- post-mask and softmax numerators (log2 domain).  The exponent base m_ref of a row
         //      only follows the row's maximum when some score exceeds it by more than kMaxSlack
         //      (then every lane group of the wave exchanges its maxima and rescales); otherwise no
@@ -258,33 +272,41 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) mx = fmaxf(mx, c[ob][kb][r]);
-            mloc[ob] = mx;
-            m_true[ob] = fmaxf(m_true[ob], mx);
+            mloc[ob] = mx;                                           // relative to the base
+            m_true[ob] = fmaxf(m_true[ob], mx - neg_base[ob][0]);   // absolute
         }
-        if (__builtin_amdgcn_ballot_w64(mloc[0] > m_ref[0] + kMaxSlack || mloc[1] > m_ref[1] + kMaxSlack) != 0) {
+        if (__builtin_amdgcn_ballot_w64(mloc[0] > slack[0] || mloc[1] > slack[1]) != 0) {
 #pragma unroll
             for (int ob = 0; ob < 2; ++ob) {
-                float mx = mloc[ob];
+                const float old_use = -neg_base[ob][0];
+                float mx = mloc[ob] + old_use;
                 mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
                 mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
                 const float m_new = fmaxf(m_ref[ob], mx);
                 // rows with nothing visible yet keep m = -inf; 0 is the exponent base there
-                const float alpha = fast_exp2(m_ref[ob] - ((m_new == kNegInf) ? 0.f : m_new));
+                const float new_use = (m_new == kNegInf) ? 0.f : m_new;
+                const float alpha = fast_exp2(m_ref[ob] - new_use);
+                const float delta = new_use - old_use;
                 m_ref[ob] = m_new;
+                slack[ob] = (m_new == kNegInf) ? kNegInf : kMaxSlack;
+                neg_base[ob] = (f32x4){-new_use, -new_use, -new_use, -new_use};
                 l_run[ob] *= alpha;
 #pragma unroll
                 for (int db = 0; db < DB; ++db) acc_o[ob][db] *= alpha;
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) c[ob][kb][r] -= delta;
             }
         }
 #pragma unroll
         for (int ob = 0; ob < 2; ++ob) {
-            const float m_use = (m_ref[ob] == kNegInf) ? 0.f : m_ref[ob];
             float psum = 0.f;
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    float e = fast_exp2(c[ob][kb][r] - m_use);
+                    float e = fast_exp2(c[ob][kb][r]);
                     c[ob][kb][r] = e;
                     psum += e;
                 }
@@ -301,22 +323,14 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
                 pf[ob][r] = (bf16_t)c[ob][0][r];
                 pf[ob][4 + r] = (bf16_t)c[ob][1][r];
             }
-        bf16x8 vf[2];
-        auto load_vf = [&](int buf, int db) {
-            bf16x4 lo = lds_read_tr4x16(Vs, KST, 4 * g, db * 16, n);
-            bf16x4 hi = lds_read_tr4x16(Vs, KST, 16 + 4 * g, db * 16, n);
-            vf[buf] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        };
-        load_vf(0, 0);
-        SCHED_DS_READ(2);
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
-            if (db + 1 < DB) {
-                load_vf((db + 1) & 1, db + 1);
+            if (db + 2 < DB) {
+                load_vf((db + 2) % 3, db + 2);
                 SCHED_DS_READ(2);
             }
 #pragma unroll
-            for (int ob = 0; ob < 2; ++ob) acc_o[ob][db] = mfma_bf16(vf[db & 1], pf[ob], acc_o[ob][db]);
+            for (int ob = 0; ob < 2; ++ob) acc_o[ob][db] = mfma_bf16(vf[db % 3], pf[ob], acc_o[ob][db]);
             SCHED_MFMA(2);
         }
     };
