@@ -349,3 +349,23 @@ def test_seeded_random_shapes_forward_and_both_backward_paths():
             assert max_abs(dK, ref[1]) <= TOL_BF16, case
             assert max_abs(dV, ref[2]) <= TOL_BF16, case
             assert rel_max(dW, ref[3]) <= TOL_DW_REL, case
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_forward_rising_row_maxima_and_wide_score_range(causal):
+    # Scores that grow along the keys (the softmax base of every row has to be raised again and
+    # again) on top of a wide random range (exponents tens of binary orders apart).
+    B, H, N, d, c_q, c_k = 1, 2, 300, 128, 6, 11
+    Q, K, V, _, W = rand_case(B, H, N, N, d, c_q, c_k, torch.float32, seed=33)
+    u = torch.nn.functional.normalize(torch.randn(d, generator=torch.Generator().manual_seed(1)), dim=0)
+    ramp = torch.linspace(0.0, 1.0, N)[None, None, :, None]
+    K = (K + 24.0 * ramp * u).to(torch.bfloat16)
+    Q = (Q + 5.0 * u).to(torch.bfloat16)
+    V = V.to(torch.bfloat16)
+    O_ref, M_ref, L_ref = oracle_fwd(Q, K, V, W, causal)
+    assert float(M_ref.max() - M_ref.min()) > 8.0   # the case is what it claims to be
+    O, M, L = ops.forward(Q.to(DEV), K.to(DEV), V.to(DEV), W.to(DEV), scale_of(d), c_q - 1, (c_k - 1) // 2, causal,
+                          out_dtype=torch.bfloat16)
+    assert max_abs(O, O_ref) <= TOL_BF16
+    assert max_abs(M, M_ref) <= TOL_BF16
+    assert rel_max(L, L_ref) <= TOL_BF16
