@@ -31,7 +31,6 @@ UNITS = [
     ("api.hip", "api", []),
     ("generic_kernels.hip", "generic_kernels", []),
     ("reduce_kernels.hip", "reduce_kernels", []),
-    ("fwd_mfma.hip", "fwd_mfma", []),
     ("fwd_reg_mfma.hip", "fwd_reg_mfma", []),
     ("bwd_dq_mfma.hip", "bwd_dq_mfma", VGPR_FORM),
     ("bwd_dkdv_mfma.hip", "bwd_dkdv_mfma_narrow", ["-DCONVATTN_DKDV_UNIT=0"]),

@@ -46,7 +46,7 @@ int validate(const convattn_desc *d, int op, Problem *out) {
 
 // 0 = fp32-arithmetic kernels, 1 = bf16 MFMA kernels.
 int pick_path(const convattn_desc *d, const Problem &p, int op) {
-    if (op == CONVATTN_OP_FWD) return mfma_shape_ok(p, d->in_dtype, d->flags) ? 1 : 0;
+    if (op == CONVATTN_OP_FWD) return mfma_fwd_shape_ok(p, d->in_dtype, d->flags) ? 1 : 0;
     if (op == CONVATTN_OP_BWD) return mfma_bwd_shape_ok(p, d->in_dtype, d->flags) ? 1 : 0;
     if (op == CONVATTN_OP_DECODE) return decode_stream_ok(p, d->in_dtype, d->flags) ? 1 : 0;
     return 0;

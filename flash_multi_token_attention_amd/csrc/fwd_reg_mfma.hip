@@ -1,5 +1,4 @@
-// Training forward of conv-attention on bf16 MFMA (gfx950) for windows of up to 6 query taps:
-// the scores never leave the registers.
+// Training forward of conv-attention on bf16 MFMA (gfx950): the scores never leave the registers.
 //
 // Workgroup = 4 waves of one (batch, head); a wave computes scores for 32 consecutive query rows
 // (the first CQT-1 of them only as the window's halo above its 33-CQT output rows) and keeps
@@ -418,13 +417,14 @@ template <int D, typename TO>
 hipError_t pick_cq(const Problem &p, const void *q, const void *k, const void *v, const float *w,
                    void *o, float *m, float *l, hipStream_t s) {
     if (p.c_q <= 3) return launch_fwd<D, 3, TO>(p, q, k, v, w, o, m, l, s);
-    if (p.c_q <= kMfmaFwdRegMaxCq) return launch_fwd<D, 6, TO>(p, q, k, v, w, o, m, l, s);
-    return hipErrorInvalidValue;
+    if (p.c_q <= 6) return launch_fwd<D, 6, TO>(p, q, k, v, w, o, m, l, s);
+    if (p.c_q <= 8) return launch_fwd<D, 8, TO>(p, q, k, v, w, o, m, l, s);
+    return launch_fwd<D, 11, TO>(p, q, k, v, w, o, m, l, s);
 }
 
 }  // namespace
 
-hipError_t mfma_fwd_reg(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
+hipError_t mfma_fwd(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
                     const float *w, void *o, float *m, float *l, hipStream_t s) {
     if (p.d == 128) {
         if (out_dt == CONVATTN_BF16) return pick_cq<128, bf16_t>(p, q, k, v, w, o, m, l, s);

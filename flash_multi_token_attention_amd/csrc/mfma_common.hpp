@@ -160,16 +160,17 @@ inline bool mfma_shape_ok(const Problem &p, int in_dt, unsigned flags) {
     return in_dt == CONVATTN_BF16 && !(flags & CONVATTN_FLAG_EXACT) && (p.d == 64 || p.d == 128) &&
            p.pk <= kMfmaMaxPk && p.c_q <= 11;
 }
+// The forward addresses K and V of one (batch, head) through buffer descriptors, which count
+// bytes in 32 bits.
+inline bool mfma_fwd_shape_ok(const Problem &p, int in_dt, unsigned flags) {
+    return mfma_shape_ok(p, in_dt, flags) && (size_t)p.Nk * p.d * 2 < (1ull << 31);
+}
 // The backward kernels put the key taps on one 16-wide MFMA dimension.
 inline bool mfma_bwd_shape_ok(const Problem &p, int in_dt, unsigned flags) {
     return mfma_shape_ok(p, in_dt, flags) && p.c_k <= 15;
 }
 
 // ---- bf16 MFMA kernels ----
-// mfma_fwd runs the register-resident kernel (fwd_reg_mfma.hip) up to this many query taps
-constexpr int kMfmaFwdRegMaxCq = 6;
-hipError_t mfma_fwd_reg(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
-                        const float *w, void *o, float *m, float *l, hipStream_t s);
 hipError_t mfma_fwd(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
                     const float *w, void *o, float *m, float *l, hipStream_t s);
 
