@@ -19,6 +19,8 @@ FWD_SHAPES = [
     (1, 2, 100, 64, 3, 5),
     (1, 1, 64, 128, 1, 1),
     (1, 2, 200, 64, 11, 11),
+    (1, 2, 257, 128, 8, 9),
+    (1, 1, 200, 64, 7, 7),
     (1, 1, 130, 128, 6, 17),
     (1, 2, 31, 64, 2, 3),
     (1, 1, 1, 64, 6, 11),
