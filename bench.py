@@ -194,7 +194,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; run with --gpus 1 "
-                 "(the path shards by batch/head with no exchange, see DESIGN.md)")
+                 "(the path shards by batch and head with no exchange between GPUs)")
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     dev = torch.device("cuda:0")
