@@ -4,8 +4,8 @@
 // (the first CQT-1 of them only as the window's halo above its 33-CQT output rows) and keeps
 // O^T, the row sums and the softmax bases of its rows in registers for the whole key loop.
 // Lane n of score fragment f holds row base + 2n + f.  Per 32-key step:
-//   1. all waves write the K / V rows they loaded two steps ago to the LDS buffer of the next
-//      step and issue the loads for the step after it (one barrier per step);
+//   1. all waves write the K / V rows they loaded during the previous step to the LDS buffer
+//      of the next step and issue the loads for the step after it (one barrier per step);
 //   2. S^T = K Q^T for two 16-key blocks; the accumulator layout (lane = query row, 4 keys per
 //      lane group) is, packed to fp16 after the causal pre-mask, already the B operand layout of
 //      the convolution MFMA: k slots 0..3 of a lane group come from one block, 4..7 from the next
@@ -132,7 +132,8 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
     // 2u-1, 2u (keys 32u-16 .. 32u+15, V rows of the step); an output block needs the score
     // block 8 keys before it and the one 8 keys after it, so the packed scores of block 2u-1
     // are carried from the previous step.
-    // Staging registers: every thread holds its 16-byte chunks of K / V rows two steps ahead.
+    // Staging registers: every thread holds its 16-byte chunks of the K / V rows of step u+2
+    // while step u is computed.
     u32x4 kr[N_LD], vr[N_LD];
     // Buffer loads: rows before the first or after the last key are outside the descriptor's
     // range and read as zeros, which is what the window's zero padding asks for.
