@@ -75,7 +75,8 @@ __global__ __launch_bounds__(NW * 64) void dq_from_ds_kernel(Problem p, const bf
             tv[i] = kt * kDsKeys < p.Nk && rt < n_rt &&
                     (!causal || kt * kDsKeys < (rt + 1) * kDsRows - kDsRowShift);  // first key <= last row of the block
             const size_t blk = (size_t)min(kt, n_kt - 1) * n_rt + min(rt, n_rt - 1);
-            tr[i] = *reinterpret_cast<const u32x4 *>(ws + blk * BLK + t_key * kDsRows + t_ch * 8);
+            // every dS block is read once: non-temporal, so that it does not push K out of the caches
+            tr[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(ws + blk * BLK + t_key * kDsRows + t_ch * 8));
         }
     };
 

@@ -24,6 +24,15 @@
 namespace convattn {
 namespace {
 
+// 8 bf16 of the row nearest to `row` inside [0, N), as a non-temporal load: every K / V row is
+// read exactly once, and keeping it out of the caches' replacement order is worth 10 % of the
+// stream's bandwidth here.
+template <int D>
+__device__ __forceinline__ u32x4 load_row16_stream(const bf16_t *__restrict__ base, int row, int N, int col) {
+    const int rr = min(max(row, 0), N - 1);
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base + (size_t)rr * D + col));
+}
+
 constexpr int NW = 4;
 constexpr int IT = 64;             // keys per wave iteration
 constexpr int SW = IT + 16;        // score strip width: 16 carried + 64 new
@@ -113,13 +122,13 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(
         for (int blk = 0; blk < 4; ++blk)
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks)
-                kreg[blk][ks] = load_row16_clamped<D>(Kb, lo + 8 + blk * 16 + n, p.Nk, ks * 32 + g * 8);
+                kreg[blk][ks] = load_row16_stream<D>(Kb, lo + 8 + blk * 16 + n, p.Nk, ks * 32 + g * 8);
 
         for (int j0 = lo; j0 < hi; j0 += IT) {
             // V of this iteration: keys j0 .. j0+63
             u32x4 vreg[VT];
 #pragma unroll
-            for (int t = 0; t < VT; ++t) vreg[t] = load_row16_clamped<D>(Vb, j0 + RPI * t + gph, p.Nk, cc * 8);
+            for (int t = 0; t < VT; ++t) vreg[t] = load_row16_stream<D>(Vb, j0 + RPI * t + gph, p.Nk, cc * 8);
 
             // scores of keys j0+8 .. j0+71 -> strip columns 16 .. 79
 #pragma unroll
@@ -148,7 +157,7 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(
                 for (int blk = 0; blk < 4; ++blk)
 #pragma unroll
                     for (int ks = 0; ks < KS; ++ks)
-                        kreg[blk][ks] = load_row16_clamped<D>(Kb, j0 + IT + 8 + blk * 16 + n, p.Nk, ks * 32 + g * 8);
+                        kreg[blk][ks] = load_row16_stream<D>(Kb, j0 + IT + 8 + blk * 16 + n, p.Nk, ks * 32 + g * 8);
             }
             __builtin_amdgcn_wave_barrier();
 
