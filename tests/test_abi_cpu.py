@@ -144,3 +144,18 @@ def test_drop_in_import_path():
     for name in ("FlashConvAttention", "FlashConvAttentionFunction", "forward", "dq_backward",
                  "dkdv_backward", "fwd_conv_attn", "dq_bwd_conv_attn", "dkdv_bwd_conv_attn"):
         assert hasattr(ca, name)
+
+
+def test_kernel_path_selection(lib):
+    # 1 = bf16 MFMA kernels, 0 = fp32-arithmetic kernels
+    assert lib.convattn_kernel_path(C.byref(desc()), _lib.OP_FWD) == 1
+    assert lib.convattn_kernel_path(C.byref(desc()), _lib.OP_BWD) == 1
+    assert lib.convattn_kernel_path(C.byref(desc(in_dtype=_lib.F32, out_dtype=_lib.F32)), _lib.OP_FWD) == 0
+    assert lib.convattn_kernel_path(C.byref(desc(flags=_lib.FLAG_EXACT)), _lib.OP_FWD) == 0
+    assert lib.convattn_kernel_path(C.byref(desc(c_k=17)), _lib.OP_FWD) == 1
+    assert lib.convattn_kernel_path(C.byref(desc(c_k=17)), _lib.OP_BWD) == 0   # backward: c_k <= 15
+    assert lib.convattn_kernel_path(C.byref(desc(c_k=19)), _lib.OP_FWD) == 0
+    # the forward addresses K / V of one (batch, head) with 32-bit byte offsets
+    big = 1 << 24
+    assert lib.convattn_kernel_path(C.byref(desc(Nq=big, Nk=big, d=64)), _lib.OP_FWD) == 0
+    assert lib.convattn_kernel_path(C.byref(desc(Nq=big - 64, Nk=big - 64, d=64)), _lib.OP_FWD) == 1
