@@ -346,9 +346,11 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
             acc_k[m][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
             acc_v[m][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
         }
-    f32x4 acc_w[4];
+    // dW: one accumulator per row of a group of RPL rows (see the dW loop)
+    constexpr int RPL = 4;
+    f32x4 acc_w[RPL];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) acc_w[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < RPL; ++i) acc_w[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
     const int bcl = n < ck ? n : ck - 1;  // dW: lanes past the last key tap re-read a valid one
     const int pq = p.pq;
     // dS workspace blocks of this pair: [key tile][row tile of 64][32 keys][64 rows]
@@ -464,14 +466,15 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
             const int boff = 8 + 8 * g - bcl + pk;
             const unsigned char *bbase = Cs + HT * CST + (boff & ~1) * 2;
             const unsigned int bsh = (boff & 1) * 16;
-            // The S operand of row i+1 is the one of row i moved down by one lane (lane n holds S row
-            // i + n - pq), so it is read from LDS once per RPL rows and shifted within the 16-lane
-            // rows in between; only lanes n < c_q matter, and (c_q - 1) + (RPL - 1) <= 15.
-            constexpr int RPL = CQT <= 6 ? 8 : 4;
+            // The S operand is read once per group of RPL rows: lane m holds S row i + m - pq, which
+            // for row i + u of the group is the row of tap a = m - u.  Row u of every group
+            // therefore accumulates into its own accumulator, whose row m belongs to tap m - u; the
+            // accumulators are added up with that shift once, after the tile loop.  Only rows
+            // m - u < c_q matter, and (c_q - 1) + (RPL - 1) <= 15.
             static_assert(BR % RPL == 0 && (CQT - 1) + (RPL - 1) <= 15, "dW row groups");
 #pragma unroll 1
             for (int i = 0; i < BR; i += RPL) {
-                u32x4 af = *reinterpret_cast<const u32x4 *>(abase + i * SST);
+                const u32x4 af = *reinterpret_cast<const u32x4 *>(abase + i * SST);
                 u32x4 bw[RPL];
                 unsigned int bx[RPL];
 #pragma unroll
@@ -486,11 +489,7 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
                     sh[1] = __builtin_amdgcn_alignbit(bw[u][2], bw[u][1], bsh);
                     sh[2] = __builtin_amdgcn_alignbit(bw[u][3], bw[u][2], bsh);
                     sh[3] = __builtin_amdgcn_alignbit(bx[u], bw[u][3], bsh);
-                    acc_w[u & 3] = mfma_f16(__builtin_bit_cast(f16x8, af), __builtin_bit_cast(f16x8, sh), acc_w[u & 3]);
-                    if (u + 1 < RPL) {
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) af[r] = lane_from_next(af[r]);
-                    }
+                    acc_w[u] = mfma_f16(__builtin_bit_cast(f16x8, af), __builtin_bit_cast(f16x8, sh), acc_w[u]);
                 }
             }
         }
@@ -529,11 +528,27 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
         }
     }
 
-    // ---- dW of this pair into its own LDS ([16][16], over the S buffer nobody reads any more) ----
+    // ---- dW of this pair into its own LDS (over the tile buffers nobody reads any more): first the
+    // RPL accumulators as [u][row m][tap b], then dW[a][b] = sum_u acc_u[a + u][b] as [16][16] ----
     float *red = reinterpret_cast<float *>(pair_base);
+    static_assert(RPL * 1024 <= 2 * Lds::pair_bytes, "room for the dW accumulators");
 #pragma unroll
-    for (int r = 0; r < 4; ++r)
-        red[(4 * g + r) * 16 + n] = (acc_w[0][r] + acc_w[1][r]) + (acc_w[2][r] + acc_w[3][r]);
+    for (int u = 0; u < RPL; ++u)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) red[u * 256 + (4 * g + r) * 16 + n] = acc_w[u][r];
+    __builtin_amdgcn_wave_barrier();
+    float dw_out[4];
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+        const int o = lane + 64 * q4, a = o >> 4;
+        float sum = 0.f;
+#pragma unroll
+        for (int u = 0; u < RPL; ++u) sum += (a + u < 16) ? red[u * 256 + o + 16 * u] : 0.f;
+        dw_out[q4] = sum;
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) red[lane + 64 * q4] = dw_out[q4];
     }  // consumer
 
     // ---- dW partial of this workgroup: ordered sum over the 4 pairs; S was raw, so * scale ----
