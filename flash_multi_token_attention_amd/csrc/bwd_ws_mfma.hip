@@ -107,16 +107,20 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
     // Staging registers: this thread's 16-byte chunks of the next Q / dO tile and its LSE / D entry.
     u32x4 qr[Q_LD], gr[G_LD];
     float ls = 0.f, dd = 0.f;
+    // Buffer loads: rows before the first or after the last query row are outside the descriptor's
+    // range and read as zeros, which is what the window's zero padding and the tail tile ask for.
+    const __amdgpu_buffer_rsrc_t q_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)Qb, 0, p.Nq * D * 2, 0x00020000);
+    const __amdgpu_buffer_rsrc_t g_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)dOb, 0, p.Nq * D * 2, 0x00020000);
     auto load_tile = [&](int r0) {
 #pragma unroll
         for (int i = 0; i < Q_LD; ++i) {
             const int c = min(tid + i * NT, Q_CH - 1), row = c / CPR, cc = c % CPR;
-            qr[i] = load_row16_clamped<D>(Qb, r0 - HT + row, p.Nq, cc * 8);
+            qr[i] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, ((r0 - HT + row) * D + cc * 8) * 2, 0, 0);
         }
 #pragma unroll
         for (int i = 0; i < G_LD; ++i) {
             const int c = min(tid + i * NT, G_CH - 1), row = c / CPR, cc = c % CPR;
-            gr[i] = load_row16_clamped<D>(dOb, r0 + row, p.Nq, cc * 8);
+            gr[i] = __builtin_amdgcn_raw_buffer_load_b128(g_rsrc, ((r0 + row) * D + cc * 8) * 2, 0, 0);
         }
         ls = 1e30f; dd = 0.f;  // rows past the end: exp2(C - LSE) = 0
         if (tid < BR && r0 + tid < p.Nq) { ls = lse_b[r0 + tid] * kLog2e; dd = dl_b[r0 + tid]; }
@@ -125,15 +129,6 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
     auto stage_tile = [&](int it, int r0) {
         unsigned char *Qs = stage_q(it & 1), *Gs = stage_g(it & 1);
         float *lse_s = stage_lse(it & 1);
-        if (r0 == 0 || r0 + BR > p.Nq) {  // rows outside the sequence count as zeros
-#pragma unroll
-            for (int i = 0; i < Q_LD; ++i) {
-                const int row = r0 - HT + (tid + i * NT) / CPR;
-                qr[i] = zero_unless(row >= 0 && row < p.Nq, qr[i]);
-            }
-#pragma unroll
-            for (int i = 0; i < G_LD; ++i) gr[i] = zero_unless(r0 + (tid + i * NT) / CPR < p.Nq, gr[i]);
-        }
 #pragma unroll
         for (int i = 0; i < Q_LD; ++i) {
             const int c = tid + i * NT, row = c / CPR, cc = c % CPR;

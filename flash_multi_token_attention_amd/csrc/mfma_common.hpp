@@ -167,7 +167,8 @@ inline bool mfma_fwd_shape_ok(const Problem &p, int in_dt, unsigned flags) {
 }
 // The backward kernels put the key taps on one 16-wide MFMA dimension.
 inline bool mfma_bwd_shape_ok(const Problem &p, int in_dt, unsigned flags) {
-    return mfma_shape_ok(p, in_dt, flags) && p.c_k <= 15;
+    // (the one-pass kernel addresses Q and dO of one (batch, head) with 32-bit byte offsets)
+    return mfma_shape_ok(p, in_dt, flags) && p.c_k <= 15 && (size_t)p.Nq * p.d * 2 < (1ull << 31);
 }
 
 // ---- bf16 MFMA kernels ----
