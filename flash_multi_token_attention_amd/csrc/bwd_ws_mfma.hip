@@ -171,7 +171,10 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
             __syncthreads();
             if (it + 1 < n_tiles) load_tile(r0 + BR);
             if (it == n_tiles || is_skipped(r0)) continue;
-            const bool edge = is_edge(r0);
+            // the tile body exists twice: with the masks (tiles on the diagonal or at an end of a
+            // sequence) and without, as straight-line code
+            auto ptile = [&](auto edge_tag) {
+            constexpr bool edge = decltype(edge_tag)::value;
             const unsigned char *Qs = stage_q(it & 1), *Gs = stage_g(it & 1);
             const float *lse_s = stage_lse(it & 1), *dl_s = lse_s + BR;
             unsigned char *Ss = pair_s(it & 1), *Cs = pair_c(it & 1), *Ps = pair_p(it & 1);
@@ -328,6 +331,9 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
                 }
                 *reinterpret_cast<bf16x8 *>(Ps + (kb * 64 + lane) * 16) = pf;
             }
+            };
+            if (is_edge(r0)) ptile(std::true_type{});
+            else ptile(std::false_type{});
         }
     } else {
     // ================================ consumer ================================
