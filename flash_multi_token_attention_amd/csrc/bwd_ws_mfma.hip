@@ -169,7 +169,8 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
             __syncthreads();
             if (it < n_tiles) stage_tile(it, r0);
             __syncthreads();
-            if (it + 1 < n_tiles) load_tile(r0 + BR);
+            load_tile(r0 + BR);  // unconditional: rows past the end read as zeros, and a conditional
+                                 // load would keep the previous tile's registers alive through the tile
             if (it == n_tiles || is_skipped(r0)) continue;
             // the tile body exists twice: with the masks (tiles on the diagonal or at an end of a
             // sequence) and without, as straight-line code
@@ -362,7 +363,7 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
         __syncthreads();
         if (it < n_tiles) stage_tile(it, r_begin + it * BR);
         __syncthreads();
-        if (it + 1 < n_tiles) load_tile(r_begin + (it + 1) * BR);
+        load_tile(r_begin + (it + 1) * BR);
         if (it == 0) continue;
         const int r0 = r_begin + (it - 1) * BR;   // the tile the producer finished in the last iteration
         if (is_skipped(r0)) continue;
@@ -380,7 +381,7 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
             for (int m = 0; m < 2; ++m) ds[ob][m] = (f32x4){0.f, 0.f, 0.f, 0.f};
         {
             constexpr int NST = NRB * CQT;  // stage = (tap slot, row block)
-            f16x8 cf[2][2];
+            f16x8 cf[3][2];  // fragments two stages ahead
             auto load_cf = [&](int b2, int st) {
                 const int a = st / NRB, ob = st % NRB;
                 const unsigned char *base = Cs + (ob * 16 + n + (CQT - 1) - a) * CST + (8 * g) * 2;
@@ -388,15 +389,16 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
                 cf[b2][1] = *reinterpret_cast<const f16x8 *>(base + 32);
             };
             load_cf(0, 0);
-            SCHED_DS_READ_ID(2, 31);
+            load_cf(1, 1);
+            SCHED_DS_READ_ID(4, 31);
 #pragma unroll
             for (int st = 0; st < NST; ++st) {
-                if (st + 1 < NST) {
-                    load_cf((st + 1) & 1, st + 1);
+                if (st + 2 < NST) {
+                    load_cf((st + 2) % 3, st + 2);
                     SCHED_DS_READ_ID(2, 31);
                 }
 #pragma unroll
-                for (int m = 0; m < 2; ++m) ds[st % NRB][m] = mfma_f16(cf[st & 1][m], tfl[st / NRB], ds[st % NRB][m]);
+                for (int m = 0; m < 2; ++m) ds[st % NRB][m] = mfma_f16(cf[st % 3][m], tfl[st / NRB], ds[st % NRB][m]);
                 SCHED_MFMA_ID(2, 31);
             }
         }
