@@ -173,7 +173,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
         }
         if (tid < BR) { lse_s[tid] = ls; dl_s[tid] = dd; }
         __syncthreads();
-        if (r0 + BR < r_end) load_tile(r0 + BR);
+        load_tile(r0 + BR);  // unconditional (rows are clamped into the sequence): a conditional load keeps the old registers alive
         if (causal && r0 + BR - 1 < c0 - 8) return;  // none of the tile's rows sees the wave's keys (only on masked tiles)
         // Past the last row only the dS / dK work of the 16 carried rows is left.
         const bool tail = EDGE && r0 >= p.Nq;

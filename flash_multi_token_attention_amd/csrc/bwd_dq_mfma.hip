@@ -157,7 +157,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_mfma_kernel(
             if (c < V_CH) *reinterpret_cast<u32x4 *>(Vs + row * RST + cc * 16) = vr[i];
         }
         __syncthreads();
-        if (c0 + BK < k_end) load_tile(c0 + BK);
+        load_tile(c0 + BK);  // unconditional (rows are clamped into the sequence): a conditional load keeps the old registers alive
         if (causal && c0 > r0 + WR - 1) continue;
         // masks matter only where the tile can reach the diagonal or the end of the keys
         const bool edge = c0 == 0 || (causal && c0 + BK + 16 > r0 - 16) || (c0 + BK + 8 > p.Nk) ||
