@@ -12,10 +12,12 @@
 //   consumer (odd waves):  keeps the dK / dV / dW accumulators; one tile behind the producer:
 //       dV^T += dO^T P, dS (rows r0-16 .. r0+15, flipped-band MFMAs over dC) -> workspace,
 //       dK^T += Q^T dS, dW += S (x) dC
-// Everything the consumer reads (Q, dO, S, dC, P of the previous tile) is double-buffered in
-// LDS; one pair of workgroup barriers per tile orders the buffers, and both roles run the same
-// number of iterations.  dS / dK trail their tile by 16 rows (they need the dC rows below), the
-// dC buffer of a tile starts with the last 16 rows of the previous one.
+// Everything the consumer reads of the previous tile is still in LDS while the producer writes the
+// next one: Q, dO and P are double-buffered, S and dC sit in rings of three 32-row slots per pair
+// (a tile's 48-row window = its own slot + the second half of the previous tile's slot, so the 16
+// rows above a tile are never copied or recomputed).  One pair of workgroup barriers per tile orders
+// the buffers, and both roles run the same number of iterations.  dS / dK trail their tile by 16
+// rows (they need the dC rows below).
 #include <type_traits>
 
 #include "mfma_common.hpp"
@@ -39,6 +41,8 @@ constexpr int NSB = S_COLS / 16;       // 4 key blocks of S
 constexpr int NCB = C_COLS / 16;       // 3 key blocks of C / dP / dC
 constexpr int NRB = BR / 16;           // 2 own row blocks per tile
 constexpr int P_BYTES = 2 * 64 * 16;   // P of a tile as two MFMA operands per lane
+constexpr int RING_ROWS = 3 * BR;      // S / dC ring of a pair: three tiles of 32 rows
+static_assert(2 * (S_ROWS * SST + C_ROWS * CST) == RING_ROWS * (SST + CST), "rings fill the pair buffers");
 static_assert(BKW == kKvKeysPerWg && WK == kDsKeys && kDsRows == 2 * BR && kDsRowShift == HT, "dS workspace layout");
 
 template <int D> struct WsLds {
@@ -75,9 +79,16 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
         return reinterpret_cast<float *>(smem + buf * Lds::stage_bytes + Lds::q_bytes + Lds::g_bytes);
     };
     unsigned char *pair_base = smem + 2 * Lds::stage_bytes + pr * 2 * Lds::pair_bytes;
-    auto pair_s = [&](int buf) { return pair_base + buf * Lds::pair_bytes; };
-    auto pair_c = [&](int buf) { return pair_base + buf * Lds::pair_bytes + S_ROWS * SST; };
-    auto pair_p = [&](int buf) { return pair_base + buf * Lds::pair_bytes + S_ROWS * SST + C_ROWS * CST; };
+    // S and dC of a pair live in rings of three 32-row slots: tile `it` writes its own 32 rows into
+    // slot it % 3, and the 16 rows above them (the last 16 of the previous tile) are the second half
+    // of slot (it - 1) % 3, where that tile left them.  Row rho of a tile's 48-row window
+    // (rho = row - (r0 - 16)) is ring row (rho < 16 ? ring_hb(it) : ring_tb(it)) + rho; the two
+    // bases differ only when the window wraps around the ring.
+    unsigned char *s_ring = pair_base;
+    unsigned char *c_ring = pair_base + RING_ROWS * SST;
+    auto ring_tb = [](int it) { return (it % 3) * BR - HT; };
+    auto ring_hb = [](int it) { return ((it + 2) % 3) * BR + HT; };
+    auto pair_p = [&](int buf) { return pair_base + RING_ROWS * (SST + CST) + buf * P_BYTES; };
 
     // x = head, y = batch, z = key tile: the first key tiles see the most rows and go first
     const int h = blockIdx.x, b = blockIdx.y;
@@ -178,29 +189,14 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
             constexpr bool edge = decltype(edge_tag)::value;
             const unsigned char *Qs = stage_q(it & 1), *Gs = stage_g(it & 1);
             const float *lse_s = stage_lse(it & 1), *dl_s = lse_s + BR;
-            unsigned char *Ss = pair_s(it & 1), *Cs = pair_c(it & 1), *Ps = pair_p(it & 1);
-
-            // the last 16 dC rows of the previous tile open this tile's buffer
-            {
-                const unsigned char *prev = pair_c((it & 1) ^ 1) + BR * CST;
-                for (int c = lane; c < HT * (CST / 16); c += 64) {
-                    const int off = (c / (CST / 16)) * CST + (c % (CST / 16)) * 16;
-                    *reinterpret_cast<u32x4 *>(Cs + off) = *reinterpret_cast<const u32x4 *>(prev + off);
-                }
-            }
+            unsigned char *Ps = pair_p(it & 1);
+            const int tb = ring_tb(it), hb = ring_hb(it);
 
             // ---- S^T tile (raw) -> fp16 LDS; Q fragments one row block ahead.  The first 16 rows
             // are the last 16 of the previous tile (masks depend on positions only): taken over from
             // the other buffer when that tile was computed. ----
             {
                 const bool carry_s = it > 0 && !is_skipped(r0 - BR);
-                if (carry_s) {
-                    const unsigned char *prev = pair_s((it & 1) ^ 1) + BR * SST;
-                    for (int c = lane; c < HT * (S_COLS / 8); c += 64) {
-                        const int off = (c / (S_COLS / 8)) * SST + (c % (S_COLS / 8)) * 16;
-                        *reinterpret_cast<u32x4 *>(Ss + off) = *reinterpret_cast<const u32x4 *>(prev + off);
-                    }
-                }
                 bf16x8 qf[2][KS];
                 auto load_qf = [&](int buf, int rb) {
 #pragma unroll
@@ -238,7 +234,7 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
 #pragma unroll
                         for (int r = 0; r < 4; ++r)
                             hv[r] = (_Float16)__builtin_amdgcn_fmed3f(acc[kb][r], -kF16Max, kF16Max);
-                        *reinterpret_cast<f16x4 *>(Ss + (rb * 16 + n) * SST + (kb * 16 + 4 * g) * 2) = hv;
+                        *reinterpret_cast<f16x4 *>(s_ring + ((rb == 0 ? hb : tb) + rb * 16 + n) * SST + (kb * 16 + 4 * g) * 2) = hv;
                     }
                 });
             }
@@ -259,12 +255,17 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
                     dp[kb] = (f32x4){0.f, 0.f, 0.f, 0.f};
                 }
                 {
-                    const unsigned char *sbase = Ss + (HT + rb * 16 + n - (CQT - 1)) * SST + (8 * g) * 2;
+                    // window row HT + rb*16 + n - (CQT-1) + a: above the tile's own rows for the first
+                    // n + a < CQT-1 taps of the first row block
+                    const int srow = HT + rb * 16 + n - (CQT - 1);
+                    const unsigned char *sbase = s_ring + (tb + srow) * SST + (8 * g) * 2;
+                    const unsigned char *sbase_h = s_ring + (hb + srow) * SST + (8 * g) * 2;
                     f16x8 sf[2][NCB];
                     auto load_sf = [&](int buf, int a) {
+                        const unsigned char *base = (rb == 0 && n + a < CQT - 1) ? sbase_h : sbase;
 #pragma unroll
                         for (int kb = 0; kb < NCB; ++kb)
-                            sf[buf][kb] = *reinterpret_cast<const f16x8 *>(sbase + a * SST + kb * 32);
+                            sf[buf][kb] = *reinterpret_cast<const f16x8 *>(base + a * SST + kb * 32);
                     };
                     load_sf(0, 0);
                     SCHED_DS_READ_ID(NCB, SID);
@@ -315,7 +316,7 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
                     }
 #pragma unroll
                     for (int r = 0; r < 4; ++r)
-                        *reinterpret_cast<_Float16 *>(Cs + (HT + rb * 16 + 4 * g + r) * CST + (kb * 16 + n) * 2) =
+                        *reinterpret_cast<_Float16 *>(c_ring + (tb + HT + rb * 16 + 4 * g + r) * CST + (kb * 16 + n) * 2) =
                             (_Float16)__builtin_amdgcn_fmed3f(dc[r], -kF16Max, kF16Max);
                     if (kb < 2) pkeep[rb][kb] = prob;
                 }
@@ -370,7 +371,8 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
         const bool edge = is_edge(r0);
         const int buf = (it - 1) & 1;
         const unsigned char *Qs = stage_q(buf), *Gs = stage_g(buf);
-        const unsigned char *Ss = pair_s(buf), *Cs = pair_c(buf), *Ps = pair_p(buf);
+        const unsigned char *Ps = pair_p(buf);
+        const int tb = ring_tb(it - 1), hb = ring_hb(it - 1);
 
         // ---- dS, rows r0-16 .. r0+15 (keys c0 .. c0+31): chains over the taps; the dC buffer
         // starts at row r0-16 ----
@@ -384,7 +386,8 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
             f16x8 cf[3][2];  // fragments two stages ahead
             auto load_cf = [&](int b2, int st) {
                 const int a = st / NRB, ob = st % NRB;
-                const unsigned char *base = Cs + (ob * 16 + n + (CQT - 1) - a) * CST + (8 * g) * 2;
+                const int crow = ob * 16 + n + (CQT - 1) - a;  // window row: above the tile's own rows if < 16
+                const unsigned char *base = c_ring + ((crow < HT ? hb : tb) + crow) * CST + (8 * g) * 2;
                 cf[b2][0] = *reinterpret_cast<const f16x8 *>(base);
                 cf[b2][1] = *reinterpret_cast<const f16x8 *>(base + 32);
             };
@@ -463,11 +466,12 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
         if (r0 < p.Nq) {
             // A: S[i + a - pq][c0 + 8g ..]        (S-tile row HT + i + a - pq, column 16 + 8g)
             // B: dC[i][c0 + 8g - b + pk ..]       (dC-tile row HT + i, column 8 + 8g - b + pk)
-            const unsigned char *abase = Ss + (HT + n - pq) * SST + (16 + 8 * g) * 2;
+            const unsigned char *abase = s_ring + (tb + HT + n - pq) * SST + (16 + 8 * g) * 2;
+            const unsigned char *abase_h = s_ring + (hb + HT + n - pq) * SST + (16 + 8 * g) * 2;
             // LDS reads at odd 2-byte offsets are slow: read 5 dwords from the even
             // element below and funnel-shift by 0 or 16 bits per lane instead.
             const int boff = 8 + 8 * g - bcl + pk;
-            const unsigned char *bbase = Cs + HT * CST + (boff & ~1) * 2;
+            const unsigned char *bbase = c_ring + (tb + HT) * CST + (boff & ~1) * 2;
             const unsigned int bsh = (boff & 1) * 16;
             // The S operand is read once per group of RPL rows: lane m holds S row i + m - pq, which
             // for row i + u of the group is the row of tap a = m - u.  Row u of every group
@@ -477,7 +481,7 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
             static_assert(BR % RPL == 0 && (CQT - 1) + (RPL - 1) <= 15, "dW row groups");
 #pragma unroll 1
             for (int i = 0; i < BR; i += RPL) {
-                const u32x4 af = *reinterpret_cast<const u32x4 *>(abase + i * SST);
+                const u32x4 af = *reinterpret_cast<const u32x4 *>((i + n < pq ? abase_h : abase) + i * SST);
                 u32x4 bw[RPL];
                 unsigned int bx[RPL];
 #pragma unroll
