@@ -12,12 +12,14 @@
 //   consumer (odd waves):  keeps the dK / dV / dW accumulators; one tile behind the producer:
 //       dV^T += dO^T P, dS (rows r0-16 .. r0+15, flipped-band MFMAs over dC) -> workspace,
 //       dK^T += Q^T dS, dW += S (x) dC
-// Everything the consumer reads of the previous tile is still in LDS while the producer writes the
-// next one: Q, dO and P are double-buffered, S and dC sit in rings of three 32-row slots per pair
-// (a tile's 48-row window = its own slot + the second half of the previous tile's slot, so the 16
-// rows above a tile are never copied or recomputed).  One pair of workgroup barriers per tile orders
-// the buffers, and both roles run the same number of iterations.  dS / dK trail their tile by 16
-// rows (they need the dC rows below).
+// One workgroup barrier per tile.  In iteration `it` every thread stages tile it+1 (Q, dO, LSE, D:
+// global loads issued an iteration earlier), the producers work on tile it and the consumers on
+// tile it-1, so three tiles are alive in LDS: Q sits in a ring of seven 16-row blocks (the 16 rows
+// above a tile are the previous tile's, never loaded twice), dO in three tile slots, S in a ring of
+// five 16-row blocks and dC in a ring of three 32-row slots per pair (a tile's 48-row window = its
+// own rows + the last 16 of the previous tile, never copied or recomputed), P in two buffers.  Both
+// roles run the same number of iterations.  dS / dK trail their tile by 16 rows (they need the dC
+// rows below).
 #include <type_traits>
 
 #include "mfma_common.hpp"
@@ -31,8 +33,8 @@ constexpr int WK = 32;                 // own keys per pair
 constexpr int BKW = NP * WK;           // 128 keys per workgroup
 constexpr int BR = 32;                 // query rows per tile
 constexpr int HT = 16;                 // rows staged above a tile's own rows (>= c_q - 1)
-constexpr int S_ROWS = BR + HT;        // 48 score rows: r0-16 .. r0+31
-constexpr int C_ROWS = BR + HT;        // 48 dC rows: 16 from the previous tile + 32 new
+constexpr int S_ROWS = BR + HT;        // 48 score rows in a tile's window: r0-16 .. r0+31
+
 constexpr int S_COLS = WK + 32;        // 64
 constexpr int C_COLS = WK + 16;        // 48
 constexpr int SST = (S_COLS + 8) * 2;  // 144
@@ -41,18 +43,19 @@ constexpr int NSB = S_COLS / 16;       // 4 key blocks of S
 constexpr int NCB = C_COLS / 16;       // 3 key blocks of C / dP / dC
 constexpr int NRB = BR / 16;           // 2 own row blocks per tile
 constexpr int P_BYTES = 2 * 64 * 16;   // P of a tile as two MFMA operands per lane
-constexpr int RING_ROWS = 3 * BR;      // S / dC ring of a pair: three tiles of 32 rows
-static_assert(2 * (S_ROWS * SST + C_ROWS * CST) == RING_ROWS * (SST + CST), "rings fill the pair buffers");
+constexpr int C_RING = 3 * BR;         // dC ring of a pair: three tiles of 32 rows
+constexpr int S_RING = 5 * 16;         // S ring of a pair: five blocks of 16 rows
+constexpr int Q_BLOCKS = 7;            // Q ring of the workgroup: seven blocks of 16 rows
 static_assert(BKW == kKvKeysPerWg && WK == kDsKeys && kDsRows == 2 * BR && kDsRowShift == HT, "dS workspace layout");
 
 template <int D> struct WsLds {
     static constexpr int RST = D * 2 + 16;
-    static constexpr int q_bytes = S_ROWS * RST;
-    static constexpr int g_bytes = BR * RST;
-    static constexpr int stat_bytes = 2 * BR * 4;
-    static constexpr int stage_bytes = q_bytes + g_bytes + stat_bytes;           // one buffer
-    static constexpr int pair_bytes = S_ROWS * SST + C_ROWS * CST + P_BYTES;      // one buffer
-    static constexpr int total = 2 * stage_bytes + NP * 2 * pair_bytes;
+    static constexpr int q_bytes = Q_BLOCKS * 16 * RST;        // Q ring
+    static constexpr int g_bytes = 3 * BR * RST;               // dO: three tile slots
+    static constexpr int stat_bytes = 2 * (2 * BR * 4);        // LSE and D of a tile: two slots
+    static constexpr int stage_bytes = q_bytes + g_bytes + stat_bytes;
+    static constexpr int pair_bytes = S_RING * SST + C_RING * CST + 2 * P_BYTES;
+    static constexpr int total = stage_bytes + NP * pair_bytes;
 };
 
 template <int D, int CQT, typename TO>
@@ -64,7 +67,7 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
     using Lds = WsLds<D>;
     constexpr int RST = Lds::RST;
     constexpr int KS = D / 32, DB = D / 16, CPR = D / 8;
-    constexpr int Q_CH = S_ROWS * CPR, G_CH = BR * CPR;
+    constexpr int Q_CH = BR * CPR, G_CH = BR * CPR;
     constexpr int Q_LD = (Q_CH + NT - 1) / NT, G_LD = (G_CH + NT - 1) / NT;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
@@ -73,22 +76,29 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
     const int g = lane >> 4, n = lane & 15;
     const bool producer = (wave & 1) == 0;   // (measured: this assignment beats waves 0-3 / 4-7)
     const int pr = wave >> 1;
-    auto stage_q = [&](int buf) { return smem + buf * Lds::stage_bytes; };
-    auto stage_g = [&](int buf) { return smem + buf * Lds::stage_bytes + Lds::q_bytes; };
-    auto stage_lse = [&](int buf) {
-        return reinterpret_cast<float *>(smem + buf * Lds::stage_bytes + Lds::q_bytes + Lds::g_bytes);
+    // Rows are numbered in blocks of 16 from row r_begin - 16: tile t owns blocks 2t+1 and 2t+2, and
+    // its 48-row window (the 16 rows above it included) is blocks 2t .. 2t+2.  In iteration `it` the
+    // workgroup stages tile it+1, the producers work on tile it and the consumers on tile it-1, so
+    // blocks 2it-2 .. 2it+4 of Q (seven), tiles it-1 .. it+1 of dO (three) and blocks 2it-2 .. 2it+2
+    // of S (five) are alive between two barriers; dC, which the consumer reads as rows of tile it-1
+    // and the half tile above it, has a ring of three tile slots.
+    auto q_block = [&](int blk) { return smem + (blk % Q_BLOCKS) * (16 * RST); };
+    auto stage_g = [&](int t) { return smem + Lds::q_bytes + (t % 3) * (BR * RST); };
+    auto stage_lse = [&](int t) {
+        return reinterpret_cast<float *>(smem + Lds::q_bytes + Lds::g_bytes + (t & 1) * (2 * BR * 4));
     };
-    unsigned char *pair_base = smem + 2 * Lds::stage_bytes + pr * 2 * Lds::pair_bytes;
-    // S and dC of a pair live in rings of three 32-row slots: tile `it` writes its own 32 rows into
-    // slot it % 3, and the 16 rows above them (the last 16 of the previous tile) are the second half
-    // of slot (it - 1) % 3, where that tile left them.  Row rho of a tile's 48-row window
-    // (rho = row - (r0 - 16)) is ring row (rho < 16 ? ring_hb(it) : ring_tb(it)) + rho; the two
-    // bases differ only when the window wraps around the ring.
+    unsigned char *pair_base = smem + Lds::stage_bytes + pr * Lds::pair_bytes;
     unsigned char *s_ring = pair_base;
-    unsigned char *c_ring = pair_base + RING_ROWS * SST;
-    auto ring_tb = [](int it) { return (it % 3) * BR - HT; };
-    auto ring_hb = [](int it) { return ((it + 2) % 3) * BR + HT; };
-    auto pair_p = [&](int buf) { return pair_base + RING_ROWS * (SST + CST) + buf * P_BYTES; };
+    unsigned char *c_ring = pair_base + S_RING * SST;
+    // S: ring row of window row rho of tile t is (32 t + rho) mod 80; with base = 32 t mod 80 and
+    // rho < 80 that is the unsigned minimum of base + rho and base + rho - 80.
+    auto s_base = [](int t) { return (t % 5) * 32 % S_RING; };
+    auto s_row = [](int base, int rho) { return (int)min((unsigned)(base + rho), (unsigned)(base + rho - S_RING)); };
+    // dC: row rho of a tile's window is ring row (rho < 16 ? ring_hb(t) : ring_tb(t)) + rho; the two
+    // bases differ only when the window wraps around the ring.
+    auto ring_tb = [](int t) { return (t % 3) * BR - HT; };
+    auto ring_hb = [](int t) { return ((t + 2) % 3) * BR + HT; };
+    auto pair_p = [&](int buf) { return pair_base + S_RING * SST + C_RING * CST + buf * P_BYTES; };
 
     // x = head, y = batch, z = key tile: the first key tiles see the most rows and go first
     const int h = blockIdx.x, b = blockIdx.y;
@@ -102,8 +112,8 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
     const float *dl_b = Dl + bh * p.Nq;
 
     // no dC before the first tile, and nothing but zeros where a tile was skipped
-    for (int c = tid; c < NP * 2 * Lds::pair_bytes / 16; c += NT)
-        *reinterpret_cast<u32x4 *>(smem + 2 * Lds::stage_bytes + c * 16) = (u32x4){0u, 0u, 0u, 0u};
+    for (int c = tid; c < NP * Lds::pair_bytes / 16; c += NT)
+        *reinterpret_cast<u32x4 *>(smem + Lds::stage_bytes + c * 16) = (u32x4){0u, 0u, 0u, 0u};
 
     // Causal: rows before the first key this workgroup touches (k0 - 8) see none of its keys.
     const int r_begin = causal ? (max(0, k0 - 8) / BR) * BR : 0;
@@ -126,7 +136,7 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
 #pragma unroll
         for (int i = 0; i < Q_LD; ++i) {
             const int c = min(tid + i * NT, Q_CH - 1), row = c / CPR, cc = c % CPR;
-            qr[i] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, ((r0 - HT + row) * D + cc * 8) * 2, 0, 0);
+            qr[i] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, ((r0 + row) * D + cc * 8) * 2, 0, 0);
         }
 #pragma unroll
         for (int i = 0; i < G_LD; ++i) {
@@ -136,14 +146,14 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
         ls = 1e30f; dd = 0.f;  // rows past the end: exp2(C - LSE) = 0
         if (tid < BR && r0 + tid < p.Nq) { ls = lse_b[r0 + tid] * kLog2e; dd = dl_b[r0 + tid]; }
     };
-    // Both roles: between the two barriers of iteration `it`, write tile `it` into buffer it & 1.
-    auto stage_tile = [&](int it, int r0) {
-        unsigned char *Qs = stage_q(it & 1), *Gs = stage_g(it & 1);
-        float *lse_s = stage_lse(it & 1);
+    // Both roles: the registers of tile t into its Q blocks, dO slot and LSE / D slot.
+    auto stage_tile = [&](int t) {
+        unsigned char *Q1 = q_block(2 * t + 1), *Q2 = q_block(2 * t + 2), *Gs = stage_g(t);
+        float *lse_s = stage_lse(t);
 #pragma unroll
         for (int i = 0; i < Q_LD; ++i) {
             const int c = tid + i * NT, row = c / CPR, cc = c % CPR;
-            if (c < Q_CH) *reinterpret_cast<u32x4 *>(Qs + row * RST + cc * 16) = qr[i];
+            if (c < Q_CH) *reinterpret_cast<u32x4 *>((row < 16 ? Q1 : Q2) + (row & 15) * RST + cc * 16) = qr[i];
         }
 #pragma unroll
         for (int i = 0; i < G_LD; ++i) {
@@ -153,8 +163,18 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
         if (tid < BR) { lse_s[tid] = ls; lse_s[BR + tid] = dd; }
     };
 
+    // Q rows r_begin-16 .. r_begin-1 (block 0), then tile 0; tile 1 waits in the registers
+    for (int c = tid; c < 16 * CPR; c += NT) {
+        const int row = c / CPR, cc = c % CPR;
+        *reinterpret_cast<u32x4 *>(q_block(0) + row * RST + cc * 16) =
+            __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, ((r_begin - HT + row) * D + cc * 8) * 2, 0, 0);
+    }
     load_tile(r_begin);
-    __syncthreads();  // zero-filled pair buffers
+    stage_tile(0);
+    load_tile(r_begin + BR);
+    // One barrier per iteration: it makes tile `it` (staged in the previous iteration) and the
+    // previous tile's S / dC / P visible, and frees what iteration it-1 read.  The first one also
+    // covers the zero-filled pair buffers.
 
     if (producer) {
         // ================================ producer ================================
@@ -178,19 +198,18 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
         for (int it = 0; it <= n_tiles; ++it) {
             const int r0 = r_begin + it * BR;
             __syncthreads();
-            if (it < n_tiles) stage_tile(it, r0);
-            __syncthreads();
-            load_tile(r0 + BR);  // unconditional: rows past the end read as zeros, and a conditional
-                                 // load would keep the previous tile's registers alive through the tile
+            if (it + 1 < n_tiles) stage_tile(it + 1);
+            load_tile(r0 + 2 * BR);  // unconditional: rows past the end read as zeros, and a conditional
+                                     // load would keep the previous tile's registers alive through the tile
             if (it == n_tiles || is_skipped(r0)) continue;
             // the tile body exists twice: with the masks (tiles on the diagonal or at an end of a
             // sequence) and without, as straight-line code
             auto ptile = [&](auto edge_tag) {
             constexpr bool edge = decltype(edge_tag)::value;
-            const unsigned char *Qs = stage_q(it & 1), *Gs = stage_g(it & 1);
-            const float *lse_s = stage_lse(it & 1), *dl_s = lse_s + BR;
+            const unsigned char *Gs = stage_g(it);
+            const float *lse_s = stage_lse(it), *dl_s = lse_s + BR;
             unsigned char *Ps = pair_p(it & 1);
-            const int tb = ring_tb(it), hb = ring_hb(it);
+            const int tb = ring_tb(it), sb = s_base(it);
 
             // ---- S^T tile (raw) -> fp16 LDS; Q fragments one row block ahead.  The first 16 rows
             // are the last 16 of the previous tile (masks depend on positions only): taken over from
@@ -201,7 +220,7 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
                 auto load_qf = [&](int buf, int rb) {
 #pragma unroll
                     for (int ks = 0; ks < KS; ++ks)
-                        qf[buf][ks] = *reinterpret_cast<const bf16x8 *>(Qs + (rb * 16 + n) * RST + (ks * 32 + g * 8) * 2);
+                        qf[buf][ks] = *reinterpret_cast<const bf16x8 *>(q_block(2 * it + rb) + n * RST + (ks * 32 + g * 8) * 2);
                 };
                 load_qf(0, 0);
                 SCHED_DS_READ_ID(KS, 10);
@@ -234,7 +253,7 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
 #pragma unroll
                         for (int r = 0; r < 4; ++r)
                             hv[r] = (_Float16)__builtin_amdgcn_fmed3f(acc[kb][r], -kF16Max, kF16Max);
-                        *reinterpret_cast<f16x4 *>(s_ring + ((rb == 0 ? hb : tb) + rb * 16 + n) * SST + (kb * 16 + 4 * g) * 2) = hv;
+                        *reinterpret_cast<f16x4 *>(s_ring + s_row(sb, rb * 16 + n) * SST + (kb * 16 + 4 * g) * 2) = hv;
                     }
                 });
             }
@@ -255,17 +274,14 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
                     dp[kb] = (f32x4){0.f, 0.f, 0.f, 0.f};
                 }
                 {
-                    // window row HT + rb*16 + n - (CQT-1) + a: above the tile's own rows for the first
-                    // n + a < CQT-1 taps of the first row block
+                    // tap a reads window row HT + rb*16 + n - (CQT-1) + a
                     const int srow = HT + rb * 16 + n - (CQT - 1);
-                    const unsigned char *sbase = s_ring + (tb + srow) * SST + (8 * g) * 2;
-                    const unsigned char *sbase_h = s_ring + (hb + srow) * SST + (8 * g) * 2;
                     f16x8 sf[2][NCB];
                     auto load_sf = [&](int buf, int a) {
-                        const unsigned char *base = (rb == 0 && n + a < CQT - 1) ? sbase_h : sbase;
+                        const unsigned char *base = s_ring + s_row(sb, srow + a) * SST + (8 * g) * 2;
 #pragma unroll
                         for (int kb = 0; kb < NCB; ++kb)
-                            sf[buf][kb] = *reinterpret_cast<const f16x8 *>(base + a * SST + kb * 32);
+                            sf[buf][kb] = *reinterpret_cast<const f16x8 *>(base + kb * 32);
                     };
                     load_sf(0, 0);
                     SCHED_DS_READ_ID(NCB, SID);
@@ -362,17 +378,16 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
 
     for (int it = 0; it <= n_tiles; ++it) {
         __syncthreads();
-        if (it < n_tiles) stage_tile(it, r_begin + it * BR);
-        __syncthreads();
-        load_tile(r_begin + (it + 1) * BR);
+        if (it + 1 < n_tiles) stage_tile(it + 1);
+        load_tile(r_begin + (it + 2) * BR);
         if (it == 0) continue;
         const int r0 = r_begin + (it - 1) * BR;   // the tile the producer finished in the last iteration
         if (is_skipped(r0)) continue;
         const bool edge = is_edge(r0);
-        const int buf = (it - 1) & 1;
-        const unsigned char *Qs = stage_q(buf), *Gs = stage_g(buf);
-        const unsigned char *Ps = pair_p(buf);
-        const int tb = ring_tb(it - 1), hb = ring_hb(it - 1);
+        // the Q rows of this tile's dS (r0-16 .. r0+15) are blocks 2(it-1) and 2(it-1)+1
+        const unsigned char *Qa = q_block(2 * (it - 1)), *Qb2 = q_block(2 * (it - 1) + 1), *Gs = stage_g(it - 1);
+        const unsigned char *Ps = pair_p((it - 1) & 1);
+        const int tb = ring_tb(it - 1), hb = ring_hb(it - 1), sb = s_base(it - 1);
 
         // ---- dS, rows r0-16 .. r0+15 (keys c0 .. c0+31): chains over the taps; the dC buffer
         // starts at row r0-16 ----
@@ -438,8 +453,8 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
             for (int kb = 0; kb < 2; ++kb) pf[kb] = *reinterpret_cast<const bf16x8 *>(Ps + (kb * 64 + lane) * 16);
             bf16x8 qt[2], gt[2];
             auto load_qg = [&](int b2, int db) {
-                bf16x4 lo = lds_read_tr4x16(Qs, RST, 4 * g, db * 16, n);
-                bf16x4 hi = lds_read_tr4x16(Qs, RST, 16 + 4 * g, db * 16, n);
+                bf16x4 lo = lds_read_tr4x16(Qa, RST, 4 * g, db * 16, n);
+                bf16x4 hi = lds_read_tr4x16(Qb2, RST, 4 * g, db * 16, n);
                 qt[b2] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
                 lo = lds_read_tr4x16(Gs, RST, 4 * g, db * 16, n);
                 hi = lds_read_tr4x16(Gs, RST, 16 + 4 * g, db * 16, n);
@@ -466,8 +481,7 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
         if (r0 < p.Nq) {
             // A: S[i + a - pq][c0 + 8g ..]        (S-tile row HT + i + a - pq, column 16 + 8g)
             // B: dC[i][c0 + 8g - b + pk ..]       (dC-tile row HT + i, column 8 + 8g - b + pk)
-            const unsigned char *abase = s_ring + (tb + HT + n - pq) * SST + (16 + 8 * g) * 2;
-            const unsigned char *abase_h = s_ring + (hb + HT + n - pq) * SST + (16 + 8 * g) * 2;
+            const unsigned char *abase = s_ring + (16 + 8 * g) * 2;
             // LDS reads at odd 2-byte offsets are slow: read 5 dwords from the even
             // element below and funnel-shift by 0 or 16 bits per lane instead.
             const int boff = 8 + 8 * g - bcl + pk;
@@ -481,7 +495,7 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
             static_assert(BR % RPL == 0 && (CQT - 1) + (RPL - 1) <= 15, "dW row groups");
 #pragma unroll 1
             for (int i = 0; i < BR; i += RPL) {
-                const u32x4 af = *reinterpret_cast<const u32x4 *>((i + n < pq ? abase_h : abase) + i * SST);
+                const u32x4 af = *reinterpret_cast<const u32x4 *>(abase + s_row(sb, HT + n - pq + i) * SST);
                 u32x4 bw[RPL];
                 unsigned int bx[RPL];
 #pragma unroll
@@ -538,7 +552,7 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
     // ---- dW of this pair into its own LDS (over the tile buffers nobody reads any more): first the
     // RPL accumulators as [u][row m][tap b], then dW[a][b] = sum_u acc_u[a + u][b] as [16][16] ----
     float *red = reinterpret_cast<float *>(pair_base);
-    static_assert(RPL * 1024 <= 2 * Lds::pair_bytes, "room for the dW accumulators");
+    static_assert(RPL * 1024 <= Lds::pair_bytes, "room for the dW accumulators");
 #pragma unroll
     for (int u = 0; u < RPL; ++u)
 #pragma unroll
@@ -566,7 +580,7 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
         float sum = 0.f;
 #pragma unroll
         for (int w = 0; w < NP; ++w)
-            sum += reinterpret_cast<const float *>(smem + 2 * Lds::stage_bytes + w * 2 * Lds::pair_bytes)[a * 16 + bb];
+            sum += reinterpret_cast<const float *>(smem + Lds::stage_bytes + w * Lds::pair_bytes)[a * 16 + bb];
         dW_part[(bh * gridDim.z + blockIdx.z) * ntap + tid] = sum * p.scale;
     }
 }
