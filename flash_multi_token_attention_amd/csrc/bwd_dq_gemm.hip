@@ -6,8 +6,8 @@
 // 64 keys the workgroup stages the K rows (row-major) and the four dS blocks (as [key][128
 // rows]) in LDS; both MFMA operands are LDS transpose reads with the keys as the k index:
 //   dQ^T[d][row] += K^T[d][key] dS^T[key][row]
-// Two LDS buffers, one barrier per step, the next step's global loads in flight during the
-// MFMAs.  Blocks the fused kernel never wrote (key tile entirely after the row tile under the
+// Two LDS buffers, one barrier per step, the global loads of the next two steps in flight during
+// the MFMAs (two register sets, the step loop unrolled by two).  Blocks the fused kernel never wrote (key tile entirely after the row tile under the
 // causal mask, or past the last key) are not used: zeros are staged in their place.
 #include "mfma_common.hpp"
 
@@ -61,9 +61,11 @@ __global__ __launch_bounds__(NW * 64) void dq_from_ds_kernel(Problem p, const bf
 
     // this thread's chunk of each of the 4 dS blocks of a step: key tid/8, rows 8*(tid%8) .. +7
     const int t_key = tid >> 3, t_ch = tid & 7;
-    u32x4 kr[K_LD], tr[4];
-    bool tv[4];
-    auto load_step = [&](int s) {
+    // two register sets: the loads of steps s+1 and s+2 are in flight while step s is multiplied
+    // (one step of MFMAs is shorter than the memory latency)
+    u32x4 kr_a[K_LD], tr_a[4], kr_b[K_LD], tr_b[4];
+    bool tv_a[4], tv_b[4];
+    auto load_step = [&](int s, u32x4 (&kr)[K_LD], u32x4 (&tr)[4], bool (&tv)[4]) {
 #pragma unroll
         for (int i = 0; i < K_LD; ++i) {
             const int c = tid + i * NW * 64, row = c / CPR, cc = c % CPR;
@@ -80,8 +82,8 @@ __global__ __launch_bounds__(NW * 64) void dq_from_ds_kernel(Problem p, const bf
         }
     };
 
-    if (n_steps > 0) load_step(0);
-    for (int s = 0; s < n_steps; ++s) {
+    // loads past the last step re-read clamped addresses and are never staged
+    auto run_step = [&](int s, u32x4 (&kr)[K_LD], u32x4 (&tr)[4], bool (&tv)[4]) {
         unsigned char *Ks = smem + (s & 1) * (Lds::k_bytes + Lds::t_bytes);
         unsigned char *Ts = Ks + Lds::k_bytes;
 #pragma unroll
@@ -94,8 +96,8 @@ __global__ __launch_bounds__(NW * 64) void dq_from_ds_kernel(Problem p, const bf
             *reinterpret_cast<u32x4 *>(Ts + ((i >> 1) * kDsKeys + t_key) * TST + ((i & 1) * kDsRows + t_ch * 8) * 2) =
                 zero_unless(tv[i], tr[i]);
         __syncthreads();
-        if (s + 1 < n_steps) load_step(s + 1);
-        if (causal && s * BKS > rw + 31) continue;  // every key of the step is after the wave's rows
+        load_step(s + 2, kr, tr, tv);
+        if (causal && s * BKS > rw + 31) return;  // every key of the step is after the wave's rows
 
 #pragma unroll
         for (int kp = 0; kp < BKS / 32; ++kp) {
@@ -115,6 +117,12 @@ __global__ __launch_bounds__(NW * 64) void dq_from_ds_kernel(Problem p, const bf
                 for (int ob = 0; ob < 2; ++ob) acc[ob][db] = mfma_bf16(kf, sf[ob], acc[ob][db]);
             }
         }
+    };
+    load_step(0, kr_a, tr_a, tv_a);
+    load_step(1, kr_b, tr_b, tv_b);
+    for (int s = 0; s < n_steps; s += 2) {
+        run_step(s, kr_a, tr_a, tv_a);
+        if (s + 1 < n_steps) run_step(s + 1, kr_b, tr_b, tv_b);
     }
 
     // lane = position ob*16+n of the wave's 32 rows in the dS blocks' row order;
