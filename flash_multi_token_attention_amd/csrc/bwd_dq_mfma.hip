@@ -370,8 +370,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_mfma_kernel(
                 for (int u = 0; u < 4; ++u) {
                     const int ii = i + (u >> 1), jb = u & 1;
                     af[u] = *reinterpret_cast<const f16x8 *>(abase + ii * SST + jb * 64);
-                    bw[u] = reinterpret_cast<const U32x4A4 *>(bbase + ii * CST + jb * 64)->v;
-                    bx[u] = *reinterpret_cast<const unsigned int *>(bbase + ii * CST + jb * 64 + 16);
+                    lds_read_dwords5(bbase + ii * CST + jb * 64, bw[u], bx[u]);
                 }
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {

@@ -482,8 +482,9 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
             // A: S[i + a - pq][c0 + 8g ..]        (S-tile row HT + i + a - pq, column 16 + 8g)
             // B: dC[i][c0 + 8g - b + pk ..]       (dC-tile row HT + i, column 8 + 8g - b + pk)
             const unsigned char *abase = s_ring + (16 + 8 * g) * 2;
-            // LDS reads at odd 2-byte offsets are slow: read 5 dwords from the even
-            // element below and funnel-shift by 0 or 16 bits per lane instead.
+            // LDS reads at odd 2-byte offsets are slow, and so are 128-bit reads off a 16-byte
+            // boundary: read 5 single dwords from the even element below and funnel-shift by 0 or
+            // 16 bits per lane instead.
             const int boff = 8 + 8 * g - bcl + pk;
             const unsigned char *bbase = c_ring + (tb + HT) * CST + (boff & ~1) * 2;
             const unsigned int bsh = (boff & 1) * 16;
@@ -500,8 +501,7 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
                 unsigned int bx[RPL];
 #pragma unroll
                 for (int u = 0; u < RPL; ++u) {
-                    bw[u] = reinterpret_cast<const U32x4A4 *>(bbase + (i + u) * CST)->v;
-                    bx[u] = *reinterpret_cast<const unsigned int *>(bbase + (i + u) * CST + 16);
+                    lds_read_dwords5(bbase + (i + u) * CST, bw[u], bx[u]);
                 }
 #pragma unroll
                 for (int u = 0; u < RPL; ++u) {

@@ -25,9 +25,15 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-// 16 bytes at a 4-byte boundary (gfx950 LDS reads need no natural alignment, and
-// dword-aligned ones run at full speed)
-struct __attribute__((packed, aligned(4))) U32x4A4 { u32x4 v; };
+// Five consecutive dwords at a 4-byte boundary of LDS, as 32-bit reads (the compiler pairs them
+// into ds_read2_b32).  A 128-bit LDS read that is not 16-byte aligned is legal on gfx950 but slow:
+// measured with four waves reading, one costs about 66 clocks of the LDS pipe against about 12 for
+// the five dwords read separately.
+__device__ __forceinline__ void lds_read_dwords5(const unsigned char *p, u32x4 &lo, unsigned int &hi) {
+    const unsigned int *q = reinterpret_cast<const unsigned int *>(p);
+    lo = (u32x4){q[0], q[1], q[2], q[3]};
+    hi = q[4];
+}
 
 constexpr int kKeyHalo = 8;          // LDS columns before a block's first output key
 constexpr int kMfmaMaxPk = 8;        // so c_k <= 17 on the MFMA path
