@@ -46,6 +46,9 @@ HIPCC_FLAGS = [
     "-Wno-unused-command-line-argument",
     # keep the compiler from forming packed-fp32 VALU ops
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # machine scheduler tuned for instruction-level parallelism rather than occupancy: every kernel
+    # here runs at a fixed one or two waves per SIMD (measured: forward, backward and decode 0.5-1 % faster)
+    "-mllvm", "-amdgpu-sched-strategy=max-ilp",
 ]
 
 
