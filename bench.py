@@ -182,8 +182,10 @@ def cpu_baseline(wl, budget_s=12.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=3)
+    # a step takes under 3 ms: the defaults are long enough for the clocks to settle (10 steps after 3
+    # warm-up steps read 5 % slower per step than 50 after 10)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c3_fwd_bwd", choices=["c3_fwd_bwd", "c5_long", "c2_fwd"])
     ap.add_argument("--exact", action="store_true", help="force the fp32-arithmetic kernels")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
