@@ -47,6 +47,7 @@ _SIGNATURES = {
     "convattn_bwd_fused_dw": (C.c_int, [_D] + [_P] * 3),
     "convattn_decode_partial_bytes": (C.c_size_t, [_D]),
     "convattn_decode": (C.c_int, [_D] + [_P] * 8),
+    "convattn_decode_strided": (C.c_int, [_D] + [_P] * 4 + [C.c_longlong] * 2 + [_P] * 4),
     "convattn_decode_combine": (C.c_int, [_D] + [_P] * 7),
 }
 EXPORTS = tuple(_SIGNATURES)

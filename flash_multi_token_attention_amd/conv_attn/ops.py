@@ -39,9 +39,22 @@ def _check_input(t: torch.Tensor, name: str) -> None:
         raise RuntimeError(f"{name} must be contiguous")
 
 
-def _check_qkv(Q, K, V, names=("Q", "K", "V")):
+def _is_cache_view(t: torch.Tensor) -> bool:
+    """[B,H,N,d] view of a longer cache: rows of a head dense, heads and batches strided."""
+    if t.dim() != 4:
+        return False
+    B, H, N, d = t.shape
+    sb, sh, sn, sd = t.stride()
+    return (sd == 1 and sn == d and sh >= N * d and sh % 8 == 0 and sb % 8 == 0
+            and (B == 1 or sb >= N * d))
+
+
+def _check_qkv(Q, K, V, names=("Q", "K", "V"), kv_views=False):
     for t, n in zip((Q, K, V), names):
-        _check_input(t, n)
+        if kv_views and t is not Q and t.is_cuda and _is_cache_view(t):
+            pass  # decode reads K / V views of a preallocated cache in place
+        else:
+            _check_input(t, n)
         if t.dim() != 4:
             raise RuntimeError(f"{n} must be [batch, heads, seq_len, d_head]")
     if Q.dtype not in _DT:
@@ -216,8 +229,13 @@ def default_k_splits(B: int, H: int, Nk: int) -> int:
 def decode(Q, K, V, conv_kernel, k_splits, scale, causal=False, out_dtype=torch.float32,
            exact=False, workspace=None):
     """Decode step -> (O [B,H,1,d], M, L [B,H,1], partials).  Q holds the resident
-    last rows (1..16).  ``k_splits`` None/0 picks a split count from the shape."""
-    _check_qkv(Q, K, V)
+    last rows (1..16).  ``k_splits`` None/0 picks a split count from the shape.
+    K and V may be views ``cache[:, :, :Nk]`` of a cache allocated as [B,H,N_max,d] (same
+    strides for both): they are read in place, where the reference's CHECK_CONTIGUOUS
+    (conv_attn/kernels/fwd_inference_wrapper.cu:8,26-27) forces a copy per step."""
+    _check_qkv(Q, K, V, kv_views=True)
+    if K.stride() != V.stride():
+        raise RuntimeError("K and V must have the same strides")
     B, H, r, d = Q.shape
     c_q, c_k = conv_kernel.shape[1], conv_kernel.shape[2]
     W = _weights(conv_kernel, H, c_q - 1, (c_k - 1) // 2, Q.device)
@@ -239,8 +257,11 @@ def decode(Q, K, V, conv_kernel, k_splits, scale, causal=False, out_dtype=torch.
     M = torch.empty((B, H, 1), dtype=torch.float32, device=Q.device)
     L = torch.empty((B, H, 1), dtype=torch.float32, device=Q.device)
     st = _stream(Q)
-    rc = lib.convattn_decode(C.byref(desc), _ptr(Q), _ptr(K), _ptr(V), _ptr(W), _ptr(O_part),
-                             _ptr(M_part), _ptr(L_part), st)
+    Nk = K.shape[2]
+    kv_bs, kv_hs = (H * Nk * d, Nk * d) if K.is_contiguous() else (K.stride(0), K.stride(1))
+    rc = lib.convattn_decode_strided(C.byref(desc), _ptr(Q), _ptr(K), _ptr(V), _ptr(W),
+                                     C.c_longlong(kv_bs), C.c_longlong(kv_hs),
+                                     _ptr(O_part), _ptr(M_part), _ptr(L_part), st)
     _lib.check(rc, "conv_attn.forward_inference")
     rc = lib.convattn_decode_combine(C.byref(desc), _ptr(O_part), _ptr(M_part), _ptr(L_part), _ptr(O),
                                      _ptr(M), _ptr(L), st)

@@ -30,6 +30,7 @@ int validate(const convattn_desc *d, int op, Problem *out) {
     p.B = d->B; p.H = d->H; p.Nq = d->Nq; p.Nk = d->Nk; p.d = d->d;
     p.c_q = d->c_q; p.c_k = d->c_k; p.pq = d->c_q - 1; p.pk = (d->c_k - 1) / 2;
     p.scale = d->scale; p.causal = d->causal ? 1 : 0; p.n_splits = 1;
+    p.kv_hstride = (long long)d->Nk * d->d; p.kv_bstride = p.kv_hstride * d->H;
     if (op == CONVATTN_OP_DECODE) {
         if (d->Nq > 16) return CONVATTN_ERR_QROWS;
         if (d->n_splits < 1 || d->n_splits > d->Nk || d->n_splits > 1024) return CONVATTN_ERR_SPLITS;
@@ -238,9 +239,22 @@ size_t convattn_decode_partial_bytes(const convattn_desc *desc) {
 
 int convattn_decode(const convattn_desc *desc, const void *q, const void *k, const void *v,
                     const float *w, float *o_part, float *m_part, float *l_part, void *stream) {
+    if (!desc) return CONVATTN_ERR_NULL;
+    const long long hs = (long long)desc->Nk * desc->d;
+    return convattn_decode_strided(desc, q, k, v, w, hs * desc->H, hs, o_part, m_part, l_part, stream);
+}
+
+int convattn_decode_strided(const convattn_desc *desc, const void *q, const void *k, const void *v,
+                            const float *w, long long kv_batch_stride, long long kv_head_stride,
+                            float *o_part, float *m_part, float *l_part, void *stream) {
     Problem p;
     int rc = validate(desc, CONVATTN_OP_DECODE, &p);
     if (rc) return rc;
+    // rows of a head stay dense (d elements apart) and 16-byte aligned; heads and batches must not overlap
+    if (kv_head_stride < (long long)p.Nk * p.d || kv_head_stride % 8 != 0 || kv_batch_stride % 8 != 0 ||
+        (p.B > 1 && kv_batch_stride < (long long)p.Nk * p.d))
+        return CONVATTN_ERR_SHAPE;
+    p.kv_bstride = kv_batch_stride; p.kv_hstride = kv_head_stride;
     REQUIRE_PTR(q); REQUIRE_PTR(k); REQUIRE_PTR(v); REQUIRE_PTR(w);
     REQUIRE_PTR(o_part); REQUIRE_PTR(m_part); REQUIRE_PTR(l_part);
     hipStream_t s = static_cast<hipStream_t>(stream);

@@ -15,6 +15,9 @@ struct Problem {
     float scale;
     int causal;
     int n_splits;
+    // decode only: elements between consecutive batches / heads of K and V (a dense [B,H,Nk,d]
+    // tensor has H*Nk*d and Nk*d; a view of a longer cache has the cache's)
+    long long kv_bstride, kv_hstride;
 };
 
 typedef __bf16 bf16_t;

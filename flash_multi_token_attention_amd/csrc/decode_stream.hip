@@ -63,8 +63,8 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(
     const int cq = p.c_q, ck = p.c_k, pk = p.pk;
     const size_t bh = (size_t)b * p.H + h;
     const bf16_t *Qb = Q + bh * p.Nq * D;
-    const bf16_t *Kb = K + bh * p.Nk * D;
-    const bf16_t *Vb = V + bh * p.Nk * D;
+    const bf16_t *Kb = K + b * p.kv_bstride + h * p.kv_hstride;
+    const bf16_t *Vb = V + b * p.kv_bstride + h * p.kv_hstride;
     float *strip = s_strip[wave];
 
     for (int i = tid; i < cq * ck; i += NW * 64) s_w[i] = W[(size_t)h * cq * ck + i];

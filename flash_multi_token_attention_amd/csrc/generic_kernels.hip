@@ -403,8 +403,8 @@ __global__ __launch_bounds__(NT) void gen_decode_kernel(Problem p, const TI *__r
 
     const size_t bh = (size_t)b * p.H + h;
     const TI *Qb = Q + bh * p.Nq * d;
-    const TI *Kb = K + bh * p.Nk * d;
-    const TI *Vb = V + bh * p.Nk * d;
+    const TI *Kb = K + b * p.kv_bstride + h * p.kv_hstride;
+    const TI *Vb = V + b * p.kv_bstride + h * p.kv_hstride;
     load_rows(Qs, d, Qb, p.Nq - cq, cq, p.Nq, d);
     for (int i = tid; i < ntap; i += NT) Ws[i] = W[(size_t)h * ntap + i];
     if (tid == 0) { st[0] = kNegInf; st[1] = 0.f; }

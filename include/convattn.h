@@ -198,6 +198,19 @@ int convattn_decode(const convattn_desc *desc, const void *q, const void *k, con
                     const float *w, float *o_part, float *m_part, float *l_part, void *stream);
 
 /*
+ * The same over K and V that are views of a longer cache: rows of one head are dense
+ * ([Nk][d]), consecutive heads are kv_head_stride elements apart and consecutive batches
+ * kv_batch_stride (both multiples of 8, kv_head_stride >= Nk*d).  A cache allocated as
+ * [B,H,N_max,d] and read as cache[:, :, :Nk] has kv_head_stride = N_max*d and
+ * kv_batch_stride = H*N_max*d.  The reference requires contiguous K and V
+ * (CHECK_CONTIGUOUS, conv_attn/kernels/fwd_inference_wrapper.cu:8,28-30), so its callers copy
+ * such a view on every step; convattn_decode is this call with the dense strides.
+ */
+int convattn_decode_strided(const convattn_desc *desc, const void *q, const void *k, const void *v,
+                            const float *w, long long kv_batch_stride, long long kv_head_stride,
+                            float *o_part, float *m_part, float *l_part, void *stream);
+
+/*
  * Log-sum-exp merge of the split partials into O [B,H,1,d] (out_dtype), M, L
  * [B,H,1] fp32.  Replaces combine_splits_kernel (conv_attn/kernels/
  * fwd_inference.cu:286-369); unlike the reference it also runs for n_splits == 1,

@@ -79,6 +79,13 @@ def test_null_and_misaligned_pointers_rejected_before_launch(lib):
     assert lib.convattn_fwd(C.byref(d), ok, ok, odd, ok, ok, ok, ok, null) == -6
     assert lib.convattn_bwd_dkdv(C.byref(d), ok, ok, ok, ok, ok, ok, ok, ok, null, null) == -1
     assert lib.convattn_validate(None, 0) == -1
+    # strided decode: heads closer together than Nk*d, or strides that break the 16-byte alignment
+    dd = desc(Nq=6, causal=0, n_splits=2)
+    LL = C.c_longlong
+    dense_h = dd.Nk * dd.d
+    assert lib.convattn_decode_strided(C.byref(dd), ok, ok, ok, ok, LL(dense_h * dd.H), LL(dense_h - 8), ok, ok, ok, null) == -2
+    assert lib.convattn_decode_strided(C.byref(dd), ok, ok, ok, ok, LL(dense_h * dd.H), LL(dense_h + 4), ok, ok, ok, null) == -2
+    assert lib.convattn_decode_strided(C.byref(dd), null, ok, ok, ok, LL(dense_h * dd.H), LL(dense_h), ok, ok, ok, null) == -1
     assert lib.convattn_dw_partial_bytes(C.byref(desc(d=3))) == 0
     assert lib.convattn_decode_partial_bytes(C.byref(desc(Nq=6, causal=0, n_splits=8))) == 2 * 4 * 8 * 64 * 4
 

@@ -214,6 +214,35 @@ def test_decode_bf16_stream(r, Nk, d, c_q, c_k, splits, causal):
     assert rel_max(L, L_ref) <= 1e-3
 
 
+@pytest.mark.parametrize("dtype,d,n_max", [(torch.bfloat16, 128, 700), (torch.bfloat16, 64, 512), (torch.float32, 64, 333)])
+def test_decode_reads_views_of_a_longer_cache_in_place(dtype, d, n_max):
+    """K / V as cache[:, :, :Nk] of a [B,H,N_max,d] cache: same bits as a dense copy, both kernel
+    families; the rows after Nk are poisoned and must not be read into the result."""
+    from flash_multi_token_attention_amd.conv_attn import fwd_conv_attn_inference
+    B, H, r, Nk, c_q, c_k = 2, 3, 6, 300, 6, 11
+    Q, K, V, _, W = rand_case(B, H, r, Nk, d, c_q, c_k, dtype, seed=n_max)
+    g = [t.to(DEV) for t in (Q, K, V, W)]
+    Kc = torch.full((B, H, n_max, d), float("nan"), dtype=dtype, device=DEV)
+    Vc = torch.full((B, H, n_max, d), float("nan"), dtype=dtype, device=DEV)
+    Kc[:, :, :Nk] = g[1]
+    Vc[:, :, :Nk] = g[2]
+    Kv, Vv = Kc[:, :, :Nk], Vc[:, :, :Nk]
+    assert not Kv.is_contiguous()
+    for causal in (False, True):
+        for splits in (1, 3):
+            dense = fwd_conv_attn_inference(g[0], g[1], g[2], g[3], splits, scale_of(d), c_q - 1, (c_k - 1) // 2, causal)
+            view = fwd_conv_attn_inference(g[0], Kv, Vv, g[3], splits, scale_of(d), c_q - 1, (c_k - 1) // 2, causal)
+            for a, b in zip(dense, view):
+                assert torch.equal(a, b)
+    # a sequence-major cache ([B,N,H,d] permuted) has no dense rows per head: rejected, as a
+    # non-contiguous tensor is by the reference
+    Ks = g[1].permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        fwd_conv_attn_inference(g[0], Ks, Ks, g[3], 1, scale_of(d), c_q - 1, (c_k - 1) // 2, False)
+    with pytest.raises(RuntimeError, match="same strides"):
+        fwd_conv_attn_inference(g[0], Kv, g[2], g[3], 1, scale_of(d), c_q - 1, (c_k - 1) // 2, False)
+
+
 def test_decode_full_size_properties():
     # c4-sized cache per (batch, head) (fewer pairs): split invariance, agreement with
     # the fp32-arithmetic kernel, and sum of probabilities == 1 (V = 1 -> O = 1).
