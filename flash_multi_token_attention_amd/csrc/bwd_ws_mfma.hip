@@ -211,6 +211,9 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
             unsigned char *Ps = pair_p(it & 1);
             const int tb = ring_tb(it), sb = s_base(it);
 
+            // a wave in an MFMA phase gets the issue slot before the SIMD's other wave (which is in
+            // the same role, somewhere else in its tile); element-wise phases run at priority 0
+            __builtin_amdgcn_s_setprio(1);
             // ---- S^T tile (raw) -> fp16 LDS; Q fragments one row block ahead.  The first 16 rows
             // are the last 16 of the previous tile (masks depend on positions only): taken over from
             // the other buffer when that tile was computed. ----
@@ -314,6 +317,7 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
                         SCHED_MFMA_ID(NCB, SID);
                     }
                 }
+                __builtin_amdgcn_s_setprio(0);
 #pragma unroll
                 for (int kb = 0; kb < NCB; ++kb) {
                     f32x4 prob, dc;
@@ -336,6 +340,7 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
                             (_Float16)__builtin_amdgcn_fmed3f(dc[r], -kF16Max, kF16Max);
                     if (kb < 2) pkeep[rb][kb] = prob;
                 }
+                if (rb + 1 < NRB) __builtin_amdgcn_s_setprio(1);
             });
             // P of the tile as the consumer's MFMA operand: lane = key, elements = rows 4g.. of the
             // two row blocks
@@ -429,6 +434,7 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
                     for (int r = 0; r < 4; ++r)
                         if (c0 + m * 16 + n > r0 - HT + ob * 16 + 4 * g + r) ds[ob][m][r] = 0.f;
         }
+        __builtin_amdgcn_s_setprio(1);  // the dense MFMA phase of the consumer
         // ---- dK^T += Q^T dS (the Q tile starts at row r0-16 as well) and dV ----
         {
             bf16x8 sf[2];
@@ -477,6 +483,7 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
             }
         }
 
+        __builtin_amdgcn_s_setprio(0);
         // ---- dW: rows m = tap a, columns n = tap b, contraction over (own row, 8 own keys) ----
         if (r0 < p.Nq) {
             // A: S[i + a - pq][c0 + 8g ..]        (S-tile row HT + i + a - pq, column 16 + 8g)
