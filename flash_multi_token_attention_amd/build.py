@@ -37,6 +37,8 @@ UNITS = [
     ("bwd_dkdv_mfma.hip", "bwd_dkdv_mfma_wide", ["-DCONVATTN_DKDV_UNIT=1"]),
     ("bwd_ws_mfma.hip", "bwd_ws_mfma", []),
     ("bwd_dq_gemm.hip", "bwd_dq_gemm", []),
+    ("bwd_chain_mfma.hip", "bwd_chain_mfma", []),
+    ("bwd_dq_rows.hip", "bwd_dq_rows", []),
     ("decode_stream.hip", "decode_stream", []),
 ]
 SOURCES = sorted({u[0] for u in UNITS})

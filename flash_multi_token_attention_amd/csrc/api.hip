@@ -170,11 +170,27 @@ int convattn_bwd_dkdv(const convattn_desc *desc, const void *q, const void *k, c
     return (int)generic_bwd_dkdv(p, desc->in_dtype, desc->out_dtype, q, k, v, d_o, D, lse, w, dk, dv, s);
 }
 
+// Workspace of the one-pass backward on the MFMA path: dS blocks, dW partials and (windows of up
+// to 6 query taps) the dC scale of every (batch, head), each part 256-byte aligned.
+struct FusedWs {
+    size_t ds_bytes, part_off, scale_off, total;
+    bool chain;
+};
+static FusedWs fused_ws(const Problem &p) {
+    FusedWs w;
+    w.chain = chain_ok(p);
+    w.ds_bytes = w.chain ? chain_ds_bytes(p) : mfma_ds_bytes(p);
+    w.part_off = align256(w.ds_bytes);
+    w.scale_off = w.part_off + align256(fused_dw_bytes(p));
+    w.total = w.scale_off + (w.chain ? align256(chain_scale_bytes(p)) : 0);
+    return w;
+}
+
 size_t convattn_bwd_fused_workspace_bytes(const convattn_desc *desc) {
     Problem p;
     if (validate(desc, CONVATTN_OP_BWD, &p)) return 0;
     if (pick_path(desc, p, CONVATTN_OP_BWD) != 1) return align256(convattn_dw_partial_bytes(desc));
-    return align256(mfma_ds_bytes(p)) + align256(fused_dw_bytes(p));
+    return fused_ws(p).total;
 }
 
 int convattn_bwd_fused_dkdv(const convattn_desc *desc, const void *q, const void *k, const void *v,
@@ -189,8 +205,14 @@ int convattn_bwd_fused_dkdv(const convattn_desc *desc, const void *q, const void
     if (pick_path(desc, p, CONVATTN_OP_BWD) != 1)
         return (int)generic_bwd_dkdv(p, desc->in_dtype, desc->out_dtype, q, k, v, d_o, D, lse, w, dk, dv, s);
     unsigned char *ws = static_cast<unsigned char *>(workspace);
-    float *part = reinterpret_cast<float *>(ws + align256(mfma_ds_bytes(p)));
-    return (int)mfma_bwd_fused_ws(p, desc->out_dtype, q, k, v, d_o, D, lse, w, dk, dv, ws, part, s);
+    const FusedWs lay = fused_ws(p);
+    float *part = reinterpret_cast<float *>(ws + lay.part_off);
+    if (!lay.chain)
+        return (int)mfma_bwd_fused_ws(p, desc->out_dtype, q, k, v, d_o, D, lse, w, dk, dv, ws, part, s);
+    float *scale = reinterpret_cast<float *>(ws + lay.scale_off);
+    hipError_t e = mfma_dc_scale(p, d_o, v, scale, s);
+    if (e != hipSuccess) return (int)e;
+    return (int)mfma_bwd_chain(p, desc->out_dtype, q, k, v, d_o, D, lse, w, scale, dk, dv, ws, part, s);
 }
 
 int convattn_bwd_fused_dq(const convattn_desc *desc, const void *q, const void *k, const void *v,
@@ -207,7 +229,10 @@ int convattn_bwd_fused_dq(const convattn_desc *desc, const void *q, const void *
         return (int)generic_bwd_dq_dw(p, desc->in_dtype, desc->out_dtype, q, k, v, d_o, D, lse, w, dq,
                                       static_cast<float *>(workspace), s);
     }
-    return (int)mfma_dq_from_ds(p, desc->out_dtype, k, workspace, dq, s);
+    const FusedWs lay = fused_ws(p);
+    if (!lay.chain) return (int)mfma_dq_from_ds(p, desc->out_dtype, k, workspace, dq, s);
+    const float *scale = reinterpret_cast<const float *>(static_cast<const unsigned char *>(workspace) + lay.scale_off);
+    return (int)mfma_dq_from_rows(p, desc->out_dtype, k, workspace, scale, dq, s);
 }
 
 int convattn_bwd_fused_dw(const convattn_desc *desc, const void *workspace, float *dw, void *stream) {
@@ -219,7 +244,7 @@ int convattn_bwd_fused_dw(const convattn_desc *desc, const void *workspace, floa
     if (pick_path(desc, p, CONVATTN_OP_BWD) != 1)
         return (int)dw_reduce(p, dw_tiles(desc, p), static_cast<const float *>(workspace), dw, s);
     const unsigned char *ws = static_cast<const unsigned char *>(workspace);
-    return (int)dw_reduce(p, mfma_kv_tiles(p), reinterpret_cast<const float *>(ws + align256(mfma_ds_bytes(p))), dw, s);
+    return (int)dw_reduce(p, mfma_kv_tiles(p), reinterpret_cast<const float *>(ws + fused_ws(p).part_off), dw, s);
 }
 
 int convattn_bwd_fused(const convattn_desc *desc, const void *q, const void *k, const void *v,

@@ -1,0 +1,897 @@
+// Whole backward of conv-attention on bf16 MFMA (gfx950): the score chain stays in registers.
+//
+// Key-stationary: a workgroup of 8 waves owns 128 keys of one (batch, head) and walks down the
+// query rows in tiles of 32.  Pair p (waves p and p+4, one SIMD) owns keys c0 = k0 + 32p .. c0+31
+// for dK and dS, c0-8 .. c0+23 for dV and dW.  Everything between the two products of a tile is
+// kept in the layout "lane = query row, registers = 4 keys" that the accumulators of
+// S^T = K Q^T come out in (lane n of fragment f holds row r0 + 2n + f):
+//   producer (waves 0-3): dP^T = V dO^T - D; S^T (raw, pre-masked, packed to fp16); the
+//       convolution as Toeplitz MFMAs whose B operand is the packed S^T itself, row-shifted by
+//       DPP moves (rows above the tile come from the previous tile's registers);
+//       P = exp2(C - LSE), dC = P dP.  P (bf16), dC and S (fp16) go to LDS as [row][key] tiles.
+//   consumer (waves 4-7), one tile behind: dV^T += dO^T P and dW += dC^T S with the operands read
+//       back through LDS transpose reads; two tiles behind: dS^T by flipped-band MFMAs over the
+//       packed dC^T (rows below a tile come from the next tile, hence the extra tile of delay),
+//       dS -> workspace (bf16, [row][key] blocks) and -> LDS, dK^T += Q^T dS.
+// One workgroup barrier per tile; Q and dO tiles are staged row-major with the 16-byte chunks of a
+// 256-byte line XOR-swizzled by the line number, so that both the row fragments (b128) and the
+// transpose reads are spread over all banks without padding.
+//
+// dW[a][b] = sum_i sum_j dC[i][j] S_m[i+a-pq][j+b-pk] is computed as G_a = dC^T S(rows shifted by
+// a), a [key j] x [key j'] product contracted over the rows on the matrix cores; only its
+// diagonals |j'-j| <= pk are wanted, so a 16-key block of j needs two 16-key blocks of j' and both
+// blocks of j add into the same two accumulators per tap.  The diagonals are summed once, after
+// the last tile.
+//
+// dC is carried as fp16 times a power of two chosen per (batch, head) from the magnitudes of dO
+// and V (dc_scale), which makes the backward linear in dO over the whole range of bf16: dK, dV, dW
+// and (in the dQ product) dQ are multiplied by its inverse when they are stored.
+#include <type_traits>
+
+#include "mfma_common.hpp"
+
+namespace convattn {
+namespace {
+
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int NP = 4;            // wave pairs = 32-key ranges per workgroup
+constexpr int NT = 2 * NP * 64;  // 512 threads
+constexpr int WK = 32;           // own keys per pair
+constexpr int BKW = NP * WK;     // 128 keys per workgroup
+constexpr int BR = 32;           // query rows per tile
+constexpr int NSB = 4;           // S^T blocks of a pair: keys c0-16+16kb
+constexpr int NCB = 3;           // C / dP / dC blocks: keys c0-8+16cb
+constexpr int NDB = 2;           // dS blocks: keys c0+16sb
+constexpr int SST = 112;         // bytes per row of the S tile in LDS (48 keys fp16 + 16)
+constexpr int S_RING = 72;       // rows of the S ring: a tile being written, the tile before it and 8 rows more (>= c_q - 1)
+constexpr int CST = 112;         // bytes per row of the dC tile (48 keys fp16 + 16)
+constexpr int PST = 72;          // bytes per row of the P and dS tiles (32 keys bf16 + 8)
+static_assert(BKW == kKvKeysPerWg && WK == kChainKeys && BR == kChainRows, "dS workspace layout");
+
+template <int D, int CQT> struct ChainLds {
+    static constexpr int RST = D * 2 + 16;                          // bytes per staged Q / dO row
+    static constexpr int tile_bytes = BR * RST;
+    static constexpr int q_off = 0, q_slots = 4;                    // tiles it-2 .. it+1
+    static constexpr int g_off = q_off + q_slots * tile_bytes, g_slots = 3;  // tiles it-1 .. it+1
+    static constexpr int stat_off = g_off + g_slots * tile_bytes;   // LSE and D of a tile: two slots
+    static constexpr int stat_bytes = 2 * (2 * BR * 4);
+    static constexpr int band_off = stat_off + stat_bytes;          // bands, then flipped bands: one KB per tap slot
+    static constexpr int band_bytes = 2 * CQT * 1024;
+    static constexpr int pair_off = band_off + band_bytes;
+    static constexpr int s_bytes = S_RING * SST;
+    static constexpr int c_bytes = 2 * BR * CST;
+    static constexpr int p_bytes = 2 * BR * PST;
+    static constexpr int ds_bytes = BR * PST;
+    static constexpr int pair_bytes = s_bytes + c_bytes + p_bytes + ds_bytes;
+    static constexpr int total = pair_off + NP * pair_bytes;
+    static_assert(CQT * 2 * 1024 <= pair_bytes, "room for the dW accumulators");
+};
+
+// A lane-dependent LDS offset the compiler may not fold or hoist: what is added to it afterwards
+// stays a constant and ends up in the instructions' offset fields instead of one address register
+// per fragment.
+__device__ __forceinline__ unsigned int opaque(unsigned int x) {
+    asm volatile("" : "+v"(x));
+    return x;
+}
+
+__device__ __forceinline__ bf16x4 lds_tr64(const unsigned char *ptr) {
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(ptr));
+    return __builtin_bit_cast(bf16x4, v);
+}
+// Transposed fragment of a row-major tile of 16-bit elements with `stride` bytes per row:
+// k = rows 4g .. 4g+3 then 16+4g .. 16+4g+3, column col0 + n.  `lane_ptr` is the tile's address plus
+// tr_lane_off(stride, g, n).
+__device__ __forceinline__ unsigned int tr_lane_off(int stride, int g, int n) {
+    return (4 * g + (n >> 2)) * stride + 4 * (n & 3) * 2;
+}
+__device__ __forceinline__ bf16x8 read_tr(const unsigned char *lane_ptr, int stride, int col0) {
+    bf16x4 lo = lds_tr64(lane_ptr + col0 * 2);
+    bf16x4 hi = lds_tr64(lane_ptr + 16 * stride + col0 * 2);
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+template <int CTRL>
+__device__ __forceinline__ unsigned int dpp_keep(unsigned int old, unsigned int src) {
+    return (unsigned int)__builtin_amdgcn_update_dpp((int)old, (int)src, CTRL, 0xf, 0xf, false);
+}
+// A DPP move that writes every lane (rotations): no previous value to keep.
+template <int CTRL>
+__device__ __forceinline__ unsigned int dpp_mov(unsigned int src) {
+    return (unsigned int)__builtin_amdgcn_mov_dpp((int)src, CTRL, 0xf, 0xf, true);
+}
+// Lane n of a row of 16 gets cur[n - S] for n >= S and prev[16 + n - S] below: a window that
+// starts S lanes before `cur` in the sequence prev | cur.
+template <int S>
+__device__ __forceinline__ unsigned int win_up(unsigned int prev, unsigned int cur) {
+    if constexpr (S == 0) {
+        return cur;
+    } else {
+        const unsigned int x = dpp_mov<0x120 + S>(prev);  // row_ror:S
+        return dpp_keep<0x110 + S>(x, cur);               // row_shr:S, lanes below S keep x
+    }
+}
+// Lane n gets a[n + S] for n + S < 16 and b[n + S - 16] above: a window that starts S lanes into
+// `a` in the sequence a | b.
+template <int S>
+__device__ __forceinline__ unsigned int win_down(unsigned int a, unsigned int b) {
+    if constexpr (S == 0) {
+        return a;
+    } else {
+        const unsigned int x = dpp_mov<0x120 + 16 - S>(b);  // row_ror:(16-S)
+        return dpp_keep<0x100 + S>(x, a);                   // row_shl:S, the last S lanes keep x
+    }
+}
+
+__device__ __forceinline__ unsigned int pack_f16_rtz(float a, float b) {
+    return __builtin_bit_cast(unsigned int, __builtin_amdgcn_cvt_pkrtz(a, b));
+}
+
+// Toeplitz bands for the packed operand order: k slot 8g+e of a 32-key window is key 4g+e of its
+// first 16-key block for e < 4 and key 4g+e-4 of its second for e >= 4; the output block starts 8
+// keys into the window.  Tap slot t stands for query tap a = t - (CQT - c_q) (zero taps in front).
+// `flip` builds the bands of the transposed convolution.
+template <int CQT>
+__device__ __forceinline__ f16x8 band_frag(int t, const float *__restrict__ w_head, int c_q, int c_k, int pk,
+                                           int g, int n, bool flip, float mul) {
+    const int a = t - (CQT - c_q);
+    f16x8 f = (f16x8)(_Float16)0.f;
+    if (a >= 0) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int kappa = e < 4 ? 4 * g + e : 16 + 4 * g + e - 4;
+            const int off = kappa - kKeyHalo - n;
+            const int bb = flip ? pk - off : pk + off;
+            float v = 0.f;
+            if (bb >= 0 && bb < c_k) v = w_head[a * c_k + bb] * mul;
+            f[e] = (_Float16)v;
+        }
+    }
+    return f;
+}
+
+#ifdef CHAIN_PHASE_BARRIERS
+#define CHAIN_SCHED_BARRIER __builtin_amdgcn_sched_barrier(0)
+#else
+#define CHAIN_SCHED_BARRIER
+#endif
+
+#ifdef CHAIN_TS
+__device__ long long g_chain_ts[8][64][12];
+#define TS(i)                                                                                     \
+    do {                                                                                          \
+        if (lane == 0 && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == CHAIN_TS && it < 64) \
+            g_chain_ts[wave][it][i] = clock64();                                                  \
+    } while (0)
+#else
+#define TS(i)
+#endif
+
+// Kernel arguments as one block: each role reads them from the kernel argument segment with
+// scalar loads (arguments of a device function would arrive in vector registers).
+struct ChainArgs {
+    Problem p;
+    const bf16_t *Q, *K, *V, *dO;
+    const float *Dl, *LSE, *W, *dc_scale;
+    void *dK, *dV;
+    bf16_t *dS_ws;
+    float *dW_part;
+    int n_rt;
+};
+
+// The kernel argument segment lives in the constant address space; host passes of the compiler
+// do not know that attribute.
+#if defined(__HIP_DEVICE_COMPILE__)
+#define CHAIN_CONST_AS __attribute__((address_space(4)))
+#else
+#define CHAIN_CONST_AS
+#endif
+
+// One role of the workgroup (ROLE 0 = producer waves, 1 = consumer waves) as a function of its
+// own: the two roles have disjoint register sets of 256 each, and compiled into one function body
+// the register allocator spills where either role alone does not.
+template <int D, int CQT, typename TO, int ROLE>
+__device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainArgs *args_in) {
+    // the pointer arrives in vector registers; it is the same in every lane, and as a scalar the
+    // arguments are fetched with scalar loads into scalar registers
+    const unsigned long long av = reinterpret_cast<unsigned long long>(args_in);
+    const unsigned long long as =
+        ((unsigned long long)(unsigned int)__builtin_amdgcn_readfirstlane((int)(av >> 32)) << 32) |
+        (unsigned int)__builtin_amdgcn_readfirstlane((int)(unsigned int)av);
+    const ChainArgs args = *reinterpret_cast<const CHAIN_CONST_AS ChainArgs *>(as);
+    const Problem p = args.p;
+    const bf16_t *__restrict__ Q = args.Q, *__restrict__ K = args.K, *__restrict__ V = args.V, *__restrict__ dO = args.dO;
+    const float *__restrict__ Dl = args.Dl, *__restrict__ LSE = args.LSE, *__restrict__ W = args.W;
+    const float *__restrict__ dc_scale = args.dc_scale;
+    TO *__restrict__ dK = static_cast<TO *>(args.dK), *__restrict__ dV = static_cast<TO *>(args.dV);
+    bf16_t *__restrict__ dS_ws = args.dS_ws;
+    float *__restrict__ dW_part = args.dW_part;
+    const int n_rt = args.n_rt;
+    using Lds = ChainLds<D, CQT>;
+    constexpr int KS = D / 32, DB = D / 16, CPR = D / 8, RST = Lds::RST;
+    constexpr int CH = BR * CPR;                 // 16-byte chunks of a staged tile
+    constexpr int LD = (CH + NT - 1) / NT;       // per thread
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int g = lane >> 4, n = lane & 15;
+    constexpr bool producer = ROLE == 0;
+    const int pr = wave & (NP - 1);
+
+    auto q_slot = [&](int t) { return smem + Lds::q_off + (t & 3) * Lds::tile_bytes; };
+    auto g_slot = [&](int t) { return smem + Lds::g_off + (t % 3) * Lds::tile_bytes; };
+    auto stat_slot = [&](int t) { return reinterpret_cast<float *>(smem + Lds::stat_off + (t & 1) * (2 * BR * 4)); };
+    unsigned char *pair_base = smem + Lds::pair_off + pr * Lds::pair_bytes;
+    unsigned char *s_ring = pair_base;
+    auto c_stage = [&](int t) { return pair_base + Lds::s_bytes + (t & 1) * (BR * CST); };
+    auto p_stage = [&](int t) { return pair_base + Lds::s_bytes + Lds::c_bytes + (t & 1) * (BR * PST); };
+    unsigned char *ds_tile = pair_base + Lds::s_bytes + Lds::c_bytes + Lds::p_bytes;
+
+    // x = head, y = batch, z = key tile: the first key tiles see the most rows and go first
+    const int h = blockIdx.x, b = blockIdx.y;
+    const int k0 = blockIdx.z * BKW, c0 = k0 + pr * WK;
+    const int pk = p.pk, cq = p.c_q, ck = p.c_k;
+    const bool causal = p.causal != 0;
+    const size_t bh = (size_t)b * p.H + h;
+    const bf16_t *Qb = Q + bh * p.Nq * D;
+    const bf16_t *dOb = dO + bh * p.Nq * D;
+    const float *lse_b = LSE + bh * p.Nq;
+    const float *dl_b = Dl + bh * p.Nq;
+    const float dcs = dc_scale ? dc_scale[2 * bh] : 1.f;       // power of two
+    const float dcs_log2 = dc_scale ? dc_scale[2 * bh + 1] : 0.f;
+
+    // Causal: rows before the first key this workgroup touches (k0 - 8) see none of its keys.
+    const int r_begin = causal ? (max(0, k0 - 8) / BR) * BR : 0;
+    const int n_tiles = (p.Nq - r_begin + BR - 1) / BR;
+    // masks are needed next to the diagonal, at both ends of the key axis and past the last row
+    const bool always_edge = c0 < 8 || c0 + 40 > p.Nk;
+    auto is_edge = [&](int r0) { return always_edge || (causal && r0 < c0 + 64) || r0 + BR > p.Nq; };
+    // no (row, key) pair of the tile is visible: only its scores are needed, by the tile below
+    auto is_skipped = [&](int r0) { return causal && r0 + BR - 1 < c0 - 8; };
+
+    // Staging registers: this thread's 16-byte chunks of the next Q / dO tile and its LSE / D entry.
+    u32x4 qr[LD], gr[LD];
+    float ls = 0.f, dd = 0.f;
+    // Buffer loads: rows before the first or after the last query row are outside the descriptor's
+    // range and read as zeros.
+    const __amdgpu_buffer_rsrc_t q_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)Qb, 0, p.Nq * D * 2, 0x00020000);
+    const __amdgpu_buffer_rsrc_t g_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)dOb, 0, p.Nq * D * 2, 0x00020000);
+    // (the thread's chunk coordinates are recomputed from an opaque copy of its index at every use:
+    // kept in registers across the tile loop they are what the register allocator spills first)
+    auto load_tile = [&](int r0) {
+        const int tt = (int)opaque((unsigned int)tid);
+#pragma unroll
+        for (int i = 0; i < LD; ++i) {
+            const int c = min(tt + i * NT, CH - 1), row = c / CPR, cc = c % CPR;
+            qr[i] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, ((r0 + row) * D + cc * 8) * 2, 0, 0);
+            gr[i] = __builtin_amdgcn_raw_buffer_load_b128(g_rsrc, ((r0 + row) * D + cc * 8) * 2, 0, 0);
+        }
+        if constexpr (producer) {
+            ls = 1e30f; dd = 0.f;  // rows past the end: exp2(C - LSE) = 0
+            if (tt < BR && r0 + tt < p.Nq) { ls = lse_b[r0 + tt] * kLog2e - dcs_log2; dd = dl_b[r0 + tt]; }
+        }
+    };
+    auto stage_tile = [&](int t) {
+        const int tt = (int)opaque((unsigned int)tid);
+        unsigned char *Qs = q_slot(t), *Gs = g_slot(t);
+#pragma unroll
+        for (int i = 0; i < LD; ++i) {
+            const int c = tt + i * NT, row = c / CPR, cc = c % CPR;
+            if (c < CH) {
+                *reinterpret_cast<u32x4 *>(Qs + row * RST + cc * 16) = qr[i];
+                *reinterpret_cast<u32x4 *>(Gs + row * RST + cc * 16) = gr[i];
+            }
+        }
+        if constexpr (producer) {
+            float *st = stat_slot(t);
+            if (tt < BR) { st[tt] = ls; st[BR + tt] = dd; }
+        }
+    };
+
+    load_tile(r_begin);
+    stage_tile(0);
+    load_tile(r_begin + BR);
+
+    if constexpr (producer) {
+        // ================================ producer ================================
+        const bf16_t *Kb = K + bh * p.Nk * D;
+        const bf16_t *Vb = V + bh * p.Nk * D;
+        // bands (times scale * log2 e: the convolved scores come out in log2 units) in LDS, one KB
+        // per tap slot, written by one wave; the first barrier of the tile loop publishes them
+        const unsigned char *bands = smem + Lds::band_off;
+        if (pr == 0) {
+#pragma unroll
+            for (int t = 0; t < CQT; ++t)
+                *reinterpret_cast<f16x8 *>(smem + Lds::band_off + t * 1024 + lane * 16) =
+                    band_frag<CQT>(t, W + (size_t)h * cq * ck, cq, ck, pk, g, n, false, p.scale * kLog2e);
+        }
+        bf16x8 kf[NSB][KS];  // K rows c0-16 .. c0+47
+        bf16x8 vf[NCB][KS];  // V rows c0-8 .. c0+39
+#pragma unroll
+        for (int kb = 0; kb < NSB; ++kb)
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+                kf[kb][ks] = __builtin_bit_cast(bf16x8, load_row16_nb<D>(Kb, c0 - 16 + kb * 16 + n, p.Nk, ks * 32 + g * 8));
+#pragma unroll
+        for (int kb = 0; kb < NCB; ++kb)
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+                vf[kb][ks] = __builtin_bit_cast(bf16x8, load_row16_nb<D>(Vb, c0 - 8 + kb * 16 + n, p.Nk, ks * 32 + g * 8));
+
+        // packed fp16 scores of the previous tile: [block][fragment][dword]
+        unsigned int prev_pd[NSB][2][2];
+
+        // S^T of the 32 rows r0 .. r0+31 (ring tile tp), pre-masked, packed and stored for dW
+        auto s_phase = [&](int r0, int tp, unsigned int (&pd)[NSB][2][2], auto edge_tag, auto &&load_qf) {
+            constexpr bool EDGE = decltype(edge_tag)::value;
+            f32x4 acc[NSB][2];
+#pragma unroll
+            for (int kb = 0; kb < NSB; ++kb)
+#pragma unroll
+                for (int f = 0; f < 2; ++f) acc[kb][f] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                bf16x8 qf[2];
+#pragma unroll
+                for (int f = 0; f < 2; ++f) qf[f] = load_qf(f, ks);
+#pragma unroll
+                for (int kb = 0; kb < NSB; ++kb)
+#pragma unroll
+                    for (int f = 0; f < 2; ++f) acc[kb][f] = mfma_bf16(kf[kb][ks], qf[f], acc[kb][f]);
+            }
+            const int rbase = (tp * BR) % S_RING;
+#pragma unroll
+            for (int kb = 0; kb < NSB; ++kb)
+#pragma unroll
+                for (int f = 0; f < 2; ++f) {
+                    if constexpr (EDGE) {
+                        if (causal) {
+                            const int qpos = r0 + 2 * n + f, key0 = c0 - 16 + kb * 16 + 4 * g;
+#pragma unroll
+                            for (int r = 0; r < 4; ++r)
+                                if (key0 + r > qpos) acc[kb][f][r] = 0.f;
+                        }
+                    }
+                    pd[kb][f][0] = pack_f16_rtz(acc[kb][f][0], acc[kb][f][1]);
+                    pd[kb][f][1] = pack_f16_rtz(acc[kb][f][2], acc[kb][f][3]);
+                    if (kb < 3) {
+                        const int rr = rbase + 2 * n + f;
+                        *reinterpret_cast<u32x2 *>(s_ring + (rr >= S_RING ? rr - S_RING : rr) * SST + (kb * 16 + 4 * g) * 2) =
+                            (u32x2){pd[kb][f][0], pd[kb][f][1]};
+                    }
+                }
+        };
+
+        // the 32 rows above the first tile: their scores are the window's halo for tile 0
+        {
+            const int rp = r_begin - BR;
+            s_phase(rp, 0, prev_pd, std::true_type{}, [&](int f, int ks) {
+                return __builtin_bit_cast(bf16x8, load_row16_nb<D>(Qb, rp + 2 * n + f, p.Nq, ks * 32 + g * 8));
+            });
+        }
+
+        for (int it = 0; it <= n_tiles + 1; ++it) {
+            const int r0 = r_begin + it * BR;
+            TS(0);
+            __syncthreads();
+            TS(1);
+            if (it + 1 < n_tiles) stage_tile(it + 1);
+            load_tile(r0 + 2 * BR);
+            TS(2);
+            if (it >= n_tiles) continue;
+#if defined(CHAIN_SKIP_ROLE) && CHAIN_SKIP_ROLE == 0
+            continue;
+#endif
+
+            auto ptile = [&](auto edge_tag, auto full_tag) {
+                constexpr bool EDGE = decltype(edge_tag)::value;
+                constexpr bool FULL = decltype(full_tag)::value;
+                // row fragments: lane n of fragment f reads row 2n + f, 16 bytes at column 32 ks + 8 g
+                const unsigned char *Qs = smem + opaque((unsigned int)(q_slot(it) - smem) + 2 * n * RST + g * 16);
+                const unsigned char *Gs = smem + opaque((unsigned int)(g_slot(it) - smem) + 2 * n * RST + g * 16);
+                __builtin_amdgcn_s_setprio(1);
+                // ---- dP^T = V dO^T - D: depends on the staged tile only, so it goes first and its
+                // MFMAs run back to back with those of S^T ----
+                f32x4 dp[NCB][2];
+                float2 l2 = {0.f, 0.f};
+                if constexpr (FULL) {
+                    const float *st = stat_slot(it);
+                    l2 = *reinterpret_cast<const float2 *>(st + 2 * n);
+                    const float2 d2 = *reinterpret_cast<const float2 *>(st + BR + 2 * n);
+#pragma unroll
+                    for (int cb = 0; cb < NCB; ++cb) {
+                        dp[cb][0] = (f32x4){-d2.x, -d2.x, -d2.x, -d2.x};
+                        dp[cb][1] = (f32x4){-d2.y, -d2.y, -d2.y, -d2.y};
+                    }
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) {
+                        bf16x8 gf[2];
+#pragma unroll
+                        for (int f = 0; f < 2; ++f)
+                            gf[f] = *reinterpret_cast<const bf16x8 *>(Gs + f * RST + ks * 64);
+#pragma unroll
+                        for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+                            for (int f = 0; f < 2; ++f) dp[cb][f] = mfma_bf16(vf[cb][ks], gf[f], dp[cb][f]);
+                    }
+                }
+                TS(4);
+                // ---- S^T ----
+                unsigned int pd[NSB][2][2];
+                s_phase(r0, it + 1, pd, edge_tag, [&](int f, int ks) {
+                    return *reinterpret_cast<const bf16x8 *>(Qs + f * RST + ks * 64);
+                });
+                CHAIN_SCHED_BARRIER;
+                TS(3);
+                if constexpr (FULL) {
+                    unsigned char *Cs = c_stage(it), *Ps = p_stage(it);
+                    // ---- convolution: C^T block cb from score blocks cb (k slots 0..3 of a lane
+                    // group) and cb+1 (4..7).  Operand of row offset delta = DL - (CQT-1): fragment
+                    // f = delta & 1 shifted s = (f - delta) / 2 lanes down; it serves output parity
+                    // 0 with tap slot DL and parity 1 with tap slot DL - 1. ----
+                    f32x4 c[NCB][2];
+#pragma unroll
+                    for (int cb = 0; cb < NCB; ++cb) {
+                        c[cb][0] = (f32x4){-l2.x, -l2.x, -l2.x, -l2.x};
+                        c[cb][1] = (f32x4){-l2.y, -l2.y, -l2.y, -l2.y};
+                    }
+                    f16x8 tf_prev = (f16x8)(_Float16)0.f;
+                    static_for<CQT + 1>([&](auto DL) {
+                        constexpr int t0 = decltype(DL)::value;
+                        constexpr int delta = t0 - (CQT - 1);
+                        constexpr int f = delta & 1, s = (f - delta) / 2;
+                        f16x8 tf_cur = tf_prev;
+                        if constexpr (t0 < CQT) tf_cur = *reinterpret_cast<const f16x8 *>(bands + t0 * 1024 + lane * 16);
+                        unsigned int sh[NSB][2];
+#pragma unroll
+                        for (int kb = 0; kb < NSB; ++kb)
+#pragma unroll
+                            for (int dw = 0; dw < 2; ++dw) sh[kb][dw] = win_up<s>(prev_pd[kb][f][dw], pd[kb][f][dw]);
+#pragma unroll
+                        for (int cb = 0; cb < NCB; ++cb) {
+                            const u32x4 bv = {sh[cb][0], sh[cb][1], sh[cb + 1][0], sh[cb + 1][1]};
+                            if constexpr (t0 < CQT) c[cb][0] = mfma_f16(tf_cur, __builtin_bit_cast(f16x8, bv), c[cb][0]);
+                            if constexpr (t0 >= 1) c[cb][1] = mfma_f16(tf_prev, __builtin_bit_cast(f16x8, bv), c[cb][1]);
+                        }
+                        tf_prev = tf_cur;
+                    });
+#pragma unroll
+                    for (int kb = 0; kb < NSB; ++kb)
+#pragma unroll
+                        for (int f = 0; f < 2; ++f) { prev_pd[kb][f][0] = pd[kb][f][0]; prev_pd[kb][f][1] = pd[kb][f][1]; }
+                    CHAIN_SCHED_BARRIER;
+                    TS(5);
+                    // ---- P = exp2(C - LSE) (times the dC scale), dC = P dP ----
+                    static_for<NCB>([&](auto CB) {
+                        constexpr int cb = decltype(CB)::value;
+                        __builtin_amdgcn_s_setprio(0);
+#pragma unroll
+                        for (int ob = 0; ob < 2; ++ob) {
+                            f32x4 prob, dc;
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) {
+                                prob[r] = fast_exp2(c[cb][ob][r]);
+                                dc[r] = prob[r] * dp[cb][ob][r];
+                            }
+                            if constexpr (EDGE) {
+                                const int qpos = r0 + 2 * n + ob;
+#pragma unroll
+                                for (int r = 0; r < 4; ++r) {
+                                    const int key = c0 - 8 + cb * 16 + 4 * g + r;
+                                    if (key < 0 || key >= p.Nk || (causal && key > qpos)) { prob[r] = 0.f; dc[r] = 0.f; }
+                                }
+                            }
+                            *reinterpret_cast<u32x2 *>(Cs + (2 * n + ob) * CST + (cb * 16 + 4 * g) * 2) =
+                                (u32x2){pack_f16_rtz(dc[0], dc[1]), pack_f16_rtz(dc[2], dc[3])};
+                            if constexpr (cb < 2) {
+                                bf16x4 pv;
+#pragma unroll
+                                for (int r = 0; r < 4; ++r) pv[r] = (bf16_t)prob[r];
+                                *reinterpret_cast<bf16x4 *>(Ps + (2 * n + ob) * PST + (cb * 16 + 4 * g) * 2) = pv;
+                            }
+                        }
+                    });
+                } else {
+#pragma unroll
+                    for (int kb = 0; kb < NSB; ++kb)
+#pragma unroll
+                        for (int f = 0; f < 2; ++f) { prev_pd[kb][f][0] = pd[kb][f][0]; prev_pd[kb][f][1] = pd[kb][f][1]; }
+                }
+            };
+            if (is_skipped(r0)) ptile(std::true_type{}, std::false_type{});
+            else if (is_edge(r0)) ptile(std::true_type{}, std::true_type{});
+            else ptile(std::false_type{}, std::true_type{});
+            TS(6);
+        }
+        __syncthreads();  // the consumers' barrier before they hand over their dW accumulators
+    } else {
+        // ================================ consumer ================================
+        const float *w_head = W + (size_t)h * cq * ck;
+        // flipped bands (times the softmax scale) in LDS, one KB per tap slot, written by one wave
+        unsigned char *bands = smem + Lds::band_off + CQT * 1024;
+        if (pr == 0) {
+#pragma unroll
+            for (int t = 0; t < CQT; ++t)
+                *reinterpret_cast<f16x8 *>(bands + t * 1024 + lane * 16) = band_frag<CQT>(t, w_head, cq, ck, pk, g, n, true, p.scale);
+        }
+        // dW: this wave takes the key blocks of two pairs (pg) and half of the tap slots (t_lo ..)
+        constexpr int TH = (CQT + 1) / 2;
+        const int pg = pr >> 1, t_lo = (pr & 1) * TH;
+        f32x4 acc_k[NDB][DB], acc_v[2][DB];
+#pragma unroll
+        for (int m = 0; m < 2; ++m)
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                acc_k[m][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
+                acc_v[m][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            }
+        f32x4 acc_w[TH][2];
+#pragma unroll
+        for (int t = 0; t < TH; ++t) acc_w[t][0] = acc_w[t][1] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        unsigned int prev_dc[NCB][2][2];
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+            for (int f = 0; f < 2; ++f) prev_dc[cb][f][0] = prev_dc[cb][f][1] = 0u;
+        const int n_kt = gridDim.z * NP, kt = blockIdx.z * NP + pr;
+        bf16_t *ds_pair = dS_ws + (bh * n_kt + kt) * (size_t)n_rt * (WK * BR);
+
+        for (int it = 0; it <= n_tiles + 1; ++it) {
+            TS(0);
+            __syncthreads();
+            TS(1);
+            if (it + 1 < n_tiles) stage_tile(it + 1);
+            load_tile(r_begin + (it + 2) * BR);
+            TS(2);
+            const int u = it - 1, v = it - 2;
+            const int r0u = r_begin + u * BR, r0v = r_begin + v * BR;
+#if defined(CHAIN_SKIP_ROLE) && CHAIN_SKIP_ROLE == 1
+            continue;
+#endif
+            const bool u_in = it >= 1 && u < n_tiles;
+            const bool u_ok = u_in && !is_skipped(r0u);
+            const bool v_ok = it >= 2 && !is_skipped(r0v);
+
+            // Order of the iteration: dV (operands of the staged tiles only, so the first MFMAs
+            // start while the dC loads are in flight), dS, dW (independent of dS: its MFMAs cover
+            // the round trip of dS through LDS), dK.
+            if (u_ok) {
+                const unsigned char *Ps = smem + opaque((unsigned int)(p_stage(u) - smem) + tr_lane_off(PST, g, n));
+                const unsigned char *Gs = smem + opaque((unsigned int)(g_slot(u) - smem) + tr_lane_off(RST, g, n));
+                __builtin_amdgcn_s_setprio(1);
+                // ---- dV^T += dO^T P (keys c0-8 .. c0+23) ----
+                bf16x8 pf[2];
+#pragma unroll
+                for (int cb = 0; cb < 2; ++cb) pf[cb] = read_tr(Ps, PST, cb * 16);
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    const bf16x8 gt = read_tr(Gs, RST, db * 16);
+#pragma unroll
+                    for (int cb = 0; cb < 2; ++cb) acc_v[cb][db] = mfma_bf16(gt, pf[cb], acc_v[cb][db]);
+                }
+            }
+            CHAIN_SCHED_BARRIER;
+            TS(3);
+            // packed dC^T of tile u, as the producer's lanes held it (zeros when the tile has none)
+            unsigned int cur_dc[NCB][2][2];
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+                for (int f = 0; f < 2; ++f) {
+                    u32x2 t2 = {0u, 0u};
+                    if (u_ok) t2 = *reinterpret_cast<const u32x2 *>(c_stage(u) + (2 * n + f) * CST + (cb * 16 + 4 * g) * 2);
+                    cur_dc[cb][f][0] = t2[0];
+                    cur_dc[cb][f][1] = t2[1];
+                }
+            if (v_ok) {
+                const bool edge = is_edge(r0v);
+                bf16_t *ds_blk = ds_pair + (size_t)(r0v / BR) * (WK * BR);
+                __builtin_amdgcn_s_setprio(1);
+                // ---- dS^T of tile v: rows below it come from tile v+1.  Operand of row offset
+                // e = parity + (CQT-1 - tap slot): fragment e & 1 shifted e >> 1 lanes up. ----
+                f32x4 ds[NDB][2];
+#pragma unroll
+                for (int sb = 0; sb < NDB; ++sb) ds[sb][0] = ds[sb][1] = (f32x4){0.f, 0.f, 0.f, 0.f};
+                f16x8 tb_prev = (f16x8)(_Float16)0.f;
+                static_for<CQT + 1>([&](auto E) {
+                    constexpr int e = decltype(E)::value, f = e & 1, s = e >> 1;
+                    // tap slot CQT-1-e for parity 0 (this step's band), CQT-e for parity 1 (the last step's)
+                    f16x8 tb_cur = tb_prev;
+                    if constexpr (e <= CQT - 1) tb_cur = *reinterpret_cast<const f16x8 *>(bands + (CQT - 1 - e) * 1024 + lane * 16);
+                    unsigned int sh[NCB][2];
+#pragma unroll
+                    for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+                        for (int dw = 0; dw < 2; ++dw) sh[cb][dw] = win_down<s>(prev_dc[cb][f][dw], cur_dc[cb][f][dw]);
+#pragma unroll
+                    for (int sb = 0; sb < NDB; ++sb) {
+                        const u32x4 bv = {sh[sb][0], sh[sb][1], sh[sb + 1][0], sh[sb + 1][1]};
+                        if constexpr (e <= CQT - 1) ds[sb][0] = mfma_f16(tb_cur, __builtin_bit_cast(f16x8, bv), ds[sb][0]);
+                        if constexpr (e >= 1) ds[sb][1] = mfma_f16(tb_prev, __builtin_bit_cast(f16x8, bv), ds[sb][1]);
+                    }
+                    tb_prev = tb_cur;
+                });
+#pragma unroll
+                for (int sb = 0; sb < NDB; ++sb)
+#pragma unroll
+                    for (int ob = 0; ob < 2; ++ob) {
+                        if (edge && causal) {
+#pragma unroll
+                            for (int r = 0; r < 4; ++r)
+                                if (c0 + sb * 16 + 4 * g + r > r0v + 2 * n + ob) ds[sb][ob][r] = 0.f;
+                        }
+                        bf16x4 sv;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) sv[r] = (bf16_t)ds[sb][ob][r];
+                        *reinterpret_cast<bf16x4 *>(ds_blk + (2 * n + ob) * WK + sb * 16 + 4 * g) = sv;
+                        *reinterpret_cast<bf16x4 *>(ds_tile + (2 * n + ob) * PST + (sb * 16 + 4 * g) * 2) = sv;
+                    }
+            }
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+                for (int f = 0; f < 2; ++f) { prev_dc[cb][f][0] = cur_dc[cb][f][0]; prev_dc[cb][f][1] = cur_dc[cb][f][1]; }
+            CHAIN_SCHED_BARRIER;
+            TS(4);
+            // ---- dW, key blocks jb = 0..3 of the pairs 2 pg and 2 pg + 1 (block jb = dC block jb & 1 of
+            // pair 2 pg + jb / 2, keys k0 + 64 pg - 8 + 16 jb ..), tap slots t_lo .. t_lo + TH - 1:
+            // G_t[j][j'] += sum_rows dC[row][j] S[row + t - (CQT-1)][j'] with j' in the score block
+            // 8 keys before the dC block (x = 0) and the one 8 keys after it (x = 1) ----
+            if (u_in) {
+                // Ring rows of this lane's two transpose reads at the wave's first tap slot: tile row 0
+                // at tap slot 0 is ring row wbase; the TH tap slots are consecutive rows (mod S_RING).
+                const int wbase = ((u + 1) * BR - (CQT - 1) + S_RING) % S_RING;
+                const unsigned int c_lane = opaque(tr_lane_off(CST, g, n));
+                const unsigned int ring0 = Lds::pair_off + 2 * pg * Lds::pair_bytes + 4 * (n & 3) * 2;
+                unsigned int a_lo[TH], a_hi[TH];
+#pragma unroll
+                for (int tt = 0; tt < TH; ++tt) {
+                    const unsigned int ra = wbase + 4 * g + (n >> 2) + min(t_lo + tt, CQT - 1), rb = ra + 16;
+                    a_lo[tt] = opaque(ring0 + min(ra, ra - S_RING) * SST);
+                    a_hi[tt] = opaque(ring0 + min(rb, rb - S_RING) * SST);
+                }
+                // score block jb' = 0..4 of the group: block jb' & 1 (or 2 for the last) of pair 2 pg + jb' / 2
+                auto s_frag = [&](int jbp, int tt) {
+                    const int dq = min(jbp >> 1, NP - 1 - 2 * pg), kb = jbp - 2 * dq;   // dq: wave-uniform
+                    bf16x4 l4 = lds_tr64(smem + a_lo[tt] + dq * Lds::pair_bytes + kb * 32);
+                    bf16x4 h4 = lds_tr64(smem + a_hi[tt] + dq * Lds::pair_bytes + kb * 32);
+                    return __builtin_bit_cast(f16x8, __builtin_shufflevector(l4, h4, 0, 1, 2, 3, 4, 5, 6, 7));
+                };
+                // dC^T block jb of the group (zeros where the pair's tile is entirely above the diagonal:
+                // its dC buffer was not written)
+                auto c_frag = [&](int jb) {
+                    const int dq = jb >> 1;
+                    const bool has = !(causal && r0u + BR - 1 < k0 + (2 * pg + dq) * WK - 8);
+                    const f16x8 v = __builtin_bit_cast(
+                        f16x8, read_tr(smem + Lds::pair_off + 2 * pg * Lds::pair_bytes + Lds::s_bytes + (u & 1) * (BR * CST) +
+                                           c_lane + dq * Lds::pair_bytes, CST, (jb & 1) * 16));
+                    return has ? v : (f16x8)(_Float16)0.f;
+                };
+                // Software pipeline over the four key blocks: the operands of block jb + 1 are read
+                // while block jb is multiplied.  Every tap slot of the wave is multiplied, also the
+                // zero taps in front of a narrow window (their sums are not used).
+                f16x8 af = c_frag(0), b0[TH], b1[TH];
+#pragma unroll
+                for (int tt = 0; tt < TH; ++tt) { b0[tt] = s_frag(0, tt); b1[tt] = s_frag(1, tt); }
+                static_for<4>([&](auto JB) {
+                    constexpr int jb = decltype(JB)::value;
+                    f16x8 af_n = af, b2[TH];
+#pragma unroll
+                    for (int tt = 0; tt < TH; ++tt) b2[tt] = b1[tt];
+                    if constexpr (jb < 3) {
+                        af_n = c_frag(jb + 1);
+#pragma unroll
+                        for (int tt = 0; tt < TH; ++tt) b2[tt] = s_frag(jb + 2, tt);
+                        SCHED_DS_READ_ID(2 + 2 * TH, 40 + jb);
+                    }
+#pragma unroll
+                    for (int tt = 0; tt < TH; ++tt) {
+                        acc_w[tt][0] = mfma_f16(af, b0[tt], acc_w[tt][0]);
+                        acc_w[tt][1] = mfma_f16(af, b1[tt], acc_w[tt][1]);
+                    }
+                    SCHED_MFMA_ID(2 * TH, 40 + jb);
+                    af = af_n;
+#pragma unroll
+                    for (int tt = 0; tt < TH; ++tt) { b0[tt] = b1[tt]; b1[tt] = b2[tt]; }
+                });
+            }
+            CHAIN_SCHED_BARRIER;
+            TS(5);
+            if (v_ok) {
+                const unsigned char *Qs = smem + opaque((unsigned int)(q_slot(v) - smem) + tr_lane_off(RST, g, n));
+                const unsigned char *Dsl = smem + opaque((unsigned int)(ds_tile - smem) + tr_lane_off(PST, g, n));
+                asm volatile("" ::: "memory");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_s_setprio(1);
+                // ---- dK^T += Q^T dS ----
+                {
+                    bf16x8 sf[2];
+#pragma unroll
+                    for (int sb = 0; sb < 2; ++sb) sf[sb] = read_tr(Dsl, PST, sb * 16);
+#pragma unroll
+                    for (int db = 0; db < DB; ++db) {
+                        const bf16x8 qt = read_tr(Qs, RST, db * 16);
+#pragma unroll
+                        for (int sb = 0; sb < 2; ++sb) acc_k[sb][db] = mfma_bf16(qt, sf[sb], acc_k[sb][db]);
+                    }
+                }
+                asm volatile("" ::: "memory");
+                __builtin_amdgcn_wave_barrier();
+            }
+            __builtin_amdgcn_s_setprio(0);
+            TS(6);
+        }
+
+        // ---- stores: lane = key, 4 consecutive head-dim columns per block ----
+        const float inv = 1.f / dcs;
+#pragma unroll
+        for (int m = 0; m < 2; ++m) {
+            const int key_k = c0 + m * 16 + n;
+            const int key_v = c0 - 8 + m * 16 + n;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                const int col = db * 16 + 4 * g;
+                if (key_k < p.Nk) {
+                    TO *dst = dK + (bh * p.Nk + key_k) * D + col;
+                    if constexpr (sizeof(TO) == 2) {
+                        bf16x4 ov;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) ov[r] = (bf16_t)(acc_k[m][db][r] * inv);
+                        *reinterpret_cast<bf16x4 *>(dst) = ov;
+                    } else {
+                        *reinterpret_cast<f32x4 *>(dst) = acc_k[m][db] * inv;
+                    }
+                }
+                if (key_v >= 0 && key_v < p.Nk) {
+                    TO *dst = dV + (bh * p.Nk + key_v) * D + col;
+                    if constexpr (sizeof(TO) == 2) {
+                        bf16x4 ov;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) ov[r] = (bf16_t)(acc_v[m][db][r] * inv);
+                        *reinterpret_cast<bf16x4 *>(dst) = ov;
+                    } else {
+                        *reinterpret_cast<f32x4 *>(dst) = acc_v[m][db] * inv;
+                    }
+                }
+            }
+        }
+
+        // ---- dW accumulators of this wave to LDS as [pair group][tap slot][x][m][n], once every
+        // wave is done with the tiles ----
+        __syncthreads();
+        float *red = reinterpret_cast<float *>(smem + Lds::pair_off);
+#pragma unroll
+        for (int tt = 0; tt < TH; ++tt)
+#pragma unroll
+            for (int x = 0; x < 2; ++x)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (t_lo + tt < CQT)
+                        red[(((pg * CQT + t_lo + tt) * 2 + x) * 16 + 4 * g + r) * 16 + n] = acc_w[tt][x][r];
+    }  // consumer
+
+    // ---- dW partial of this workgroup: G[m][n] of half x belongs to key tap b = n - m + 16 x - 8 + pk;
+    // the sum runs over the pair groups, the halves and the diagonals' elements in a fixed order.
+    // S was raw, so * scale; dC was scaled, so / dcs. ----
+    static_assert(2 * CQT * 2 * 1024 <= NP * ChainLds<D, CQT>::pair_bytes, "room for the dW accumulators");
+    __syncthreads();
+    const int ntap = cq * ck;
+    if (tid < ntap) {
+        const int a = tid / ck, bb = tid - a * ck, t = a + CQT - cq;
+        const float *red = reinterpret_cast<const float *>(smem + Lds::pair_off);
+        float sum = 0.f;
+        for (int pgi = 0; pgi < 2; ++pgi)
+            for (int x = 0; x < 2; ++x)
+                for (int m = 0; m < 16; ++m) {
+                    const int nn = bb + m - 16 * x + 8 - pk;
+                    if (nn >= 0 && nn < 16) sum += red[(((pgi * CQT + t) * 2 + x) * 16 + m) * 16 + nn];
+                }
+        dW_part[(bh * gridDim.z + blockIdx.z) * ntap + tid] = sum * p.scale / dcs;
+    }
+}
+
+template <int D, int CQT, typename TO>
+__global__ __launch_bounds__(NT) void bwd_chain_kernel(ChainArgs args) {
+    // `args` is the whole argument segment; the roles read it from there
+#if defined(__HIP_DEVICE_COMPILE__)
+    const CHAIN_CONST_AS ChainArgs *ap =
+        (const CHAIN_CONST_AS ChainArgs *)__builtin_amdgcn_kernarg_segment_ptr();
+#else
+    const ChainArgs *ap = &args;
+#endif
+    if (__builtin_amdgcn_readfirstlane(threadIdx.x >> 6) < NP) chain_role<D, CQT, TO, 0>(ap);
+    else chain_role<D, CQT, TO, 1>(ap);
+}
+
+// amax|dO| and amax|V| of one (batch, head) -> {s, log2 s}, s the power of two that brings
+// sqrt(d) * amax|dO| * amax|V| (a few times a typical |dP|) to about 2^12.
+__global__ __launch_bounds__(256) void dc_scale_kernel(int Nq, int Nk, int d, const bf16_t *__restrict__ dO,
+                                                       const bf16_t *__restrict__ V, float *__restrict__ out) {
+    const size_t bh = blockIdx.x;
+    __shared__ float red[2][4];
+    float mx[2] = {0.f, 0.f};
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+        const size_t cnt = (size_t)(which ? Nk : Nq) * d / 8;
+        const u32x4 *src = reinterpret_cast<const u32x4 *>((which ? V : dO) + bh * (which ? Nk : Nq) * (size_t)d);
+        unsigned int m = 0;
+        for (size_t i = threadIdx.x; i < cnt; i += 256) {
+            const u32x4 v = src[i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                m = max(m, (v[j] << 16) & 0x7fffffffu);
+                m = max(m, v[j] & 0x7fff0000u);
+            }
+        }
+        mx[which] = wave_max(__uint_as_float(m));
+        if ((threadIdx.x & 63) == 0) red[which][threadIdx.x >> 6] = mx[which];
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const float a = fmaxf(fmaxf(red[0][0], red[0][1]), fmaxf(red[0][2], red[0][3]));
+        const float v = fmaxf(fmaxf(red[1][0], red[1][1]), fmaxf(red[1][2], red[1][3]));
+        const float prod = sqrtf((float)d) * a * v;
+        float e = 0.f;
+        if (prod > 0.f && prod < 3e38f) e = fminf(fmaxf(floorf(12.f - log2f(prod)), -60.f), 60.f);
+        out[2 * bh] = exp2f(e);
+        out[2 * bh + 1] = e;
+    }
+}
+
+template <int D, int CQT, typename TO>
+hipError_t launch_chain(const Problem &p, const void *q, const void *k, const void *v, const void *d_o,
+                        const float *Dl, const float *lse, const float *w, const float *dc_scale, void *dk,
+                        void *dv, void *ds_ws, float *dw_part, hipStream_t s) {
+    auto kern = bwd_chain_kernel<D, CQT, TO>;
+    constexpr int lds = ChainLds<D, CQT>::total;
+    static_assert(lds <= 160 * 1024, "LDS budget");
+    static bool attr_set = false;  // per kernel instantiation; the attribute is sticky
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    dim3 grid(p.H, p.B, mfma_kv_tiles(p));
+    ChainArgs args{p, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, (const bf16_t *)d_o, Dl, lse, w,
+                   dc_scale, dk, dv, (bf16_t *)ds_ws, dw_part, chain_row_tiles(p)};
+    kern<<<grid, NT, lds, s>>>(args);
+    return hipGetLastError();
+}
+
+template <int D, typename TO>
+hipError_t pick_cq(const Problem &p, const void *q, const void *k, const void *v, const void *d_o,
+                   const float *Dl, const float *lse, const float *w, const float *dc_scale, void *dk, void *dv,
+                   void *ds_ws, float *dw_part, hipStream_t s) {
+    if (p.c_q <= 3) return launch_chain<D, 3, TO>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
+    return launch_chain<D, 6, TO>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
+}
+
+}  // namespace
+
+#ifdef CHAIN_TS
+extern "C" int convattn_debug_chain_ts(long long *host) {
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_chain_ts), sizeof(long long) * 8 * 64 * 12);
+}
+#endif
+
+hipError_t mfma_dc_scale(const Problem &p, const void *d_o, const void *v, float *dc_scale, hipStream_t s) {
+    dc_scale_kernel<<<dim3(p.B * p.H), 256, 0, s>>>(p.Nq, p.Nk, p.d, (const bf16_t *)d_o, (const bf16_t *)v, dc_scale);
+    return hipGetLastError();
+}
+
+hipError_t mfma_bwd_chain(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
+                          const void *d_o, const float *Dl, const float *lse, const float *w,
+                          const float *dc_scale, void *dk, void *dv, void *ds_ws, float *dw_part, hipStream_t s) {
+    if (p.d == 128) {
+        if (out_dt == CONVATTN_BF16) return pick_cq<128, bf16_t>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
+        return pick_cq<128, float>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
+    }
+    if (out_dt == CONVATTN_BF16) return pick_cq<64, bf16_t>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
+    return pick_cq<64, float>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
+}
+
+}  // namespace convattn

@@ -215,6 +215,26 @@ hipError_t mfma_bwd_fused_ws(const Problem &p, int out_dt, const void *q, const 
 hipError_t mfma_dq_from_ds(const Problem &p, int out_dt, const void *k, const void *ds_ws, void *dq,
                            hipStream_t s);
 
+// ---- whole backward with the score chain in registers (bwd_chain_mfma.hip, bwd_dq_rows.hip) ----
+// Windows of up to 6 query taps.  The key-stationary kernel's workgroups cover 128 keys each (+ 8:
+// the dV ranges start 8 keys early); it leaves one dW partial per workgroup and dS as bf16 blocks
+// [key tile of 32][row tile of 32][32 rows][32 keys], which mfma_dq_from_rows multiplies with K.
+// dc_scale holds {s, log2 s} per (batch, head): the power of two dC is carried at (mfma_dc_scale).
+constexpr int kChainKeys = 32, kChainRows = 32, kChainMaxCq = 6;
+inline bool chain_ok(const Problem &p) { return p.c_q <= kChainMaxCq; }
+inline int chain_key_tiles(const Problem &p) { return mfma_kv_tiles(p) * (kKvKeysPerWg / kChainKeys); }
+__host__ __device__ inline int chain_row_tiles(const Problem &p) { return (p.Nq + kChainRows - 1) / kChainRows; }
+inline size_t chain_ds_bytes(const Problem &p) {
+    return (size_t)p.B * p.H * chain_key_tiles(p) * chain_row_tiles(p) * kChainKeys * kChainRows * 2;
+}
+inline size_t chain_scale_bytes(const Problem &p) { return (size_t)p.B * p.H * 2 * sizeof(float); }
+hipError_t mfma_dc_scale(const Problem &p, const void *d_o, const void *v, float *dc_scale, hipStream_t s);
+hipError_t mfma_bwd_chain(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
+                          const void *d_o, const float *Dl, const float *lse, const float *w,
+                          const float *dc_scale, void *dk, void *dv, void *ds_ws, float *dw_part, hipStream_t s);
+hipError_t mfma_dq_from_rows(const Problem &p, int out_dt, const void *k, const void *ds_ws,
+                             const float *dc_scale, void *dq, hipStream_t s);
+
 // ---- decode as an HBM stream (decode_stream.hip) ----
 bool decode_stream_ok(const Problem &p, int in_dt, unsigned flags);
 hipError_t decode_stream(const Problem &p, const void *q, const void *k, const void *v, const float *w,

@@ -283,9 +283,9 @@ def test_c3_full_size_fwd_bwd_against_fp32_kernels():
     assert max_abs(dK, dK_x) <= TOL_BF16
     assert max_abs(dV, dV_x) <= TOL_BF16
     assert rel_max(dW, dW_x) <= TOL_DW_REL
-    # the one-pass backward: same tiles, same arithmetic for dK / dV; dQ and dW in another order
+    # the one-pass backward: another kernel (the score chain stays in registers)
     dQ1, dK1, dV1, dW1 = ops.backward(Q, K, V, dO, D, LSE, W, *args, out_dtype=torch.bfloat16)
-    assert torch.equal(dK1, dK) and torch.equal(dV1, dV)
+    assert max_abs(dK1, dK_x) <= TOL_BF16 and max_abs(dV1, dV_x) <= TOL_BF16
     assert max_abs(dQ1, dQ_x) <= TOL_BF16 and rel_max(dW1, dW_x) <= TOL_DW_REL
     # dV is linear in dO, dQ/dK/dW are too: doubling dO doubles them (D doubles with it)
     dQ2, dW2 = ops.dq_backward(Q, K, V, (2 * dO.float()).to(torch.bfloat16), 2 * D, LSE, W, *args,
