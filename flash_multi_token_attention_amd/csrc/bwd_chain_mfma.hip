@@ -152,6 +152,9 @@ __device__ __forceinline__ f16x8 band_frag(int t, const float *__restrict__ w_he
     return f;
 }
 
+#ifndef CHAIN_ABLATE
+#define CHAIN_ABLATE 0
+#endif
 #ifdef CHAIN_PHASE_BARRIERS
 #define CHAIN_SCHED_BARRIER __builtin_amdgcn_sched_barrier(0)
 #else
@@ -262,6 +265,7 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
     // (the thread's chunk coordinates are recomputed from an opaque copy of its index at every use:
     // kept in registers across the tile loop they are what the register allocator spills first)
     auto load_tile = [&](int r0) {
+        if (CHAIN_ABLATE & 256) return;
         const int tt = (int)opaque((unsigned int)tid);
 #pragma unroll
         for (int i = 0; i < LD; ++i) {
@@ -275,6 +279,7 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
         }
     };
     auto stage_tile = [&](int t) {
+        if (CHAIN_ABLATE & 256) return;
         const int tt = (int)opaque((unsigned int)tid);
         unsigned char *Qs = q_slot(t), *Gs = g_slot(t);
 #pragma unroll
@@ -333,7 +338,7 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
 #pragma unroll
                 for (int f = 0; f < 2; ++f) acc[kb][f] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
+            for (int ks = 0; ks < ((CHAIN_ABLATE & 64) ? 0 : KS); ++ks) {
                 bf16x8 qf[2];
 #pragma unroll
                 for (int f = 0; f < 2; ++f) qf[f] = load_qf(f, ks);
@@ -397,7 +402,7 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
                 // MFMAs run back to back with those of S^T ----
                 f32x4 dp[NCB][2];
                 float2 l2 = {0.f, 0.f};
-                if constexpr (FULL) {
+                if constexpr (FULL && !(CHAIN_ABLATE & 32)) {
                     const float *st = stat_slot(it);
                     l2 = *reinterpret_cast<const float2 *>(st + 2 * n);
                     const float2 d2 = *reinterpret_cast<const float2 *>(st + BR + 2 * n);
@@ -439,7 +444,7 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
                         c[cb][1] = (f32x4){-l2.y, -l2.y, -l2.y, -l2.y};
                     }
                     f16x8 tf_prev = (f16x8)(_Float16)0.f;
-                    static_for<CQT + 1>([&](auto DL) {
+                    static_for<(CHAIN_ABLATE & 16) ? 0 : CQT + 1>([&](auto DL) {
                         constexpr int t0 = decltype(DL)::value;
                         constexpr int delta = t0 - (CQT - 1);
                         constexpr int f = delta & 1, s = (f - delta) / 2;
@@ -465,7 +470,7 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
                     CHAIN_SCHED_BARRIER;
                     TS(5);
                     // ---- P = exp2(C - LSE) (times the dC scale), dC = P dP ----
-                    static_for<NCB>([&](auto CB) {
+                    static_for<(CHAIN_ABLATE & 128) ? 0 : NCB>([&](auto CB) {
                         constexpr int cb = decltype(CB)::value;
                         __builtin_amdgcn_s_setprio(0);
 #pragma unroll
@@ -558,7 +563,7 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
             // Order of the iteration: dV (operands of the staged tiles only, so the first MFMAs
             // start while the dC loads are in flight), dS, dW (independent of dS: its MFMAs cover
             // the round trip of dS through LDS), dK.
-            if (u_ok) {
+            if (u_ok && !(CHAIN_ABLATE & 4)) {
                 const unsigned char *Ps = smem + opaque((unsigned int)(p_stage(u) - smem) + tr_lane_off(PST, g, n));
                 const unsigned char *Gs = smem + opaque((unsigned int)(g_slot(u) - smem) + tr_lane_off(RST, g, n));
                 __builtin_amdgcn_s_setprio(1);
@@ -577,16 +582,20 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
             TS(3);
             // packed dC^T of tile u, as the producer's lanes held it (zeros when the tile has none)
             unsigned int cur_dc[NCB][2][2];
+            {
+                // read unconditionally (a buffer of this workgroup; its contents mean nothing when the
+                // tile has no dC), then cleared: no branch per load
+                const unsigned char *Cl = smem + opaque((unsigned int)(c_stage(max(u, 0)) - smem) + 2 * n * CST + 4 * g * 2);
 #pragma unroll
-            for (int cb = 0; cb < NCB; ++cb)
+                for (int cb = 0; cb < NCB; ++cb)
 #pragma unroll
-                for (int f = 0; f < 2; ++f) {
-                    u32x2 t2 = {0u, 0u};
-                    if (u_ok) t2 = *reinterpret_cast<const u32x2 *>(c_stage(u) + (2 * n + f) * CST + (cb * 16 + 4 * g) * 2);
-                    cur_dc[cb][f][0] = t2[0];
-                    cur_dc[cb][f][1] = t2[1];
-                }
-            if (v_ok) {
+                    for (int f = 0; f < 2; ++f) {
+                        const u32x2 t2 = *reinterpret_cast<const u32x2 *>(Cl + f * CST + cb * 32);
+                        cur_dc[cb][f][0] = u_ok ? t2[0] : 0u;
+                        cur_dc[cb][f][1] = u_ok ? t2[1] : 0u;
+                    }
+            }
+            if (v_ok && !(CHAIN_ABLATE & 512)) {
                 const bool edge = is_edge(r0v);
                 bf16_t *ds_blk = ds_pair + (size_t)(r0v / BR) * (WK * BR);
                 __builtin_amdgcn_s_setprio(1);
@@ -596,7 +605,7 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
 #pragma unroll
                 for (int sb = 0; sb < NDB; ++sb) ds[sb][0] = ds[sb][1] = (f32x4){0.f, 0.f, 0.f, 0.f};
                 f16x8 tb_prev = (f16x8)(_Float16)0.f;
-                static_for<CQT + 1>([&](auto E) {
+                static_for<(CHAIN_ABLATE & 2) ? 0 : CQT + 1>([&](auto E) {
                     constexpr int e = decltype(E)::value, f = e & 1, s = e >> 1;
                     // tap slot CQT-1-e for parity 0 (this step's band), CQT-e for parity 1 (the last step's)
                     f16x8 tb_cur = tb_prev;
@@ -640,7 +649,7 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
             // pair 2 pg + jb / 2, keys k0 + 64 pg - 8 + 16 jb ..), tap slots t_lo .. t_lo + TH - 1:
             // G_t[j][j'] += sum_rows dC[row][j] S[row + t - (CQT-1)][j'] with j' in the score block
             // 8 keys before the dC block (x = 0) and the one 8 keys after it (x = 1) ----
-            if (u_in) {
+            if (u_in && !(CHAIN_ABLATE & 1)) {
                 // Ring rows of this lane's two transpose reads at the wave's first tap slot: tile row 0
                 // at tap slot 0 is ring row wbase; the TH tap slots are consecutive rows (mod S_RING).
                 const int wbase = ((u + 1) * BR - (CQT - 1) + S_RING) % S_RING;
@@ -700,7 +709,7 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
             }
             CHAIN_SCHED_BARRIER;
             TS(5);
-            if (v_ok) {
+            if (v_ok && !(CHAIN_ABLATE & 8)) {
                 const unsigned char *Qs = smem + opaque((unsigned int)(q_slot(v) - smem) + tr_lane_off(RST, g, n));
                 const unsigned char *Dsl = smem + opaque((unsigned int)(ds_tile - smem) + tr_lane_off(PST, g, n));
                 asm volatile("" ::: "memory");
@@ -807,18 +816,21 @@ __global__ __launch_bounds__(NT) void bwd_chain_kernel(ChainArgs args) {
 }
 
 // amax|dO| and amax|V| of one (batch, head) -> {s, log2 s}, s the power of two that brings
-// sqrt(d) * amax|dO| * amax|V| (a few times a typical |dP|) to about 2^12.
-__global__ __launch_bounds__(256) void dc_scale_kernel(int Nq, int Nk, int d, const bf16_t *__restrict__ dO,
-                                                       const bf16_t *__restrict__ V, float *__restrict__ out) {
-    const size_t bh = blockIdx.x;
+// sqrt(d) * amax|dO| * amax|V| (a few times a typical |dP|) to about 2^12.  Two steps: kScaleChunks
+// workgroups per (batch, head) leave their maxima in `part`, one thread per (batch, head) finishes.
+constexpr int kScaleChunks = 32;
+__global__ __launch_bounds__(256) void dc_scale_partial_kernel(int Nq, int Nk, int d, const bf16_t *__restrict__ dO,
+                                                               const bf16_t *__restrict__ V, float *__restrict__ part) {
+    const size_t bh = blockIdx.y;
     __shared__ float red[2][4];
-    float mx[2] = {0.f, 0.f};
 #pragma unroll
     for (int which = 0; which < 2; ++which) {
-        const size_t cnt = (size_t)(which ? Nk : Nq) * d / 8;
+        const size_t cnt = (size_t)(which ? Nk : Nq) * d / 8;   // 16-byte pieces of the slab
+        const size_t per = (cnt + kScaleChunks - 1) / kScaleChunks;
+        const size_t lo = blockIdx.x * per, hi = lo + per < cnt ? lo + per : cnt;
         const u32x4 *src = reinterpret_cast<const u32x4 *>((which ? V : dO) + bh * (which ? Nk : Nq) * (size_t)d);
         unsigned int m = 0;
-        for (size_t i = threadIdx.x; i < cnt; i += 256) {
+        for (size_t i = lo + threadIdx.x; i < hi; i += 256) {
             const u32x4 v = src[i];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -826,19 +838,28 @@ __global__ __launch_bounds__(256) void dc_scale_kernel(int Nq, int Nk, int d, co
                 m = max(m, v[j] & 0x7fff0000u);
             }
         }
-        mx[which] = wave_max(__uint_as_float(m));
-        if ((threadIdx.x & 63) == 0) red[which][threadIdx.x >> 6] = mx[which];
+        // NaN / Inf inputs (exponent all ones) are left out of the maximum: they poison the results anyway
+        const float mx = wave_max(m < 0x7f800000u ? __uint_as_float(m) : 0.f);
+        if ((threadIdx.x & 63) == 0) red[which][threadIdx.x >> 6] = mx;
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-        const float a = fmaxf(fmaxf(red[0][0], red[0][1]), fmaxf(red[0][2], red[0][3]));
-        const float v = fmaxf(fmaxf(red[1][0], red[1][1]), fmaxf(red[1][2], red[1][3]));
-        const float prod = sqrtf((float)d) * a * v;
-        float e = 0.f;
-        if (prod > 0.f && prod < 3e38f) e = fminf(fmaxf(floorf(12.f - log2f(prod)), -60.f), 60.f);
-        out[2 * bh] = exp2f(e);
-        out[2 * bh + 1] = e;
+    if (threadIdx.x < 2)
+        part[(bh * kScaleChunks + blockIdx.x) * 2 + threadIdx.x] =
+            fmaxf(fmaxf(red[threadIdx.x][0], red[threadIdx.x][1]), fmaxf(red[threadIdx.x][2], red[threadIdx.x][3]));
+}
+__global__ void dc_scale_finish_kernel(int n_bh, int d, const float *__restrict__ part, float *__restrict__ out) {
+    const int bh = blockIdx.x * blockDim.x + threadIdx.x;
+    if (bh >= n_bh) return;
+    float a = 0.f, v = 0.f;
+    for (int c = 0; c < kScaleChunks; ++c) {
+        a = fmaxf(a, part[((size_t)bh * kScaleChunks + c) * 2]);
+        v = fmaxf(v, part[((size_t)bh * kScaleChunks + c) * 2 + 1]);
     }
+    const float prod = sqrtf((float)d) * a * v;
+    float e = 0.f;
+    if (prod > 0.f && prod < 3e38f) e = fminf(fmaxf(floorf(12.f - log2f(prod)), -60.f), 60.f);
+    out[2 * bh] = exp2f(e);
+    out[2 * bh + 1] = e;
 }
 
 template <int D, int CQT, typename TO>
@@ -879,7 +900,13 @@ extern "C" int convattn_debug_chain_ts(long long *host) {
 #endif
 
 hipError_t mfma_dc_scale(const Problem &p, const void *d_o, const void *v, float *dc_scale, hipStream_t s) {
-    dc_scale_kernel<<<dim3(p.B * p.H), 256, 0, s>>>(p.Nq, p.Nk, p.d, (const bf16_t *)d_o, (const bf16_t *)v, dc_scale);
+    // dc_scale holds {s, log2 s} per (batch, head), then the partial maxima
+    float *part = dc_scale + (size_t)p.B * p.H * 2;
+    dc_scale_partial_kernel<<<dim3(kScaleChunks, p.B * p.H), 256, 0, s>>>(p.Nq, p.Nk, p.d, (const bf16_t *)d_o,
+                                                                          (const bf16_t *)v, part);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    dc_scale_finish_kernel<<<dim3((p.B * p.H + 255) / 256), 256, 0, s>>>(p.B * p.H, p.d, part, dc_scale);
     return hipGetLastError();
 }
 

@@ -221,13 +221,14 @@ hipError_t mfma_dq_from_ds(const Problem &p, int out_dt, const void *k, const vo
 // [key tile of 32][row tile of 32][32 rows][32 keys], which mfma_dq_from_rows multiplies with K.
 // dc_scale holds {s, log2 s} per (batch, head): the power of two dC is carried at (mfma_dc_scale).
 constexpr int kChainKeys = 32, kChainRows = 32, kChainMaxCq = 6;
-inline bool chain_ok(const Problem &p) { return p.c_q <= kChainMaxCq; }
+inline bool chain_ok(const Problem &p) { return p.c_q <= kChainMaxCq && (long long)p.B * p.H <= 65535; }
 inline int chain_key_tiles(const Problem &p) { return mfma_kv_tiles(p) * (kKvKeysPerWg / kChainKeys); }
 __host__ __device__ inline int chain_row_tiles(const Problem &p) { return (p.Nq + kChainRows - 1) / kChainRows; }
 inline size_t chain_ds_bytes(const Problem &p) {
     return (size_t)p.B * p.H * chain_key_tiles(p) * chain_row_tiles(p) * kChainKeys * kChainRows * 2;
 }
-inline size_t chain_scale_bytes(const Problem &p) { return (size_t)p.B * p.H * 2 * sizeof(float); }
+// {s, log2 s} per (batch, head) followed by 32 x 2 partial maxima per (batch, head)
+inline size_t chain_scale_bytes(const Problem &p) { return (size_t)p.B * p.H * (2 + 64) * sizeof(float); }
 hipError_t mfma_dc_scale(const Problem &p, const void *d_o, const void *v, float *dc_scale, hipStream_t s);
 hipError_t mfma_bwd_chain(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
                           const void *d_o, const float *Dl, const float *lse, const float *w,

@@ -106,9 +106,9 @@ def test_dw_partial_size_matches_tiling(lib):
 def test_fused_backward_workspace_size(lib):
     # bf16, N = 128, d = 64, 6 query taps: dS blocks of 32 rows x 32 keys bf16 for ceil((128 + 8) / 128) * 4
     # key tiles x ceil(128 / 32) row tiles per (batch, head), then one dW partial per 128-key workgroup,
-    # then {scale, log2 scale} of dC per (batch, head); each part 256-aligned
+    # then {scale, log2 scale} of dC and 32 x 2 partial maxima per (batch, head); each part 256-aligned
     n = lib.convattn_bwd_fused_workspace_bytes(C.byref(desc()))
-    assert n == 2 * 4 * 8 * 4 * 32 * 32 * 2 + (2 * 4 * 2 * 66 * 4 + 255) // 256 * 256 + 256
+    assert n == 2 * 4 * 8 * 4 * 32 * 32 * 2 + (2 * 4 * 2 * 66 * 4 + 255) // 256 * 256 + (2 * 4 * 66 * 4 + 255) // 256 * 256
     # more than 6 query taps: dS blocks of 32 keys x 64 rows for 8 key tiles x ceil((128 + 16) / 64) row
     # tiles, then the dW partials
     n = lib.convattn_bwd_fused_workspace_bytes(C.byref(desc(c_q=8)))
