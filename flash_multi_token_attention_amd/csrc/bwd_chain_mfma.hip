@@ -360,8 +360,15 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
                                 if (key0 + r > qpos) acc[kb][f][r] = 0.f;
                         }
                     }
-                    pd[kb][f][0] = pack_f16_rtz(acc[kb][f][0], acc[kb][f][1]);
-                    pd[kb][f][1] = pack_f16_rtz(acc[kb][f][2], acc[kb][f][3]);
+                    // rounded and clamped exactly as the forward rounds its scores: P = exp2(C - LSE)
+                    // only sums to one over a row if C is the C the forward's LSE was taken from
+                    f16x4 hv;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        hv[r] = (_Float16)__builtin_amdgcn_fmed3f(acc[kb][f][r], -kF16Max, kF16Max);
+                    const u32x2 two = __builtin_bit_cast(u32x2, hv);
+                    pd[kb][f][0] = two[0];
+                    pd[kb][f][1] = two[1];
                     if (kb < 3) {
                         const int rr = rbase + 2 * n + f;
                         *reinterpret_cast<u32x2 *>(s_ring + (rr >= S_RING ? rr - S_RING : rr) * SST + (kb * 16 + 4 * g) * 2) =
