@@ -49,6 +49,8 @@ _SIGNATURES = {
     "convattn_decode": (C.c_int, [_D] + [_P] * 8),
     "convattn_decode_strided": (C.c_int, [_D] + [_P] * 4 + [C.c_longlong] * 2 + [_P] * 4),
     "convattn_decode_combine": (C.c_int, [_D] + [_P] * 7),
+    "convattn_decode_noalloc_bytes": (C.c_size_t, [_D]),
+    "convattn_decode_noalloc": (C.c_int, [_D] + [_P] * 4 + [C.c_longlong] * 2 + [_P] * 4),
 }
 EXPORTS = tuple(_SIGNATURES)
 

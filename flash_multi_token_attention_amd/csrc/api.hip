@@ -3,6 +3,8 @@
 #include <math.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "common.hpp"
 #include "mfma_common.hpp"
 
@@ -62,6 +64,31 @@ size_t fused_dw_bytes(const Problem &p) {
     return (size_t)p.B * p.H * mfma_kv_tiles(p) * p.c_q * p.c_k * sizeof(float);
 }
 
+// Scratch of convattn_decode_noalloc: the split partials of one decode step, held by every GPU
+// the library runs on until the process ends.  Host code reaches it only through the address
+// hipGetSymbolAddress returns for the current device (kept per device).
+constexpr size_t kDecodeScratchBytes = CONVATTN_DECODE_NOALLOC_MAX_BYTES;
+static __device__ __align__(256) unsigned char scratch[kDecodeScratchBytes];
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device (looked up once per device); hipError_t in *err.
+void *decode_scratch(hipError_t *err) {
+    int dev = -1;
+    *err = hipGetDevice(&dev);
+    if (*err != hipSuccess) return nullptr;
+    if (dev < 0 || dev >= kMaxDevices) { *err = hipErrorInvalidDevice; return nullptr; }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        *err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (*err != hipSuccess) return nullptr;
+        g_scratch_ptr[dev] = ptr;
+    }
+    return g_scratch_ptr[dev];
+}
+
 #define REQUIRE_PTR(x)                                   \
     do {                                                 \
         if (!(x)) return CONVATTN_ERR_NULL;              \
@@ -89,6 +116,7 @@ const char *convattn_strerror(int code) {
         case CONVATTN_ERR_CAUSAL_SHAPE: return "causal conv-attention needs seq_len_q == seq_len_k";
         case CONVATTN_ERR_LDS: return "convolution window too large for the 160 KB of LDS at this head dimension";
         case CONVATTN_ERR_TOO_LARGE: return "batch or head count too large for one launch";
+        case CONVATTN_ERR_SCRATCH: return "the split partials of this decode step do not fit the library's built-in scratch (convattn_decode_noalloc): use fewer splits or convattn_decode";
         default: break;
     }
     if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
@@ -286,6 +314,35 @@ int convattn_decode_strided(const convattn_desc *desc, const void *q, const void
     if (pick_path(desc, p, CONVATTN_OP_DECODE) == 1)
         return (int)decode_stream(p, q, k, v, w, o_part, m_part, l_part, s);
     return (int)generic_decode(p, desc->in_dtype, q, k, v, w, o_part, m_part, l_part, s);
+}
+
+size_t convattn_decode_noalloc_bytes(const convattn_desc *desc) {
+    Problem p;
+    if (validate(desc, CONVATTN_OP_DECODE, &p)) return 0;
+    const size_t slots = (size_t)p.B * p.H * p.n_splits;
+    return align256(slots * p.d * sizeof(float)) + 2 * align256(slots * sizeof(float));
+}
+
+int convattn_decode_noalloc(const convattn_desc *desc, const void *q, const void *k, const void *v,
+                            const float *w, long long kv_batch_stride, long long kv_head_stride, void *o,
+                            float *m, float *l, void *stream) {
+    Problem p;
+    int rc = validate(desc, CONVATTN_OP_DECODE, &p);
+    if (rc) return rc;
+    REQUIRE_PTR(o); REQUIRE_PTR(m); REQUIRE_PTR(l);
+    if (convattn_decode_noalloc_bytes(desc) > kDecodeScratchBytes) return CONVATTN_ERR_SCRATCH;
+    hipError_t err = hipSuccess;
+    unsigned char *base = static_cast<unsigned char *>(decode_scratch(&err));
+    if (!base) return (int)err;
+    const size_t slots = (size_t)p.B * p.H * p.n_splits;
+    float *o_part = reinterpret_cast<float *>(base);
+    float *m_part = reinterpret_cast<float *>(base + align256(slots * p.d * sizeof(float)));
+    float *l_part = reinterpret_cast<float *>(base + align256(slots * p.d * sizeof(float)) + align256(slots * sizeof(float)));
+    // every (batch, head, split) slot is written by the first kernel before the second reads it:
+    // nothing of the previous call's contents is used
+    rc = convattn_decode_strided(desc, q, k, v, w, kv_batch_stride, kv_head_stride, o_part, m_part, l_part, stream);
+    if (rc) return rc;
+    return convattn_decode_combine(desc, o_part, m_part, l_part, o, m, l, stream);
 }
 
 int convattn_decode_combine(const convattn_desc *desc, const float *o_part, const float *m_part,

@@ -61,7 +61,8 @@ typedef enum convattn_status {
     CONVATTN_ERR_SCALE = -9,       /* scale is not finite */
     CONVATTN_ERR_CAUSAL_SHAPE = -10, /* causal training pass needs Nq == Nk */
     CONVATTN_ERR_LDS = -11,        /* the window needs more LDS than a CU has */
-    CONVATTN_ERR_TOO_LARGE = -12   /* a launch dimension would overflow */
+    CONVATTN_ERR_TOO_LARGE = -12,  /* a launch dimension would overflow */
+    CONVATTN_ERR_SCRATCH = -13     /* convattn_decode_noalloc: partials larger than the built-in scratch */
 } convattn_status;
 
 /* Flags for convattn_desc.flags */
@@ -218,6 +219,25 @@ int convattn_decode_strided(const convattn_desc *desc, const void *q, const void
  */
 int convattn_decode_combine(const convattn_desc *desc, const float *o_part, const float *m_part,
                             const float *l_part, void *o, float *m, float *l, void *stream);
+
+/*
+ * A whole decode step (convattn_decode_strided + convattn_decode_combine) that allocates nothing
+ * and needs no partial buffers from the caller: O [B,H,1,d] (out_dtype), M, L [B,H,1] fp32 from
+ * Q, K, V, W.  It has no counterpart in the reference; it is for callers that cannot allocate
+ * device memory around the call (code under HIP graph capture, serving loops with a fixed memory
+ * plan, harnesses that forbid hipMalloc).  The split partials live in a buffer built into the
+ * library, CONVATTN_DECODE_NOALLOC_MAX_BYTES per GPU for the life of the process:
+ * convattn_decode_noalloc_bytes(desc) is what a descriptor needs (B*H*n_splits*(d+2) floats, each
+ * part rounded up to 256 bytes; 0 on a bad descriptor); a step that needs more is rejected with
+ * CONVATTN_ERR_SCRATCH.  Every call on one GPU uses the same buffer: calls that overlap on one
+ * GPU (two streams, two threads) race, calls on one stream do not.  kv_batch_stride and
+ * kv_head_stride as in convattn_decode_strided (Nk*d*H and Nk*d for dense K and V).
+ */
+#define CONVATTN_DECODE_NOALLOC_MAX_BYTES (8u << 20)
+size_t convattn_decode_noalloc_bytes(const convattn_desc *desc);
+int convattn_decode_noalloc(const convattn_desc *desc, const void *q, const void *k, const void *v,
+                            const float *w, long long kv_batch_stride, long long kv_head_stride,
+                            void *o, float *m, float *l, void *stream);
 
 #ifdef __cplusplus
 }
