@@ -37,7 +37,9 @@ UNITS = [
     ("bwd_dkdv_mfma.hip", "bwd_dkdv_mfma_wide", ["-DCONVATTN_DKDV_UNIT=1"]),
     ("bwd_ws_mfma.hip", "bwd_ws_mfma", []),
     ("bwd_dq_gemm.hip", "bwd_dq_gemm", []),
-    ("bwd_chain_mfma.hip", "bwd_chain_mfma", []),
+    ("bwd_chain_mfma.hip", "bwd_chain_mfma_all", ["-DCONVATTN_CHAIN_UNIT=3"]),
+    ("bwd_chain_mfma.hip", "bwd_chain_mfma_kv", ["-DCONVATTN_CHAIN_UNIT=1"]),
+    ("bwd_chain_mfma.hip", "bwd_chain_mfma_qw", ["-DCONVATTN_CHAIN_UNIT=2"]),
     ("bwd_dq_rows.hip", "bwd_dq_rows", []),
     ("decode_stream.hip", "decode_stream", []),
 ]

@@ -86,7 +86,9 @@ def _weights(conv_kernel: torch.Tensor, H: int, pad_q: int, pad_k: int, device) 
             f"(got {pad_q}, {pad_k} for a {c_q}x{c_k} kernel)")
     if not conv_kernel.is_cuda:
         raise RuntimeError("conv_kernel must be a CUDA tensor")
-    return conv_kernel.detach().to(device=device, dtype=torch.float32).contiguous()
+    W = conv_kernel.detach().to(device=device, dtype=torch.float32).contiguous()
+    # a slice of a larger parameter (heads h..h') can start off a 16-byte boundary
+    return W if W.data_ptr() % 16 == 0 else W.clone()
 
 
 def _desc(Q, K, W, scale, causal, out_dtype, n_splits=1, exact=False) -> _lib.Desc:

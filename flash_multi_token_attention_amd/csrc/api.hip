@@ -155,49 +155,6 @@ int convattn_bwd_preprocess(const convattn_desc *desc, const void *o, const void
                                static_cast<hipStream_t>(stream));
 }
 
-size_t convattn_dw_partial_bytes(const convattn_desc *desc) {
-    Problem p;
-    if (validate(desc, CONVATTN_OP_BWD, &p)) return 0;
-    return (size_t)p.B * p.H * dw_tiles(desc, p) * p.c_q * p.c_k * sizeof(float);
-}
-
-int convattn_bwd_dq_dw(const convattn_desc *desc, const void *q, const void *k, const void *v,
-                       const void *d_o, const float *D, const float *lse, const float *w, void *dq,
-                       float *dw_partial, void *stream) {
-    Problem p;
-    int rc = validate(desc, CONVATTN_OP_BWD, &p);
-    if (rc) return rc;
-    REQUIRE_PTR(q); REQUIRE_PTR(k); REQUIRE_PTR(v); REQUIRE_PTR(d_o); REQUIRE_PTR(D);
-    REQUIRE_PTR(lse); REQUIRE_PTR(w); REQUIRE_PTR(dq); REQUIRE_PTR(dw_partial);
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    if (pick_path(desc, p, CONVATTN_OP_BWD) == 1)
-        return (int)mfma_bwd_dq_dw(p, desc->out_dtype, q, k, v, d_o, D, lse, w, dq, dw_partial, s);
-    return (int)generic_bwd_dq_dw(p, desc->in_dtype, desc->out_dtype, q, k, v, d_o, D, lse, w, dq,
-                                  dw_partial, s);
-}
-
-int convattn_dw_reduce(const convattn_desc *desc, const float *dw_partial, float *dw, void *stream) {
-    Problem p;
-    int rc = validate(desc, CONVATTN_OP_BWD, &p);
-    if (rc) return rc;
-    REQUIRE_PTR(dw_partial); REQUIRE_PTR(dw);
-    return (int)dw_reduce(p, dw_tiles(desc, p), dw_partial, dw, static_cast<hipStream_t>(stream));
-}
-
-int convattn_bwd_dkdv(const convattn_desc *desc, const void *q, const void *k, const void *v,
-                      const void *d_o, const float *D, const float *lse, const float *w, void *dk,
-                      void *dv, void *stream) {
-    Problem p;
-    int rc = validate(desc, CONVATTN_OP_BWD, &p);
-    if (rc) return rc;
-    REQUIRE_PTR(q); REQUIRE_PTR(k); REQUIRE_PTR(v); REQUIRE_PTR(d_o); REQUIRE_PTR(D);
-    REQUIRE_PTR(lse); REQUIRE_PTR(w); REQUIRE_PTR(dk); REQUIRE_PTR(dv);
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    if (pick_path(desc, p, CONVATTN_OP_BWD) == 1)
-        return (int)mfma_bwd_dkdv(p, desc->out_dtype, q, k, v, d_o, D, lse, w, dk, dv, s);
-    return (int)generic_bwd_dkdv(p, desc->in_dtype, desc->out_dtype, q, k, v, d_o, D, lse, w, dk, dv, s);
-}
-
 // Workspace of the one-pass backward on the MFMA path: dS blocks, dW partials and (windows of up
 // to 6 query taps) the dC scale of every (batch, head), each part 256-byte aligned.
 struct FusedWs {
@@ -212,6 +169,75 @@ static FusedWs fused_ws(const Problem &p) {
     w.scale_off = w.part_off + align256(fused_dw_bytes(p));
     w.total = w.scale_off + (w.chain ? align256(chain_scale_bytes(p)) : 0);
     return w;
+}
+
+// The dQ + dW pass on the chain path (windows of up to 6 query taps) is the key-stationary kernel
+// without its dK / dV half plus the dQ = dS K product: its "dW partial buffer" is the one-pass
+// backward's workspace (dS blocks, dW partials, dC scales).
+static bool dq_dw_uses_chain(const convattn_desc *desc, const Problem &p) {
+    return pick_path(desc, p, CONVATTN_OP_BWD) == 1 && chain_ok(p);
+}
+
+size_t convattn_dw_partial_bytes(const convattn_desc *desc) {
+    Problem p;
+    if (validate(desc, CONVATTN_OP_BWD, &p)) return 0;
+    if (dq_dw_uses_chain(desc, p)) return fused_ws(p).total;
+    return (size_t)p.B * p.H * dw_tiles(desc, p) * p.c_q * p.c_k * sizeof(float);
+}
+
+int convattn_bwd_dq_dw(const convattn_desc *desc, const void *q, const void *k, const void *v,
+                       const void *d_o, const float *D, const float *lse, const float *w, void *dq,
+                       float *dw_partial, void *stream) {
+    Problem p;
+    int rc = validate(desc, CONVATTN_OP_BWD, &p);
+    if (rc) return rc;
+    REQUIRE_PTR(q); REQUIRE_PTR(k); REQUIRE_PTR(v); REQUIRE_PTR(d_o); REQUIRE_PTR(D);
+    REQUIRE_PTR(lse); REQUIRE_PTR(w); REQUIRE_PTR(dq); REQUIRE_PTR(dw_partial);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dq_dw_uses_chain(desc, p)) {
+        unsigned char *ws = reinterpret_cast<unsigned char *>(dw_partial);
+        const FusedWs lay = fused_ws(p);
+        float *scale = reinterpret_cast<float *>(ws + lay.scale_off);
+        hipError_t e = mfma_dc_scale(p, d_o, v, scale, s);
+        if (e == hipSuccess)
+            e = mfma_bwd_chain(p, desc->out_dtype, 2, q, k, v, d_o, D, lse, w, scale, nullptr, nullptr, ws,
+                               reinterpret_cast<float *>(ws + lay.part_off), s);
+        if (e == hipSuccess) e = mfma_dq_from_rows(p, desc->out_dtype, k, ws, scale, dq, s);
+        return (int)e;
+    }
+    if (pick_path(desc, p, CONVATTN_OP_BWD) == 1)
+        return (int)mfma_bwd_dq_dw(p, desc->out_dtype, q, k, v, d_o, D, lse, w, dq, dw_partial, s);
+    return (int)generic_bwd_dq_dw(p, desc->in_dtype, desc->out_dtype, q, k, v, d_o, D, lse, w, dq,
+                                  dw_partial, s);
+}
+
+int convattn_dw_reduce(const convattn_desc *desc, const float *dw_partial, float *dw, void *stream) {
+    Problem p;
+    int rc = validate(desc, CONVATTN_OP_BWD, &p);
+    if (rc) return rc;
+    REQUIRE_PTR(dw_partial); REQUIRE_PTR(dw);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dq_dw_uses_chain(desc, p)) {
+        const unsigned char *ws = reinterpret_cast<const unsigned char *>(dw_partial);
+        return (int)dw_reduce(p, mfma_kv_tiles(p), reinterpret_cast<const float *>(ws + fused_ws(p).part_off), dw, s);
+    }
+    return (int)dw_reduce(p, dw_tiles(desc, p), dw_partial, dw, s);
+}
+
+int convattn_bwd_dkdv(const convattn_desc *desc, const void *q, const void *k, const void *v,
+                      const void *d_o, const float *D, const float *lse, const float *w, void *dk,
+                      void *dv, void *stream) {
+    Problem p;
+    int rc = validate(desc, CONVATTN_OP_BWD, &p);
+    if (rc) return rc;
+    REQUIRE_PTR(q); REQUIRE_PTR(k); REQUIRE_PTR(v); REQUIRE_PTR(d_o); REQUIRE_PTR(D);
+    REQUIRE_PTR(lse); REQUIRE_PTR(w); REQUIRE_PTR(dk); REQUIRE_PTR(dv);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dq_dw_uses_chain(desc, p))   // the key-stationary kernel without dS and dW; it scales dC by D
+        return (int)mfma_bwd_chain(p, desc->out_dtype, 1, q, k, v, d_o, D, lse, w, nullptr, dk, dv, nullptr, nullptr, s);
+    if (pick_path(desc, p, CONVATTN_OP_BWD) == 1)
+        return (int)mfma_bwd_dkdv(p, desc->out_dtype, q, k, v, d_o, D, lse, w, dk, dv, s);
+    return (int)generic_bwd_dkdv(p, desc->in_dtype, desc->out_dtype, q, k, v, d_o, D, lse, w, dk, dv, s);
 }
 
 size_t convattn_bwd_fused_workspace_bytes(const convattn_desc *desc) {
@@ -240,7 +266,7 @@ int convattn_bwd_fused_dkdv(const convattn_desc *desc, const void *q, const void
     float *scale = reinterpret_cast<float *>(ws + lay.scale_off);
     hipError_t e = mfma_dc_scale(p, d_o, v, scale, s);
     if (e != hipSuccess) return (int)e;
-    return (int)mfma_bwd_chain(p, desc->out_dtype, q, k, v, d_o, D, lse, w, scale, dk, dv, ws, part, s);
+    return (int)mfma_bwd_chain(p, desc->out_dtype, 3, q, k, v, d_o, D, lse, w, scale, dk, dv, ws, part, s);
 }
 
 int convattn_bwd_fused_dq(const convattn_desc *desc, const void *q, const void *k, const void *v,

@@ -161,6 +161,12 @@ __device__ __forceinline__ f16x8 band_frag(int t, const float *__restrict__ w_he
 #define CHAIN_SCHED_BARRIER
 #endif
 
+#if !defined(CONVATTN_CHAIN_UNIT) || CONVATTN_CHAIN_UNIT == 3
+#define CONVATTN_CHAIN_UNIT_IS_ALL 1
+#else
+#define CONVATTN_CHAIN_UNIT_IS_ALL 0
+#endif
+
 #ifdef CHAIN_TS
 __device__ long long g_chain_ts[8][64][12];
 #define TS(i)                                                                                     \
@@ -195,7 +201,9 @@ struct ChainArgs {
 // One role of the workgroup (ROLE 0 = producer waves, 1 = consumer waves) as a function of its
 // own: the two roles have disjoint register sets of 256 each, and compiled into one function body
 // the register allocator spills where either role alone does not.
-template <int D, int CQT, typename TO, int ROLE>
+// WANT: bit 0 = dK and dV, bit 1 = dS (for dQ) and dW; the passes behind the separate dK / dV and dQ + dW
+// operations leave the other half out.
+template <int D, int CQT, typename TO, int ROLE, int WANT>
 __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainArgs *args_in) {
     // the pointer arrives in vector registers; it is the same in every lane, and as a scalar the
     // arguments are fetched with scalar loads into scalar registers
@@ -222,6 +230,7 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int g = lane >> 4, n = lane & 15;
     constexpr bool producer = ROLE == 0;
+    constexpr bool WANT_KV = (WANT & 1) != 0, WANT_QW = (WANT & 2) != 0;
     const int pr = wave & (NP - 1);
 
     auto q_slot = [&](int t) { return smem + Lds::q_off + (t & 3) * Lds::tile_bytes; };
@@ -243,8 +252,27 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
     const bf16_t *dOb = dO + bh * p.Nq * D;
     const float *lse_b = LSE + bh * p.Nq;
     const float *dl_b = Dl + bh * p.Nq;
-    const float dcs = dc_scale ? dc_scale[2 * bh] : 1.f;       // power of two
-    const float dcs_log2 = dc_scale ? dc_scale[2 * bh + 1] : 0.f;
+    // dC scale (a power of two): given by the caller, or, without one, taken from D = rowsum(dO O) of
+    // this (batch, head): D is linear in dO and of the magnitude of dP, so s |D|max ~ 2^8 keeps dC in
+    // the normal range of fp16 whatever the magnitude of dO is
+    float dcs, dcs_log2;
+    if (dc_scale) {
+        dcs = dc_scale[2 * bh];
+        dcs_log2 = dc_scale[2 * bh + 1];
+    } else {
+        float mx = 0.f;
+        for (int i = tid; i < p.Nq; i += NT) mx = fmaxf(mx, fabsf(dl_b[i]));
+        mx = wave_max(mx);
+        float *red = reinterpret_cast<float *>(smem + Lds::stat_off);
+        if (lane == 0) red[wave] = mx;
+        __syncthreads();
+        mx = 0.f;
+#pragma unroll
+        for (int w2 = 0; w2 < 2 * NP; ++w2) mx = fmaxf(mx, red[w2]);
+        __syncthreads();
+        dcs_log2 = (mx > 0.f && mx < 3e38f) ? fminf(fmaxf(floorf(8.f - __log2f(mx)), -100.f), 100.f) : 0.f;
+        dcs = exp2f(dcs_log2);
+    }
 
     // Causal: rows before the first key this workgroup touches (k0 - 8) see none of its keys.
     const int r_begin = causal ? (max(0, k0 - 8) / BR) * BR : 0;
@@ -369,7 +397,7 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
                     const u32x2 two = __builtin_bit_cast(u32x2, hv);
                     pd[kb][f][0] = two[0];
                     pd[kb][f][1] = two[1];
-                    if (kb < 3) {
+                    if (WANT_QW && kb < 3) {
                         const int rr = rbase + 2 * n + f;
                         *reinterpret_cast<u32x2 *>(s_ring + (rr >= S_RING ? rr - S_RING : rr) * SST + (kb * 16 + 4 * g) * 2) =
                             (u32x2){pd[kb][f][0], pd[kb][f][1]};
@@ -498,7 +526,7 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
                             }
                             *reinterpret_cast<u32x2 *>(Cs + (2 * n + ob) * CST + (cb * 16 + 4 * g) * 2) =
                                 (u32x2){pack_f16_rtz(dc[0], dc[1]), pack_f16_rtz(dc[2], dc[3])};
-                            if constexpr (cb < 2) {
+                            if constexpr (WANT_KV && cb < 2) {
                                 bf16x4 pv;
 #pragma unroll
                                 for (int r = 0; r < 4; ++r) pv[r] = (bf16_t)prob[r];
@@ -570,7 +598,7 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
             // Order of the iteration: dV (operands of the staged tiles only, so the first MFMAs
             // start while the dC loads are in flight), dS, dW (independent of dS: its MFMAs cover
             // the round trip of dS through LDS), dK.
-            if (u_ok && !(CHAIN_ABLATE & 4)) {
+            if (WANT_KV && u_ok && !(CHAIN_ABLATE & 4)) {
                 const unsigned char *Ps = smem + opaque((unsigned int)(p_stage(u) - smem) + tr_lane_off(PST, g, n));
                 const unsigned char *Gs = smem + opaque((unsigned int)(g_slot(u) - smem) + tr_lane_off(RST, g, n));
                 __builtin_amdgcn_s_setprio(1);
@@ -642,8 +670,8 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
                         bf16x4 sv;
 #pragma unroll
                         for (int r = 0; r < 4; ++r) sv[r] = (bf16_t)ds[sb][ob][r];
-                        *reinterpret_cast<bf16x4 *>(ds_blk + (2 * n + ob) * WK + sb * 16 + 4 * g) = sv;
-                        *reinterpret_cast<bf16x4 *>(ds_tile + (2 * n + ob) * PST + (sb * 16 + 4 * g) * 2) = sv;
+                        if constexpr (WANT_QW) *reinterpret_cast<bf16x4 *>(ds_blk + (2 * n + ob) * WK + sb * 16 + 4 * g) = sv;
+                        if constexpr (WANT_KV) *reinterpret_cast<bf16x4 *>(ds_tile + (2 * n + ob) * PST + (sb * 16 + 4 * g) * 2) = sv;
                     }
             }
 #pragma unroll
@@ -656,7 +684,7 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
             // pair 2 pg + jb / 2, keys k0 + 64 pg - 8 + 16 jb ..), tap slots t_lo .. t_lo + TH - 1:
             // G_t[j][j'] += sum_rows dC[row][j] S[row + t - (CQT-1)][j'] with j' in the score block
             // 8 keys before the dC block (x = 0) and the one 8 keys after it (x = 1) ----
-            if (u_in && !(CHAIN_ABLATE & 1)) {
+            if (WANT_QW && u_in && !(CHAIN_ABLATE & 1)) {
                 // Ring rows of this lane's two transpose reads at the wave's first tap slot: tile row 0
                 // at tap slot 0 is ring row wbase; the TH tap slots are consecutive rows (mod S_RING).
                 const int wbase = ((u + 1) * BR - (CQT - 1) + S_RING) % S_RING;
@@ -716,7 +744,7 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
             }
             CHAIN_SCHED_BARRIER;
             TS(5);
-            if (v_ok && !(CHAIN_ABLATE & 8)) {
+            if (WANT_KV && v_ok && !(CHAIN_ABLATE & 8)) {
                 const unsigned char *Qs = smem + opaque((unsigned int)(q_slot(v) - smem) + tr_lane_off(RST, g, n));
                 const unsigned char *Dsl = smem + opaque((unsigned int)(ds_tile - smem) + tr_lane_off(PST, g, n));
                 asm volatile("" ::: "memory");
@@ -750,7 +778,7 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
                 const int col = db * 16 + 4 * g;
-                if (key_k < p.Nk) {
+                if (WANT_KV && key_k < p.Nk) {
                     TO *dst = dK + (bh * p.Nk + key_k) * D + col;
                     if constexpr (sizeof(TO) == 2) {
                         bf16x4 ov;
@@ -761,7 +789,7 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
                         *reinterpret_cast<f32x4 *>(dst) = acc_k[m][db] * inv;
                     }
                 }
-                if (key_v >= 0 && key_v < p.Nk) {
+                if (WANT_KV && key_v >= 0 && key_v < p.Nk) {
                     TO *dst = dV + (bh * p.Nk + key_v) * D + col;
                     if constexpr (sizeof(TO) == 2) {
                         bf16x4 ov;
@@ -785,7 +813,7 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
             for (int x = 0; x < 2; ++x)
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
-                    if (t_lo + tt < CQT)
+                    if (WANT_QW && t_lo + tt < CQT)
                         red[(((pg * CQT + t_lo + tt) * 2 + x) * 16 + 4 * g + r) * 16 + n] = acc_w[tt][x][r];
     }  // consumer
 
@@ -795,7 +823,7 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
     static_assert(2 * CQT * 2 * 1024 <= NP * ChainLds<D, CQT>::pair_bytes, "room for the dW accumulators");
     __syncthreads();
     const int ntap = cq * ck;
-    if (tid < ntap) {
+    if (WANT_QW && tid < ntap) {
         const int a = tid / ck, bb = tid - a * ck, t = a + CQT - cq;
         const float *red = reinterpret_cast<const float *>(smem + Lds::pair_off);
         float sum = 0.f;
@@ -809,7 +837,7 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
     }
 }
 
-template <int D, int CQT, typename TO>
+template <int D, int CQT, typename TO, int WANT>
 __global__ __launch_bounds__(NT) void bwd_chain_kernel(ChainArgs args) {
     // `args` is the whole argument segment; the roles read it from there
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -818,10 +846,11 @@ __global__ __launch_bounds__(NT) void bwd_chain_kernel(ChainArgs args) {
 #else
     const ChainArgs *ap = &args;
 #endif
-    if (__builtin_amdgcn_readfirstlane(threadIdx.x >> 6) < NP) chain_role<D, CQT, TO, 0>(ap);
-    else chain_role<D, CQT, TO, 1>(ap);
+    if (__builtin_amdgcn_readfirstlane(threadIdx.x >> 6) < NP) chain_role<D, CQT, TO, 0, WANT>(ap);
+    else chain_role<D, CQT, TO, 1, WANT>(ap);
 }
 
+#if CONVATTN_CHAIN_UNIT_IS_ALL
 // amax|dO| and amax|V| of one (batch, head) -> {s, log2 s}, s the power of two that brings
 // sqrt(d) * amax|dO| * amax|V| (a few times a typical |dP|) to about 2^12.  Two steps: kScaleChunks
 // workgroups per (batch, head) leave their maxima in `part`, one thread per (batch, head) finishes.
@@ -869,11 +898,13 @@ __global__ void dc_scale_finish_kernel(int n_bh, int d, const float *__restrict_
     out[2 * bh + 1] = e;
 }
 
-template <int D, int CQT, typename TO>
+#endif
+
+template <int D, int CQT, typename TO, int WANT>
 hipError_t launch_chain(const Problem &p, const void *q, const void *k, const void *v, const void *d_o,
                         const float *Dl, const float *lse, const float *w, const float *dc_scale, void *dk,
                         void *dv, void *ds_ws, float *dw_part, hipStream_t s) {
-    auto kern = bwd_chain_kernel<D, CQT, TO>;
+    auto kern = bwd_chain_kernel<D, CQT, TO, WANT>;
     constexpr int lds = ChainLds<D, CQT>::total;
     static_assert(lds <= 160 * 1024, "LDS budget");
     static bool attr_set = false;  // per kernel instantiation; the attribute is sticky
@@ -890,12 +921,24 @@ hipError_t launch_chain(const Problem &p, const void *q, const void *k, const vo
     return hipGetLastError();
 }
 
-template <int D, typename TO>
+template <int D, typename TO, int WANT>
 hipError_t pick_cq(const Problem &p, const void *q, const void *k, const void *v, const void *d_o,
                    const float *Dl, const float *lse, const float *w, const float *dc_scale, void *dk, void *dv,
                    void *ds_ws, float *dw_part, hipStream_t s) {
-    if (p.c_q <= 3) return launch_chain<D, 3, TO>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
-    return launch_chain<D, 6, TO>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
+    if (p.c_q <= 3) return launch_chain<D, 3, TO, WANT>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
+    return launch_chain<D, 6, TO, WANT>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
+}
+
+template <int WANT>
+hipError_t pick_shape(const Problem &p, int out_dt, const void *q, const void *k, const void *v, const void *d_o,
+                      const float *Dl, const float *lse, const float *w, const float *dc_scale, void *dk, void *dv,
+                      void *ds_ws, float *dw_part, hipStream_t s) {
+    if (p.d == 128) {
+        if (out_dt == CONVATTN_BF16) return pick_cq<128, bf16_t, WANT>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
+        return pick_cq<128, float, WANT>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
+    }
+    if (out_dt == CONVATTN_BF16) return pick_cq<64, bf16_t, WANT>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
+    return pick_cq<64, float, WANT>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
 }
 
 }  // namespace
@@ -906,6 +949,7 @@ extern "C" int convattn_debug_chain_ts(long long *host) {
 }
 #endif
 
+#if CONVATTN_CHAIN_UNIT_IS_ALL
 hipError_t mfma_dc_scale(const Problem &p, const void *d_o, const void *v, float *dc_scale, hipStream_t s) {
     // dc_scale holds {s, log2 s} per (batch, head), then the partial maxima
     float *part = dc_scale + (size_t)p.B * p.H * 2;
@@ -916,16 +960,24 @@ hipError_t mfma_dc_scale(const Problem &p, const void *d_o, const void *v, float
     dc_scale_finish_kernel<<<dim3((p.B * p.H + 255) / 256), 256, 0, s>>>(p.B * p.H, p.d, part, dc_scale);
     return hipGetLastError();
 }
+#endif
 
-hipError_t mfma_bwd_chain(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
-                          const void *d_o, const float *Dl, const float *lse, const float *w,
-                          const float *dc_scale, void *dk, void *dv, void *ds_ws, float *dw_part, hipStream_t s) {
-    if (p.d == 128) {
-        if (out_dt == CONVATTN_BF16) return pick_cq<128, bf16_t>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
-        return pick_cq<128, float>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
-    }
-    if (out_dt == CONVATTN_BF16) return pick_cq<64, bf16_t>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
-    return pick_cq<64, float>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
+// This file is compiled once per value of CONVATTN_CHAIN_UNIT (1 = dK and dV only, 2 = dS and dW
+// only, 3 = everything), so that the three sets of instances build in parallel.
+#ifndef CONVATTN_CHAIN_UNIT
+#define CONVATTN_CHAIN_UNIT 3
+#endif
+#if CONVATTN_CHAIN_UNIT == 1
+#define CHAIN_ENTRY mfma_bwd_chain_kv
+#elif CONVATTN_CHAIN_UNIT == 2
+#define CHAIN_ENTRY mfma_bwd_chain_qw
+#else
+#define CHAIN_ENTRY mfma_bwd_chain_all
+#endif
+hipError_t CHAIN_ENTRY(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
+                       const void *d_o, const float *Dl, const float *lse, const float *w,
+                       const float *dc_scale, void *dk, void *dv, void *ds_ws, float *dw_part, hipStream_t s) {
+    return pick_shape<CONVATTN_CHAIN_UNIT>(p, out_dt, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
 }
 
 }  // namespace convattn

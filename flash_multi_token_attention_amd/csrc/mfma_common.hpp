@@ -230,9 +230,24 @@ inline size_t chain_ds_bytes(const Problem &p) {
 // {s, log2 s} per (batch, head) followed by 32 x 2 partial maxima per (batch, head)
 inline size_t chain_scale_bytes(const Problem &p) { return (size_t)p.B * p.H * (2 + 64) * sizeof(float); }
 hipError_t mfma_dc_scale(const Problem &p, const void *d_o, const void *v, float *dc_scale, hipStream_t s);
-hipError_t mfma_bwd_chain(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
-                          const void *d_o, const float *Dl, const float *lse, const float *w,
-                          const float *dc_scale, void *dk, void *dv, void *ds_ws, float *dw_part, hipStream_t s);
+// want: bit 0 = dK and dV, bit 1 = dS blocks (for dQ) and the dW partial; dc_scale may be null when
+// bit 1 is clear (the kernel then takes the scale from D).
+#define CHAIN_DECL(name)                                                                                   \
+    hipError_t name(const Problem &p, int out_dt, const void *q, const void *k, const void *v, const void *d_o, \
+                    const float *Dl, const float *lse, const float *w, const float *dc_scale, void *dk, void *dv, \
+                    void *ds_ws, float *dw_part, hipStream_t s)
+CHAIN_DECL(mfma_bwd_chain_kv);
+CHAIN_DECL(mfma_bwd_chain_qw);
+CHAIN_DECL(mfma_bwd_chain_all);
+#undef CHAIN_DECL
+inline hipError_t mfma_bwd_chain(const Problem &p, int out_dt, int want, const void *q, const void *k, const void *v,
+                                 const void *d_o, const float *Dl, const float *lse, const float *w,
+                                 const float *dc_scale, void *dk, void *dv, void *ds_ws, float *dw_part,
+                                 hipStream_t s) {
+    if (want == 1) return mfma_bwd_chain_kv(p, out_dt, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
+    if (want == 2) return mfma_bwd_chain_qw(p, out_dt, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
+    return mfma_bwd_chain_all(p, out_dt, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
+}
 hipError_t mfma_dq_from_rows(const Problem &p, int out_dt, const void *k, const void *ds_ws,
                              const float *dc_scale, void *dq, hipStream_t s);
 
