@@ -233,6 +233,15 @@ def main():
     torch.cuda.synchronize()
     ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
     useful = fl["fwd"] + (fl["bwd"] if wl.backward else 0.0)
+    # spread of single steps (HIP events around each of a second batch of steps; not the headline
+    # number, which is the wall clock of the back-to-back run above)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    for a, b in evs:
+        a.record()
+        step()
+        b.record()
+    torch.cuda.synchronize()
+    per_step = sorted(a.elapsed_time(b) for a, b in evs)
 
     # per-kernel launch durations (HIP events, same stream)
     allk = {**ts.kernels, **ts.two_pass}
@@ -255,7 +264,9 @@ def main():
         "dtype": wl.dtype, "data": "synthetic",
         "config": {"workload": f"{wl.name}: B={wl.B} H={wl.H} N={wl.Nq} d={wl.d} window={wl.c_q}x{wl.c_k} "
                                f"causal={wl.causal} fwd+bwd", "kernel_path": ts.path(),
-                   "useful_flop_per_step": useful, "conv_flop_per_pass": fl["conv_per_pass"]},
+                   "useful_flop_per_step": useful, "conv_flop_per_pass": fl["conv_per_pass"],
+                   **synthetic.executed_mfma_flops(wl, two_pass=args.two_pass)},
+        "ms_per_step_min": per_step[0], "ms_per_step_median": per_step[len(per_step) // 2],
         "kernel_ms": k_ms,
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": measured_traffic(dom, wl.name)},

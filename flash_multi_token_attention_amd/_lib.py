@@ -12,6 +12,7 @@ LIB_PATH = os.environ.get("CONVATTN_LIB") or os.path.join(_PKG, "libconvattn_hip
 BF16, F32 = 0, 1
 OP_FWD, OP_BWD, OP_DECODE = 0, 1, 2
 FLAG_EXACT = 1
+FLAG_LOW_MEMORY = 2
 ERR_QROWS = -8
 
 

@@ -15,6 +15,7 @@ Differences from the reference ops, all deliberate:
 from __future__ import annotations
 
 import ctypes as C
+import os
 from typing import Optional, Tuple
 
 import torch
@@ -91,12 +92,13 @@ def _weights(conv_kernel: torch.Tensor, H: int, pad_q: int, pad_k: int, device) 
     return W if W.data_ptr() % 16 == 0 else W.clone()
 
 
-def _desc(Q, K, W, scale, causal, out_dtype, n_splits=1, exact=False) -> _lib.Desc:
+def _desc(Q, K, W, scale, causal, out_dtype, n_splits=1, exact=False, low_memory=False) -> _lib.Desc:
     if out_dtype not in _DT:
         raise RuntimeError("out_dtype must be bfloat16 or float32")
     B, H, Nq, d = Q.shape
     return _lib.Desc(B, H, Nq, K.shape[2], d, W.shape[1], W.shape[2], float(scale), int(bool(causal)),
-                     _DT[Q.dtype], _DT[out_dtype], int(n_splits), _lib.FLAG_EXACT if exact else 0)
+                     _DT[Q.dtype], _DT[out_dtype], int(n_splits),
+                     (_lib.FLAG_EXACT if exact else 0) | (_lib.FLAG_LOW_MEMORY if low_memory else 0))
 
 
 def _stat(t: torch.Tensor, name: str, like: torch.Tensor) -> torch.Tensor:
@@ -152,7 +154,7 @@ def bwd_preprocess(O, dO, M, L) -> Tuple[torch.Tensor, torch.Tensor]:
     return D, LSE
 
 
-def _bwd_common(Q, K, V, dO, D, L, conv_kernel, scale, pad_q, pad_k, causal, out_dtype, exact):
+def _bwd_common(Q, K, V, dO, D, L, conv_kernel, scale, pad_q, pad_k, causal, out_dtype, exact, low_memory=False):
     _check_qkv(Q, K, V)
     _check_input(dO, "dO")
     if dO.shape != Q.shape or dO.dtype != Q.dtype:
@@ -160,21 +162,23 @@ def _bwd_common(Q, K, V, dO, D, L, conv_kernel, scale, pad_q, pad_k, causal, out
     W = _weights(conv_kernel, Q.shape[1], pad_q, pad_k, Q.device)
     D = _stat(D, "D", Q)
     L = _stat(L, "L", Q)
-    return W, D, L, _desc(Q, K, W, scale, causal, out_dtype, exact=exact)
+    return W, D, L, _desc(Q, K, W, scale, causal, out_dtype, exact=exact, low_memory=low_memory)
 
 
 def dq_backward(Q, K, V, dO, D, L, conv_kernel, scale, pad_q, pad_k, causal,
-                out_dtype=torch.float32, exact=False) -> Tuple[torch.Tensor, torch.Tensor]:
+                out_dtype=torch.float32, exact=False, low_memory=False) -> Tuple[torch.Tensor, torch.Tensor]:
     """-> (dQ [B,H,N,d], dconv_kernel [H,c_q,c_k] fp32).  ``L`` is the log-sum-exp
-    M + log L and ``D`` is rowsum(dO * O), as the reference passes them."""
+    M + log L and ``D`` is rowsum(dO * O), as the reference passes them.  On the MFMA path the
+    scratch of this op holds the bf16 dS matrix (B*H*Nq*Nk*2 bytes); ``low_memory`` runs the
+    slower query-stationary kernel whose scratch is O(N)."""
     W, D, L, desc = _bwd_common(Q, K, V, dO, D, L, conv_kernel, scale, pad_q, pad_k, causal,
-                                out_dtype, exact)
+                                out_dtype, exact, low_memory)
     lib = _lib.load()
     dQ = torch.empty(Q.shape, dtype=out_dtype, device=Q.device)
     nbytes = lib.convattn_dw_partial_bytes(C.byref(desc))
     if nbytes == 0:
         _lib.check(lib.convattn_validate(C.byref(desc), _lib.OP_BWD), "conv_attn.dq_backward")
-    part = torch.empty(nbytes // 4, dtype=torch.float32, device=Q.device)
+    part = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=Q.device)
     dW = torch.empty(W.shape, dtype=torch.float32, device=Q.device)
     st = _stream(Q)
     rc = lib.convattn_bwd_dq_dw(C.byref(desc), _ptr(Q), _ptr(K), _ptr(V), _ptr(dO), _ptr(D), _ptr(L),
@@ -198,18 +202,36 @@ def dkdv_backward(Q, K, V, dO, D, L, conv_kernel, scale, pad_q, pad_k, causal,
     return dK, dV
 
 
+def max_workspace_bytes() -> int:
+    """Largest workspace ``backward`` allocates before it falls back to the two separate passes
+    with O(N) scratch (``CONVATTN_MAX_WORKSPACE_BYTES``, default 64 GiB)."""
+    return int(os.environ.get("CONVATTN_MAX_WORKSPACE_BYTES", 64 << 30))
+
+
 def backward(Q, K, V, dO, D, L, conv_kernel, scale, pad_q, pad_k, causal,
              out_dtype=torch.float32, exact=False):
     """-> (dQ, dK, dV, dconv_kernel) from one pass over the score tiles: the results of
     ``dq_backward`` + ``dkdv_backward`` (same arguments) without computing the scores, the
-    convolution and dC twice.  Needs a workspace the size of the bf16 dS matrix."""
+    convolution and dC twice.  Needs a workspace the size of the bf16 dS matrix
+    (B*H*Nq*Nk*2 bytes: 2.2 GB at B4 H16 N4096, 17 GB at B1 H32 N16384); when that exceeds
+    ``max_workspace_bytes()`` or cannot be allocated, the two passes with O(N) scratch run instead."""
     W, D, L, desc = _bwd_common(Q, K, V, dO, D, L, conv_kernel, scale, pad_q, pad_k, causal,
                                 out_dtype, exact)
     lib = _lib.load()
     nbytes = lib.convattn_bwd_fused_workspace_bytes(C.byref(desc))
     if nbytes == 0:
         _lib.check(lib.convattn_validate(C.byref(desc), _lib.OP_BWD), "conv_attn.backward")
-    ws = torch.empty(nbytes, dtype=torch.uint8, device=Q.device)
+    ws = None
+    if nbytes <= max_workspace_bytes():
+        try:
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=Q.device)
+        except torch.OutOfMemoryError:
+            ws = None
+    if ws is None:
+        dQ, dW = dq_backward(Q, K, V, dO, D, L, conv_kernel, scale, pad_q, pad_k, causal, out_dtype, exact,
+                             low_memory=True)
+        dK, dV = dkdv_backward(Q, K, V, dO, D, L, conv_kernel, scale, pad_q, pad_k, causal, out_dtype, exact)
+        return dQ, dK, dV, dW
     dQ = torch.empty(Q.shape, dtype=out_dtype, device=Q.device)
     dK = torch.empty(K.shape, dtype=out_dtype, device=Q.device)
     dV = torch.empty(V.shape, dtype=out_dtype, device=Q.device)

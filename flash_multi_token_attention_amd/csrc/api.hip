@@ -175,7 +175,7 @@ static FusedWs fused_ws(const Problem &p) {
 // without its dK / dV half plus the dQ = dS K product: its "dW partial buffer" is the one-pass
 // backward's workspace (dS blocks, dW partials, dC scales).
 static bool dq_dw_uses_chain(const convattn_desc *desc, const Problem &p) {
-    return pick_path(desc, p, CONVATTN_OP_BWD) == 1 && chain_ok(p);
+    return pick_path(desc, p, CONVATTN_OP_BWD) == 1 && chain_ok(p) && !(desc->flags & CONVATTN_FLAG_LOW_MEMORY);
 }
 
 size_t convattn_dw_partial_bytes(const convattn_desc *desc) {
@@ -233,7 +233,7 @@ int convattn_bwd_dkdv(const convattn_desc *desc, const void *q, const void *k, c
     REQUIRE_PTR(q); REQUIRE_PTR(k); REQUIRE_PTR(v); REQUIRE_PTR(d_o); REQUIRE_PTR(D);
     REQUIRE_PTR(lse); REQUIRE_PTR(w); REQUIRE_PTR(dk); REQUIRE_PTR(dv);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (dq_dw_uses_chain(desc, p))   // the key-stationary kernel without dS and dW; it scales dC by D
+    if (pick_path(desc, p, CONVATTN_OP_BWD) == 1 && chain_ok(p))   // the key-stationary kernel without dS and dW; it scales dC by D
         return (int)mfma_bwd_chain(p, desc->out_dtype, 1, q, k, v, d_o, D, lse, w, nullptr, dk, dv, nullptr, nullptr, s);
     if (pick_path(desc, p, CONVATTN_OP_BWD) == 1)
         return (int)mfma_bwd_dkdv(p, desc->out_dtype, q, k, v, d_o, D, lse, w, dk, dv, s);

@@ -168,13 +168,18 @@ inline bool mfma_shape_ok(const Problem &p, int in_dt, unsigned flags) {
 }
 // The forward addresses K and V of one (batch, head) through buffer descriptors, which count
 // bytes in 32 bits.
+// Row / key tiles sit on the z dimension of the grids (at most 65535): the smallest forward tile has
+// 88 rows, the backward kernels' tiles 128 rows or keys.
+constexpr int kMaxGridZ = 65535;
 inline bool mfma_fwd_shape_ok(const Problem &p, int in_dt, unsigned flags) {
-    return mfma_shape_ok(p, in_dt, flags) && (size_t)p.Nk * p.d * 2 < (1ull << 31);
+    return mfma_shape_ok(p, in_dt, flags) && (size_t)p.Nk * p.d * 2 < (1ull << 31) &&
+           ((long long)p.Nq + 87) / 88 <= kMaxGridZ;
 }
 // The backward kernels put the key taps on one 16-wide MFMA dimension.
 inline bool mfma_bwd_shape_ok(const Problem &p, int in_dt, unsigned flags) {
     // (the one-pass kernel addresses Q and dO of one (batch, head) with 32-bit byte offsets)
-    return mfma_shape_ok(p, in_dt, flags) && p.c_k <= 15 && (size_t)p.Nq * p.d * 2 < (1ull << 31);
+    return mfma_shape_ok(p, in_dt, flags) && p.c_k <= 15 && (size_t)p.Nq * p.d * 2 < (1ull << 31) &&
+           ((long long)p.Nq + 16 + 127) / 128 <= kMaxGridZ && ((long long)p.Nk + 8 + 127) / 128 <= kMaxGridZ;
 }
 
 // ---- bf16 MFMA kernels ----

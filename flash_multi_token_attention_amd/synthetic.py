@@ -92,6 +92,57 @@ def useful_flops(wl: Workload) -> Dict[str, float]:
     }
 
 
+def executed_mfma_flops(wl: Workload, two_pass: bool = False) -> Dict[str, object]:
+    """FLOPs the bf16 MFMA kernels execute on the matrix cores for one step of a causal workload
+    with d in {64, 128} and at most 6 query taps, counted from their tiles (every MFMA is
+    16 x 16 x 32 = 16384 FLOP), next to the useful ones; the difference is halo, convolution, dW and
+    recompute.  Per kernel:
+
+    forward: a wave owns 33 - T output rows (T = 3 or 6 tap slots) of a 32-row score tile and walks
+      the keys in 32-key steps up to its last row + 16: per step S^T 2 (row fragments) x 2 (key
+      blocks) x d/32, convolution 4 T, P V 2 x d/16 MFMAs.
+    key-stationary backward: a wave pair owns 32 keys and walks 32-row tiles from the first row that
+      sees its keys: per tile S^T 8 d/32 (64 keys for 32 owned), convolution 6 T (48 keys), dP 6 d/32,
+      transposed convolution 4 T, dV and dK 2 d/16 each, dW 4 T MFMAs.
+    dQ = dS K: 2 x d/16 per 32 rows x 32 keys below the diagonal (nothing wasted but the diagonal
+      blocks' upper halves).
+    """
+    assert wl.causal and wl.Nq == wl.Nk
+    N, d, T, bh = wl.Nq, wl.d, (3 if wl.c_q <= 3 else 6), wl.B * wl.H
+    mf = 16.0 * 16 * 32 * 2
+    rows = 33 - T
+    fwd = 0
+    for w0 in range(0, N, rows):                       # one wave per `rows` output rows
+        wg_end = min(N, (w0 // (4 * rows) + 1) * 4 * rows)          # its workgroup's last row + 1
+        steps = min((w0 + rows + 15) // 32 + 1, (wg_end + 16 + 31) // 32)
+        fwd += steps * (4 * d // 32 + 4 * T + 2 * d // 16)
+    per_tile = 8 * d // 32 + 6 * T + 6 * d // 32 + 4 * T + 4 * d // 16 + 4 * T
+    per_tile_kv = per_tile - 4 * T                     # dK / dV pass: no dW
+    per_tile_qw = per_tile - 4 * d // 16               # dQ + dW pass: no dV, dK
+    tiles = s_only = 0
+    for c0 in range(0, (N + 8 + 127) // 128 * 128, 32):   # one wave pair per 32 keys
+        k0 = c0 // 128 * 128
+        r_begin = max(0, k0 - 8) // 32 * 32
+        n_t = max(0, (N - r_begin + 31) // 32)
+        skipped = sum(1 for t in range(n_t) if r_begin + 32 * t + 31 < c0 - 8)   # scores only
+        tiles += n_t - skipped
+        s_only += skipped + 1                           # + the 32 rows above the first tile
+    dq = sum((min(N, (r // 128 + 1) * 128) + 63) // 64 * 2 for r in range(0, N, 32)) * 2 * d // 16
+    out = {"fwd": fwd * mf * bh}
+    if wl.backward:
+        if two_pass:
+            out["bwd_dkdv"] = (tiles * per_tile_kv + s_only * 8 * d // 32) * mf * bh
+            out["bwd_dq_dw"] = (tiles * per_tile_qw + s_only * 8 * d // 32 + dq) * mf * bh
+        else:
+            out["bwd_fused_dkdv"] = (tiles * per_tile + s_only * 8 * d // 32) * mf * bh
+            out["bwd_fused_dq"] = dq * mf * bh
+    total = sum(out.values())
+    fl = useful_flops(wl)
+    useful = fl["fwd"] + (fl["bwd"] if wl.backward else 0.0)
+    return {"executed_mfma_flop_per_step": total, "executed_mfma_flop_per_kernel": out,
+            "halo_recompute_flop_per_step": total - useful}
+
+
 def decode_bytes(wl: Workload, elem: int = 2) -> int:
     """Algorithmic HBM bytes of one decode step: K + V once, Q, O and W."""
     kv = 2 * wl.B * wl.H * wl.Nk * wl.d * elem

@@ -68,6 +68,9 @@ typedef enum convattn_status {
 /* Flags for convattn_desc.flags */
 #define CONVATTN_FLAG_EXACT 1u /* force the fp32-arithmetic kernels (no MFMA, no
                                   fp16 score tile); what "fp32 mode" runs */
+#define CONVATTN_FLAG_LOW_MEMORY 2u /* convattn_bwd_dq_dw: keep the partial buffer O(N) (the
+                                  query-stationary kernel) instead of the faster pass whose
+                                  buffer holds the bf16 dS matrix, O(N^2) */
 
 /*
  * Problem descriptor (plain data, passed by pointer, read during the call only).

@@ -169,4 +169,10 @@ def test_kernel_path_selection(lib):
     # the forward addresses K / V of one (batch, head) with 32-bit byte offsets
     big = 1 << 24
     assert lib.convattn_kernel_path(C.byref(desc(Nq=big, Nk=big, d=64)), _lib.OP_FWD) == 0
-    assert lib.convattn_kernel_path(C.byref(desc(Nq=big - 64, Nk=big - 64, d=64)), _lib.OP_FWD) == 1
+    assert lib.convattn_kernel_path(C.byref(desc(Nq=big - 64, Nk=big - 64, d=64)), _lib.OP_FWD) == 0
+    # ... and puts its row tiles (88 rows at the least) on the grid's z dimension: at most 65535 of them
+    assert lib.convattn_kernel_path(C.byref(desc(Nq=65535 * 88, Nk=65535 * 88, d=64)), _lib.OP_FWD) == 1
+    assert lib.convattn_kernel_path(C.byref(desc(Nq=65535 * 88 + 1, Nk=65535 * 88 + 1, d=64)), _lib.OP_FWD) == 0
+    # the backward kernels' tiles are 128 rows or keys
+    assert lib.convattn_kernel_path(C.byref(desc(Nq=65535 * 128 - 16, Nk=65535 * 128 - 16, d=64)), _lib.OP_BWD) == 1
+    assert lib.convattn_kernel_path(C.byref(desc(Nq=65535 * 128, Nk=65535 * 128, d=64)), _lib.OP_BWD) == 0

@@ -146,3 +146,24 @@ def test_scores_at_the_fp16_limit_of_the_score_tile_stay_finite():
     # rows before key 90 enters any window (row < 90) never see the large score
     O_ref, _, _ = oracle_fwd(Qb, Kb, V, W, True)
     assert max_abs(out[0][:, :, :90], O_ref[:, :, :90]) <= TOL_BF16
+
+
+def test_backward_falls_back_to_the_two_passes_when_the_workspace_is_capped(monkeypatch):
+    # the one-pass backward's workspace is O(N^2); beyond the cap the two passes with O(N) scratch run
+    Q, K, V, dO, W = rand_case(1, 2, 260, 260, 128, 6, 11, torch.bfloat16, seed=4)
+    ref = oracle_bwd(Q, K, V, W, dO, True)
+    g = [t.to(DEV) for t in (Q, K, V, dO, W)]
+    sc = scale_of(128)
+    O, M, L = ops.forward(g[0], g[1], g[2], g[4], sc, 5, 5, True, out_dtype=torch.bfloat16)
+    D, LSE = ops.bwd_preprocess(O, g[3], M, L)
+    monkeypatch.setenv("CONVATTN_MAX_WORKSPACE_BYTES", "1024")
+    dQ, dK, dV, dW = ops.backward(g[0], g[1], g[2], g[3], D, LSE, g[4], sc, 5, 5, True, out_dtype=torch.float32)
+    assert max_abs(dQ, ref[0]) <= TOL_BF16 and max_abs(dK, ref[1]) <= TOL_BF16 and max_abs(dV, ref[2]) <= TOL_BF16
+    assert rel_max(dW, ref[3]) <= TOL_DW_REL
+    # the low-memory dQ + dW pass asks for O(N) scratch only
+    import ctypes as C
+    from flash_multi_token_attention_amd import _lib
+    d_fast = ops._desc(g[0], g[1], g[4], sc, True, torch.float32)
+    d_low = ops._desc(g[0], g[1], g[4], sc, True, torch.float32, low_memory=True)
+    lib = _lib.load()
+    assert lib.convattn_dw_partial_bytes(C.byref(d_low)) < lib.convattn_dw_partial_bytes(C.byref(d_fast)) // 8
