@@ -334,7 +334,8 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
         const bf16_t *Vb = V + bh * p.Nk * D;
         // bands (times scale * log2 e: the convolved scores come out in log2 units) in LDS, one KB
         // per tap slot, written by one wave; the first barrier of the tile loop publishes them
-        const unsigned char *bands = smem + Lds::band_off;
+        // lane's 16 bytes of a band: the tap slot is a constant offset from one address register
+        const unsigned char *bands = smem + opaque((unsigned int)Lds::band_off + lane * 16);
         if (pr == 0) {
 #pragma unroll
             for (int t = 0; t < CQT; ++t)
@@ -421,6 +422,19 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
             if (it + 1 < n_tiles) stage_tile(it + 1);
             load_tile(r0 + 2 * BR);
             TS(2);
+            // dC of a tile that has none (entirely above the diagonal, or the one after the last):
+            // zeros, so that the consumers read every tile alike
+            auto zero_dc = [&] {
+                // (address from the lane index afresh: nothing of this rare path stays in a register)
+                const unsigned int ln = opaque((unsigned int)lane);
+                unsigned char *Cs = c_stage(it) + 2 * (ln & 15) * CST + (ln >> 4) * 8;
+#pragma unroll
+                for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+                    for (int ob = 0; ob < 2; ++ob)
+                        *reinterpret_cast<u32x2 *>(Cs + ob * CST + cb * 32) = (u32x2){0u, 0u};
+            };
+            if (it == n_tiles) zero_dc();
             if (it >= n_tiles) continue;
 #if defined(CHAIN_SKIP_ROLE) && CHAIN_SKIP_ROLE == 0
             continue;
@@ -484,7 +498,7 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
                         constexpr int delta = t0 - (CQT - 1);
                         constexpr int f = delta & 1, s = (f - delta) / 2;
                         f16x8 tf_cur = tf_prev;
-                        if constexpr (t0 < CQT) tf_cur = *reinterpret_cast<const f16x8 *>(bands + t0 * 1024 + lane * 16);
+                        if constexpr (t0 < CQT) tf_cur = *reinterpret_cast<const f16x8 *>(bands + t0 * 1024);
                         unsigned int sh[NSB][2];
 #pragma unroll
                         for (int kb = 0; kb < NSB; ++kb)
@@ -539,6 +553,7 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
                     for (int kb = 0; kb < NSB; ++kb)
 #pragma unroll
                         for (int f = 0; f < 2; ++f) { prev_pd[kb][f][0] = pd[kb][f][0]; prev_pd[kb][f][1] = pd[kb][f][1]; }
+                    zero_dc();
                 }
             };
             if (is_skipped(r0)) ptile(std::true_type{}, std::false_type{});
@@ -551,11 +566,11 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
         // ================================ consumer ================================
         const float *w_head = W + (size_t)h * cq * ck;
         // flipped bands (times the softmax scale) in LDS, one KB per tap slot, written by one wave
-        unsigned char *bands = smem + Lds::band_off + CQT * 1024;
+        unsigned char *bands = smem + opaque((unsigned int)Lds::band_off + CQT * 1024 + lane * 16);
         if (pr == 0) {
 #pragma unroll
             for (int t = 0; t < CQT; ++t)
-                *reinterpret_cast<f16x8 *>(bands + t * 1024 + lane * 16) = band_frag<CQT>(t, w_head, cq, ck, pk, g, n, true, p.scale);
+                *reinterpret_cast<f16x8 *>(bands + t * 1024) = band_frag<CQT>(t, w_head, cq, ck, pk, g, n, true, p.scale);
         }
         // dW: this wave takes the key blocks of two pairs (pg) and half of the tap slots (t_lo ..)
         constexpr int TH = (CQT + 1) / 2;
@@ -618,16 +633,16 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
             // packed dC^T of tile u, as the producer's lanes held it (zeros when the tile has none)
             unsigned int cur_dc[NCB][2][2];
             {
-                // read unconditionally (a buffer of this workgroup; its contents mean nothing when the
-                // tile has no dC), then cleared: no branch per load
+                // read unconditionally: the producer writes zeros for a tile without dC; what the first
+                // iteration reads (nothing written yet) is dropped before any use
                 const unsigned char *Cl = smem + opaque((unsigned int)(c_stage(max(u, 0)) - smem) + 2 * n * CST + 4 * g * 2);
 #pragma unroll
                 for (int cb = 0; cb < NCB; ++cb)
 #pragma unroll
                     for (int f = 0; f < 2; ++f) {
                         const u32x2 t2 = *reinterpret_cast<const u32x2 *>(Cl + f * CST + cb * 32);
-                        cur_dc[cb][f][0] = u_ok ? t2[0] : 0u;
-                        cur_dc[cb][f][1] = u_ok ? t2[1] : 0u;
+                        cur_dc[cb][f][0] = t2[0];
+                        cur_dc[cb][f][1] = t2[1];
                     }
             }
             if (v_ok && !(CHAIN_ABLATE & 512)) {
@@ -644,7 +659,7 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
                     constexpr int e = decltype(E)::value, f = e & 1, s = e >> 1;
                     // tap slot CQT-1-e for parity 0 (this step's band), CQT-e for parity 1 (the last step's)
                     f16x8 tb_cur = tb_prev;
-                    if constexpr (e <= CQT - 1) tb_cur = *reinterpret_cast<const f16x8 *>(bands + (CQT - 1 - e) * 1024 + lane * 16);
+                    if constexpr (e <= CQT - 1) tb_cur = *reinterpret_cast<const f16x8 *>(bands + (CQT - 1 - e) * 1024);
                     unsigned int sh[NCB][2];
 #pragma unroll
                     for (int cb = 0; cb < NCB; ++cb)
@@ -698,28 +713,41 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
                     a_hi[tt] = opaque(ring0 + min(rb, rb - S_RING) * SST);
                 }
                 // score block jb' = 0..4 of the group: block jb' & 1 (or 2 for the last) of pair 2 pg + jb' / 2
-                auto s_frag = [&](int jbp, int tt) {
-                    const int dq = min(jbp >> 1, NP - 1 - 2 * pg), kb = jbp - 2 * dq;   // dq: wave-uniform
-                    bf16x4 l4 = lds_tr64(smem + a_lo[tt] + dq * Lds::pair_bytes + kb * 32);
-                    bf16x4 h4 = lds_tr64(smem + a_hi[tt] + dq * Lds::pair_bytes + kb * 32);
+                // (blocks 0..3: a constant offset from the lane's address; block 4 is block 0 of the pair
+                // after the group or, for the last group, block 2 of its second pair: a[][] of it apart)
+                const unsigned int off4 = pg == NP / 2 - 1 ? Lds::pair_bytes + 64 : 2 * Lds::pair_bytes;
+                unsigned int a4_lo[TH], a4_hi[TH];
+#pragma unroll
+                for (int tt = 0; tt < TH; ++tt) { a4_lo[tt] = a_lo[tt] + off4; a4_hi[tt] = a_hi[tt] + off4; }
+                auto s_frag = [&](auto JBP, int tt) {
+                    constexpr int jbp = decltype(JBP)::value;
+                    constexpr int off = (jbp >> 1) * Lds::pair_bytes + (jbp & 1) * 32;
+                    bf16x4 l4, h4;
+                    if constexpr (jbp < 4) {
+                        l4 = lds_tr64(smem + a_lo[tt] + off);
+                        h4 = lds_tr64(smem + a_hi[tt] + off);
+                    } else {
+                        l4 = lds_tr64(smem + a4_lo[tt]);
+                        h4 = lds_tr64(smem + a4_hi[tt]);
+                    }
                     return __builtin_bit_cast(f16x8, __builtin_shufflevector(l4, h4, 0, 1, 2, 3, 4, 5, 6, 7));
                 };
-                // dC^T block jb of the group (zeros where the pair's tile is entirely above the diagonal:
-                // its dC buffer was not written)
+                // dC^T block jb of the group (a pair whose tile is entirely above the diagonal holds zeros)
                 auto c_frag = [&](int jb) {
                     const int dq = jb >> 1;
-                    const bool has = !(causal && r0u + BR - 1 < k0 + (2 * pg + dq) * WK - 8);
-                    const f16x8 v = __builtin_bit_cast(
+                    return __builtin_bit_cast(
                         f16x8, read_tr(smem + Lds::pair_off + 2 * pg * Lds::pair_bytes + Lds::s_bytes + (u & 1) * (BR * CST) +
                                            c_lane + dq * Lds::pair_bytes, CST, (jb & 1) * 16));
-                    return has ? v : (f16x8)(_Float16)0.f;
                 };
                 // Software pipeline over the four key blocks: the operands of block jb + 1 are read
                 // while block jb is multiplied.  Every tap slot of the wave is multiplied, also the
                 // zero taps in front of a narrow window (their sums are not used).
                 f16x8 af = c_frag(0), b0[TH], b1[TH];
 #pragma unroll
-                for (int tt = 0; tt < TH; ++tt) { b0[tt] = s_frag(0, tt); b1[tt] = s_frag(1, tt); }
+                for (int tt = 0; tt < TH; ++tt) {
+                    b0[tt] = s_frag(std::integral_constant<int, 0>{}, tt);
+                    b1[tt] = s_frag(std::integral_constant<int, 1>{}, tt);
+                }
                 static_for<4>([&](auto JB) {
                     constexpr int jb = decltype(JB)::value;
                     f16x8 af_n = af, b2[TH];
@@ -728,7 +756,7 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
                     if constexpr (jb < 3) {
                         af_n = c_frag(jb + 1);
 #pragma unroll
-                        for (int tt = 0; tt < TH; ++tt) b2[tt] = s_frag(jb + 2, tt);
+                        for (int tt = 0; tt < TH; ++tt) b2[tt] = s_frag(std::integral_constant<int, jb + 2>{}, tt);
                         SCHED_DS_READ_ID(2 + 2 * TH, 40 + jb);
                     }
 #pragma unroll
