@@ -8,8 +8,14 @@ scripts/benchmark_fwd_inference_conv_attn.py:45-122: last-row decode over a KV c
 Each line times this library beside torch's ``scaled_dot_product_attention`` on the same
 tensors (the reference's "Flash Attention" comparison line) and prints a markdown table:
 
-    python -m flash_multi_token_attention_amd.benchmarks train  [--quick]
-    python -m flash_multi_token_attention_amd.benchmarks decode [--quick]
+    python -m flash_multi_token_attention_amd.benchmarks train  [--quick] [--md FILE]
+    python -m flash_multi_token_attention_amd.benchmarks decode [--quick] [--md FILE]
+    python -m flash_multi_token_attention_amd.benchmarks plot --train FILE [--decode FILE] [--out DIR]
+
+``plot`` draws the figures of the reference's plot scripts from such tables
+(scripts/plot_benchmark_seq_len.py:233-310: speed relative to the comparison line, forward
+times and backward times against the sequence length, one line per window;
+scripts/plot_fwd_inference_speedup.py: decode time against the cache length) and needs no GPU.
 
 The reference's third line, its materialising PyTorch module, allocates [B,H,N,N] fp32
 temporaries and is not part of this package; it is timed on the CPU by ``bench.py``.
@@ -24,8 +30,8 @@ from typing import Callable, List
 import torch
 import torch.nn.functional as F
 
-from .conv_attn.inference import fwd_conv_attn_inference
-from .conv_attn.module import ConvAttentionCUDA
+import os
+import sys
 
 # (seq_len, window) pairs of the reference's suite, then the sweep of its plots.
 TRAIN_SUITE = [(256, 3), (512, 3), (1024, 3), (2048, 7), (2048, 11), (4096, 11), (8192, 11)]
@@ -50,6 +56,7 @@ def time_ms(fn: Callable[[], None], iters: int = 20, warmup: int = 5) -> float:
 
 
 def train_case(B: int, H: int, N: int, d: int, k: int, iters: int) -> dict:
+    from .conv_attn.module import ConvAttentionCUDA
     dev = "cuda:0"
     g = torch.Generator().manual_seed(42)
     Q, K, V, dO = (torch.randn(B, H, N, d, generator=g).to(torch.bfloat16).to(dev) for _ in range(4))
@@ -85,6 +92,7 @@ def train_case(B: int, H: int, N: int, d: int, k: int, iters: int) -> dict:
 
 
 def decode_case(B: int, H: int, Nk: int, d: int, c_q: int, c_k: int, iters: int) -> dict:
+    from .conv_attn.inference import fwd_conv_attn_inference
     dev = "cuda:0"
     g = torch.Generator().manual_seed(42)
     Q = torch.randn(B, H, c_q, d, generator=g).to(torch.bfloat16).to(dev)
@@ -104,38 +112,130 @@ def decode_case(B: int, H: int, Nk: int, d: int, c_q: int, c_k: int, iters: int)
     return r
 
 
+def parse_table(path: str) -> List[dict]:
+    """Rows of the first markdown table of ``path`` as dicts keyed by the header cells."""
+    head, rows = None, []
+    for line in open(path):
+        line = line.strip()
+        if not line.startswith("|"):
+            continue
+        cells = [c.strip() for c in line.strip("|").split("|")]
+        if head is None:
+            head = cells
+        elif not all(set(c) <= set("-: ") for c in cells):
+            rows.append(dict(zip(head, cells)))
+    return rows
+
+
+def plot(train_md: str, decode_md: str, out_dir: str) -> List[str]:
+    """The reference's figures from the tables ``train`` / ``decode`` print; returns the files written."""
+    import matplotlib
+    matplotlib.use("Agg")
+    import matplotlib.pyplot as plt
+
+    os.makedirs(out_dir, exist_ok=True)
+    written = []
+
+    def save(name):
+        path = os.path.join(out_dir, name)
+        plt.tight_layout()
+        plt.savefig(path, dpi=150, bbox_inches="tight")
+        plt.close()
+        written.append(path)
+
+    if train_md:
+        rows = parse_table(train_md)
+        windows = sorted({r["window"] for r in rows}, key=lambda w: int(w.split("x")[0]))
+        per = {w: sorted((r for r in rows if r["window"] == w), key=lambda r: int(r["N"])) for w in windows}
+        # 1: time of the comparison line over this library's time (the reference plots its CUDA
+        # module against its PyTorch module; the line both suites share is plain attention)
+        plt.figure(figsize=(10, 5))
+        for w in windows:
+            n = [int(r["N"]) for r in per[w]]
+            plt.plot(n, [float(r["sdpa fwd"]) / float(r["conv fwd"]) for r in per[w]], "o-", label=f"forward, {w}")
+            plt.plot(n, [float(r["sdpa fwd+bwd"]) / float(r["conv fwd+bwd"]) for r in per[w]], "s--", label=f"forward+backward, {w}")
+        plt.axhline(1.0, color="gray", linewidth=0.8)
+        plt.xscale("log", base=2); plt.xlabel("Sequence length"); plt.ylabel("SDPA time / conv-attention time")
+        plt.title("Conv-attention against plain attention (MI355X)"); plt.grid(True, alpha=0.3); plt.legend(fontsize=7)
+        save("benchmark_seq_len_speedup.png")
+        # 2 and 3: absolute times
+        for col, other, name, title in (("conv fwd", "sdpa fwd", "benchmark_seq_len_forward_times.png", "Forward"),
+                                        ("conv fwd+bwd", "sdpa fwd+bwd", "benchmark_seq_len_backward_times.png", "Forward+backward")):
+            plt.figure(figsize=(10, 5))
+            for w in windows:
+                n = [int(r["N"]) for r in per[w]]
+                plt.plot(n, [float(r[col]) for r in per[w]], "o-", label=f"conv-attention {w}")
+            w0 = windows[0]
+            plt.plot([int(r["N"]) for r in per[w0]], [float(r[other]) for r in per[w0]], "g^-", label="SDPA (no convolution)")
+            plt.xscale("log", base=2); plt.yscale("log"); plt.xlabel("Sequence length"); plt.ylabel("Time (ms)")
+            plt.title(f"{title} time against sequence length (MI355X)"); plt.grid(True, alpha=0.3); plt.legend(fontsize=7)
+            save(name)
+    if decode_md:
+        rows = sorted(parse_table(decode_md), key=lambda r: int(r["Nk"]))
+        n = [int(r["Nk"]) for r in rows]
+        plt.figure(figsize=(10, 5))
+        plt.plot(n, [float(r["conv decode"]) for r in rows], "ro-", label="conv-attention decode step")
+        plt.plot(n, [float(r["sdpa last row"]) for r in rows], "g^-", label="SDPA, last row")
+        plt.xscale("log", base=2); plt.yscale("log"); plt.xlabel("Cache length"); plt.ylabel("Time (ms)")
+        plt.title("Decode step against cache length (MI355X)"); plt.grid(True, alpha=0.3); plt.legend()
+        save("fwd_inference_times.png")
+    return written
+
+
 def main(argv=None) -> None:
     ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
-    ap.add_argument("which", choices=["train", "decode"])
+    ap.add_argument("which", choices=["train", "decode", "plot"])
     ap.add_argument("--quick", action="store_true", help="the reference's 7-line suite / fewer decode lengths")
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--batch", type=int, default=None)
     ap.add_argument("--heads", type=int, default=None)
     ap.add_argument("--head-dim", type=int, default=None)
+    ap.add_argument("--md", default=None, help="train / decode: also write the table, with its command line, to this file")
+    ap.add_argument("--train", default=None, help="plot: table written by `train`")
+    ap.add_argument("--decode", default=None, help="plot: table written by `decode`")
+    ap.add_argument("--out", default="plots", help="plot: directory for the figures")
     a = ap.parse_args(argv)
+    if a.which == "plot":
+        if not (a.train or a.decode):
+            raise SystemExit("plot needs --train and / or --decode")
+        for path in plot(a.train, a.decode, a.out):
+            print(path)
+        return
     if not torch.cuda.is_available():
         raise SystemExit("benchmarks need a GPU")
-    print(f"device: {torch.cuda.get_device_name(0)}")
+    lines: List[str] = []
+
+    def emit(line: str) -> None:
+        print(line, flush=True)
+        lines.append(line)
+
+    emit("Command: python -m flash_multi_token_attention_amd.benchmarks " + " ".join(argv if argv is not None else sys.argv[1:]))
+    emit("")
+    emit(f"device: {torch.cuda.get_device_name(0)}")
     if a.which == "train":
         B, H, d = a.batch or 1, a.heads or 8, a.head_dim or 64
-        print(f"B={B} H={H} d={d} bf16 causal; ms per call (median of {a.iters}); "
-              "TFLOP/s = 14 d N(N+1)/2 B H / fwd+bwd time")
-        print("| N | window | conv fwd | conv fwd+bwd | sdpa fwd | sdpa fwd+bwd | fwd+bwd vs sdpa | conv TFLOP/s |")
-        print("|---|---|---|---|---|---|---|---|")
+        emit(f"B={B} H={H} d={d} bf16 causal; ms per call (median of {a.iters}); "
+             "TFLOP/s = 14 d N(N+1)/2 B H / fwd+bwd time")
+        emit("")
+        emit("| N | window | conv fwd | conv fwd+bwd | sdpa fwd | sdpa fwd+bwd | fwd+bwd vs sdpa | conv TFLOP/s |")
+        emit("|---|---|---|---|---|---|---|---|")
         for N, k in (TRAIN_SUITE if a.quick else TRAIN_SWEEP):
             r = train_case(B, H, N, d, k, a.iters)
-            print(f"| {N} | {k}x{k} | {r['conv_fwd']:.3f} | {r['conv_fwd_bwd']:.3f} | {r['sdpa_fwd']:.3f} | "
-                  f"{r['sdpa_fwd_bwd']:.3f} | {r['conv_fwd_bwd'] / r['sdpa_fwd_bwd']:.2f}x | {r['conv_tflops']:.1f} |",
-                  flush=True)
+            emit(f"| {N} | {k}x{k} | {r['conv_fwd']:.3f} | {r['conv_fwd_bwd']:.3f} | {r['sdpa_fwd']:.3f} | "
+                 f"{r['sdpa_fwd_bwd']:.3f} | {r['conv_fwd_bwd'] / r['sdpa_fwd_bwd']:.2f}x | {r['conv_tflops']:.1f} |")
     else:
         B, H, d = a.batch or 2, a.heads or 2, a.head_dim or 64
-        print(f"B={B} H={H} d={d} bf16, 11x11 window, 11 resident query rows; ms per call (median of {a.iters}); "
-              "GB/s = K and V bytes / time")
-        print("| Nk | conv decode | sdpa last row | conv GB/s |")
-        print("|---|---|---|---|")
+        emit(f"B={B} H={H} d={d} bf16, 11x11 window, 11 resident query rows; ms per call (median of {a.iters}); "
+             "GB/s = K and V bytes / time")
+        emit("")
+        emit("| Nk | conv decode | sdpa last row | conv GB/s |")
+        emit("|---|---|---|---|")
         for Nk in (DECODE_SWEEP[:2] if a.quick else DECODE_SWEEP):
             r = decode_case(B, H, Nk, d, 11, 11, a.iters)
-            print(f"| {Nk} | {r['conv']:.4f} | {r['sdpa']:.4f} | {r['conv_gbs']:.0f} |", flush=True)
+            emit(f"| {Nk} | {r['conv']:.4f} | {r['sdpa']:.4f} | {r['conv_gbs']:.0f} |")
+    if a.md:
+        with open(a.md, "w") as f:
+            f.write("\n".join(lines) + "\n")
 
 
 if __name__ == "__main__":

@@ -198,13 +198,14 @@ struct ChainArgs {
 #define CHAIN_CONST_AS
 #endif
 
-// One role of the workgroup (ROLE 0 = producer waves, 1 = consumer waves) as a function of its
-// own: the two roles have disjoint register sets of 256 each, and compiled into one function body
-// the register allocator spills where either role alone does not.
+// One role of the workgroup (ROLE 0 = producer waves, 1 = consumer waves).  The two roles have
+// disjoint register sets of 256 each and are both inlined into the kernel: as called functions
+// each wave would save and restore the 112 callee-saved vector registers it uses through scratch
+// memory (0.47 GB written and read back per C3 launch, 7 % of the kernel's time).
 // WANT: bit 0 = dK and dV, bit 1 = dS (for dQ) and dW; the passes behind the separate dK / dV and dQ + dW
 // operations leave the other half out.
 template <int D, int CQT, typename TO, int ROLE, int WANT>
-__device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainArgs *args_in) {
+__device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_in) {
     // the pointer arrives in vector registers; it is the same in every lane, and as a scalar the
     // arguments are fetched with scalar loads into scalar registers
     const unsigned long long av = reinterpret_cast<unsigned long long>(args_in);
@@ -685,7 +686,9 @@ __device__ __attribute__((noinline)) void chain_role(const CHAIN_CONST_AS ChainA
                         bf16x4 sv;
 #pragma unroll
                         for (int r = 0; r < 4; ++r) sv[r] = (bf16_t)ds[sb][ob][r];
-                        if constexpr (WANT_QW) *reinterpret_cast<bf16x4 *>(ds_blk + (2 * n + ob) * WK + sb * 16 + 4 * g) = sv;
+                        // block layout [row parity][key half][16 row pairs][16 keys]: the 64 lanes of a store
+                        // write 512 contiguous bytes
+                        if constexpr (WANT_QW) *reinterpret_cast<bf16x4 *>(ds_blk + ((ob * 2 + sb) * 16 + n) * 16 + 4 * g) = sv;
                         if constexpr (WANT_KV) *reinterpret_cast<bf16x4 *>(ds_tile + (2 * n + ob) * PST + (sb * 16 + 4 * g) * 2) = sv;
                     }
             }

@@ -1,9 +1,11 @@
 // dQ = dS K on bf16 MFMA (gfx950), second step of the one-pass backward of bwd_chain_mfma.hip.
 //
 // dS comes from the key-stationary kernel as bf16 blocks [key tile of 32][row tile of 32] of
-// [32 rows][32 keys] (row-major; the softmax scale and the dC scale are already in it).  Workgroup
+// 32 rows x 32 keys, laid out [row parity][key half][row pair][16 keys] (the order in which that
+// kernel's lanes hold it: each of its stores and each load here covers whole 128-byte lines; the
+// softmax scale and the dC scale are already in it).  Workgroup
 // = 4 waves = 128 query rows of one (batch, head); wave w owns rows i0 + 32w .. +31 and all D
-// columns.  The product is dQ^T[d][row] += K^T[d][key] dS^T[key][row]: 16 bytes of a dS row are 8
+// columns.  The product is dQ^T[d][row] += K^T[d][key] dS^T[key][row]: 16 bytes of a block are 8
 // keys of one row, which is the B operand of a lane as it lies in memory, so dS goes from global
 // memory straight into the MFMA operand registers (every block is read once, by one wave, in
 // whole 1 KB pieces).  Only K passes through LDS (row-major, read with transpose reads), staged
@@ -77,7 +79,7 @@ __global__ __launch_bounds__(NW * 64) void dq_rows_kernel(Problem p, const bf16_
             for (int ob = 0; ob < 2; ++ob) {
                 // every dS block is read once: non-temporal, so that it does not push K out of the caches
                 u32x4 v = __builtin_nontemporal_load(
-                    reinterpret_cast<const u32x4 *>(ws + blk * BLK + (ob * 16 + n) * kChainKeys + 8 * g));
+                    reinterpret_cast<const u32x4 *>(ws + blk * BLK + ((ob * 2 + (g >> 1)) * 16 + n) * 16 + 8 * (g & 1)));
                 sr[kp][ob] = zero_unless(ok, v);
             }
         }
@@ -119,11 +121,11 @@ __global__ __launch_bounds__(NW * 64) void dq_rows_kernel(Problem p, const bf16_
         if (s + 1 < n_steps) run_step(s + 1, kr_b, sr_b);
     }
 
-    // lane n of block ob = row 16 ob + n of the wave's 32; 4 consecutive head-dim columns per block
+    // lane n of block ob = row 2 n + ob of the wave's 32; 4 consecutive head-dim columns per block
     const float inv = dc_scale ? 1.f / dc_scale[2 * bh] : 1.f;
 #pragma unroll
     for (int ob = 0; ob < 2; ++ob) {
-        const int qpos = rw + ob * 16 + n;
+        const int qpos = rw + 2 * n + ob;
         if (qpos < p.Nq) {
             TO *orow = dQ + (bh * p.Nq + qpos) * D;
 #pragma unroll
