@@ -303,8 +303,9 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
             gr[i] = __builtin_amdgcn_raw_buffer_load_b128(g_rsrc, ((r0 + row) * D + cc * 8) * 2, 0, 0);
         }
         if constexpr (producer) {
+            // raw values: arithmetic on them here would wait for the loads in this iteration
             ls = 1e30f; dd = 0.f;  // rows past the end: exp2(C - LSE) = 0
-            if (tt < BR && r0 + tt < p.Nq) { ls = lse_b[r0 + tt] * kLog2e - dcs_log2; dd = dl_b[r0 + tt]; }
+            if (tt < BR && r0 + tt < p.Nq) { ls = lse_b[r0 + tt]; dd = dl_b[r0 + tt]; }
         }
     };
     auto stage_tile = [&](int t) {
@@ -321,7 +322,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
         }
         if constexpr (producer) {
             float *st = stat_slot(t);
-            if (tt < BR) { st[tt] = ls; st[BR + tt] = dd; }
+            if (tt < BR) { st[tt] = ls * kLog2e - dcs_log2; st[BR + tt] = dd; }
         }
     };
 

@@ -72,15 +72,14 @@ __global__ __launch_bounds__(NW * 64) void dq_rows_kernel(Problem p, const bf16_
 #pragma unroll
         for (int kp = 0; kp < 2; ++kp) {
             const int kt = s * 2 + kp;
-            // the block exists when its first key is a key and (causal) not after the tile's last row
-            const bool ok = row_ok && kt * kChainKeys < p.Nk && (!causal || kt * kChainKeys <= rw + 31);
             const size_t blk = (size_t)min(kt, n_kt - 1) * n_rt + min(rt, n_rt - 1);
 #pragma unroll
             for (int ob = 0; ob < 2; ++ob) {
-                // every dS block is read once: non-temporal, so that it does not push K out of the caches
-                u32x4 v = __builtin_nontemporal_load(
+                // every dS block is read once: non-temporal, so that it does not push K out of the caches.
+                // Raw: blocks that do not exist are cleared where the registers are used (a select here
+                // would wait for the load within this step)
+                sr[kp][ob] = __builtin_nontemporal_load(
                     reinterpret_cast<const u32x4 *>(ws + blk * BLK + ((ob * 2 + (g >> 1)) * 16 + n) * 16 + 8 * (g & 1)));
-                sr[kp][ob] = zero_unless(ok, v);
             }
         }
     };
@@ -94,9 +93,13 @@ __global__ __launch_bounds__(NW * 64) void dq_rows_kernel(Problem p, const bf16_
         }
         bf16x8 sf[2][2];
 #pragma unroll
-        for (int kp = 0; kp < 2; ++kp)
+        for (int kp = 0; kp < 2; ++kp) {
+            const int kt = s * 2 + kp;
+            // the block exists when its first key is a key and (causal) not after the tile's last row
+            const bool ok = row_ok && kt * kChainKeys < p.Nk && (!causal || kt * kChainKeys <= rw + 31);
 #pragma unroll
-            for (int ob = 0; ob < 2; ++ob) sf[kp][ob] = __builtin_bit_cast(bf16x8, sr[kp][ob]);
+            for (int ob = 0; ob < 2; ++ob) sf[kp][ob] = __builtin_bit_cast(bf16x8, zero_unless(ok, sr[kp][ob]));
+        }
         __syncthreads();
         load_step(s + 2, kr, sr);
         if (causal && s * BKS > rw + 31) return;  // every key of the step is after the wave's rows
