@@ -203,9 +203,10 @@ def dkdv_backward(Q, K, V, dO, D, L, conv_kernel, scale, pad_q, pad_k, causal,
 
 
 def max_workspace_bytes() -> int:
-    """Largest workspace ``backward`` allocates before it falls back to the two separate passes
-    with O(N) scratch (``CONVATTN_MAX_WORKSPACE_BYTES``, default 64 GiB)."""
-    return int(os.environ.get("CONVATTN_MAX_WORKSPACE_BYTES", 64 << 30))
+    """Largest workspace ``backward`` allocates in one piece (``CONVATTN_MAX_WORKSPACE_BYTES``,
+    default 16 GiB).  Beyond it the one-pass backward runs over groups of heads that fit, and if
+    not even one (batch, head) fits, the two separate passes with O(N) scratch run instead."""
+    return int(os.environ.get("CONVATTN_MAX_WORKSPACE_BYTES", 16 << 30))
 
 
 def backward(Q, K, V, dO, D, L, conv_kernel, scale, pad_q, pad_k, causal,
@@ -213,16 +214,37 @@ def backward(Q, K, V, dO, D, L, conv_kernel, scale, pad_q, pad_k, causal,
     """-> (dQ, dK, dV, dconv_kernel) from one pass over the score tiles: the results of
     ``dq_backward`` + ``dkdv_backward`` (same arguments) without computing the scores, the
     convolution and dC twice.  Needs a workspace the size of the bf16 dS matrix
-    (B*H*Nq*Nk*2 bytes: 2.2 GB at B4 H16 N4096, 17 GB at B1 H32 N16384); when that exceeds
-    ``max_workspace_bytes()`` or cannot be allocated, the two passes with O(N) scratch run instead."""
+    (B*H*Nq*Nk*2 bytes: 2.2 GB at B4 H16 N4096, 17 GB at B1 H32 N16384).  A workspace above
+    ``max_workspace_bytes()`` is avoided by running the pass once per group of heads of one batch
+    entry (every (batch, head) pair is independent; dconv_kernel is summed over the batch in index
+    order); when a single pair does not fit or the allocation fails, the two passes with O(N)
+    scratch run instead."""
     W, D, L, desc = _bwd_common(Q, K, V, dO, D, L, conv_kernel, scale, pad_q, pad_k, causal,
                                 out_dtype, exact)
     lib = _lib.load()
     nbytes = lib.convattn_bwd_fused_workspace_bytes(C.byref(desc))
     if nbytes == 0:
         _lib.check(lib.convattn_validate(C.byref(desc), _lib.OP_BWD), "conv_attn.backward")
+    B, H = Q.shape[0], Q.shape[1]
+    cap = max_workspace_bytes()
+    if nbytes > cap:
+        per_pair = -(-nbytes // (B * H))
+        group = min(H, int(0.95 * cap) // per_pair)
+        if group >= 1:
+            dQ = torch.empty(Q.shape, dtype=out_dtype, device=Q.device)
+            dK = torch.empty(K.shape, dtype=out_dtype, device=Q.device)
+            dV = torch.empty(V.shape, dtype=out_dtype, device=Q.device)
+            dW = torch.zeros(W.shape, dtype=torch.float32, device=Q.device)
+            for b in range(B):
+                for h0 in range(0, H, group):
+                    sl = (slice(b, b + 1), slice(h0, min(H, h0 + group)))
+                    gq, gk, gv, gw = backward(Q[sl], K[sl], V[sl], dO[sl], D[sl], L[sl], conv_kernel[sl[1]], scale,
+                                              pad_q, pad_k, causal, out_dtype, exact)
+                    dQ[sl], dK[sl], dV[sl] = gq, gk, gv
+                    dW[sl[1]] += gw
+            return dQ, dK, dV, dW
     ws = None
-    if nbytes <= max_workspace_bytes():
+    if nbytes <= cap:
         try:
             ws = torch.empty(nbytes, dtype=torch.uint8, device=Q.device)
         except torch.OutOfMemoryError:

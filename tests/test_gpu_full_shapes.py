@@ -167,3 +167,24 @@ def test_backward_falls_back_to_the_two_passes_when_the_workspace_is_capped(monk
     d_low = ops._desc(g[0], g[1], g[4], sc, True, torch.float32, low_memory=True)
     lib = _lib.load()
     assert lib.convattn_dw_partial_bytes(C.byref(d_low)) < lib.convattn_dw_partial_bytes(C.byref(d_fast)) // 8
+
+
+@pytest.mark.gpu
+def test_backward_runs_by_groups_of_heads_when_the_workspace_is_capped(monkeypatch):
+    # a cap that one (batch, head) pair fits but the whole problem does not: the one-pass backward
+    # runs per group of heads; dQ, dK, dV are those of the single call, dW is summed over the batch
+    Q, K, V, dO, W = rand_case(2, 3, 300, 300, 128, 6, 11, torch.bfloat16, seed=5)
+    g = [t.to(DEV) for t in (Q, K, V, dO, W)]
+    sc = scale_of(128)
+    O, M, L = ops.forward(g[0], g[1], g[2], g[4], sc, 5, 5, True, out_dtype=torch.bfloat16)
+    D, LSE = ops.bwd_preprocess(O, g[3], M, L)
+    whole = ops.backward(g[0], g[1], g[2], g[3], D, LSE, g[4], sc, 5, 5, True, out_dtype=torch.float32)
+    import ctypes as C
+    from flash_multi_token_attention_amd import _lib
+    desc = ops._desc(g[0], g[1], g[4], sc, True, torch.float32)
+    nbytes = _lib.load().convattn_bwd_fused_workspace_bytes(C.byref(desc))
+    monkeypatch.setenv("CONVATTN_MAX_WORKSPACE_BYTES", str(nbytes // 6 * 2 + 4096))   # two heads of one batch entry
+    parts = ops.backward(g[0], g[1], g[2], g[3], D, LSE, g[4], sc, 5, 5, True, out_dtype=torch.float32)
+    for a, b in zip(whole[:3], parts[:3]):
+        assert torch.equal(a, b)
+    assert rel_max(parts[3], whole[3]) <= 1e-5
