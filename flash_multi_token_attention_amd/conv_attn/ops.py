@@ -231,6 +231,7 @@ def backward(Q, K, V, dO, D, L, conv_kernel, scale, pad_q, pad_k, causal,
         per_pair = -(-nbytes // (B * H))
         group = min(H, int(0.95 * cap) // per_pair)
         if group >= 1:
+            group = -(-H // -(-H // group))   # equal groups: H heads in ceil(H / group) launches
             dQ = torch.empty(Q.shape, dtype=out_dtype, device=Q.device)
             dK = torch.empty(K.shape, dtype=out_dtype, device=Q.device)
             dV = torch.empty(V.shape, dtype=out_dtype, device=Q.device)

@@ -12,10 +12,10 @@
 //   consumer (waves 4-7), one tile behind: dV^T += dO^T P and dW += dC^T S with the operands read
 //       back through LDS transpose reads; two tiles behind: dS^T by flipped-band MFMAs over the
 //       packed dC^T (rows below a tile come from the next tile, hence the extra tile of delay),
-//       dS -> workspace (bf16, [row][key] blocks) and -> LDS, dK^T += Q^T dS.
-// One workgroup barrier per tile; Q and dO tiles are staged row-major with the 16-byte chunks of a
-// 256-byte line XOR-swizzled by the line number, so that both the row fragments (b128) and the
-// transpose reads are spread over all banks without padding.
+//       dS -> workspace (bf16 blocks of 32 rows x 32 keys in the order the lanes hold them) and
+//       -> LDS, dK^T += Q^T dS.
+// One workgroup barrier per tile; Q and dO tiles are staged row-major with rows padded by 16 bytes
+// (row fragments are 128-bit reads, the transposed operands of dV / dK 64-bit transpose reads).
 //
 // dW[a][b] = sum_i sum_j dC[i][j] S_m[i+a-pq][j+b-pk] is computed as G_a = dC^T S(rows shifted by
 // a), a [key j] x [key j'] product contracted over the rows on the matrix cores; only its

@@ -176,3 +176,16 @@ def test_kernel_path_selection(lib):
     # the backward kernels' tiles are 128 rows or keys
     assert lib.convattn_kernel_path(C.byref(desc(Nq=65535 * 128 - 16, Nk=65535 * 128 - 16, d=64)), _lib.OP_BWD) == 1
     assert lib.convattn_kernel_path(C.byref(desc(Nq=65535 * 128, Nk=65535 * 128, d=64)), _lib.OP_BWD) == 0
+
+
+def test_benchmark_tables_parse_and_plot(tmp_path):
+    # the sweep tables committed under profiles/ are what `benchmarks plot` draws the reference's figures from
+    import os
+    from flash_multi_token_attention_amd import benchmarks
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    train, decode = os.path.join(root, "profiles", "sweep_train.md"), os.path.join(root, "profiles", "sweep_decode.md")
+    rows = benchmarks.parse_table(train)
+    assert len(rows) == len(benchmarks.TRAIN_SWEEP) and {"N", "window", "conv fwd", "sdpa fwd+bwd"} <= set(rows[0])
+    assert all(float(r["conv fwd"]) > 0 for r in rows)
+    files = benchmarks.plot(train, decode, str(tmp_path))
+    assert len(files) == 4 and all(os.path.getsize(f) > 10000 for f in files)
