@@ -28,6 +28,17 @@ class Desc(C.Structure):
     ]
 
 
+class KvLayout(C.Structure):
+    """struct convattn_kv_layout of include/convattn.h."""
+    _fields_ = [
+        ("H_kv", C.c_int32), ("page_size", C.c_int32),
+        ("batch_stride", C.c_int64), ("head_stride", C.c_int64), ("page_stride", C.c_int64),
+        ("block_table", C.c_void_p),
+        ("table_stride", C.c_int32), ("reserved", C.c_int32),
+        ("seq_lens", C.c_void_p),
+    ]
+
+
 _P = C.c_void_p
 _D = C.POINTER(Desc)
 _SIGNATURES = {
@@ -49,6 +60,7 @@ _SIGNATURES = {
     "convattn_decode_partial_bytes": (C.c_size_t, [_D]),
     "convattn_decode": (C.c_int, [_D] + [_P] * 8),
     "convattn_decode_strided": (C.c_int, [_D] + [_P] * 4 + [C.c_longlong] * 2 + [_P] * 4),
+    "convattn_decode_kv": (C.c_int, [_D] + [_P] * 3 + [C.POINTER(KvLayout)] + [_P] * 5),
     "convattn_decode_combine": (C.c_int, [_D] + [_P] * 7),
     "convattn_decode_noalloc_bytes": (C.c_size_t, [_D]),
     "convattn_decode_noalloc": (C.c_int, [_D] + [_P] * 4 + [C.c_longlong] * 2 + [_P] * 4),

@@ -316,6 +316,97 @@ def decode(Q, K, V, conv_kernel, k_splits, scale, causal=False, out_dtype=torch.
     return O, M, L, (O_part, M_part, L_part)
 
 
+def _decode_kv(Q, K, V, layout: "_lib.KvLayout", Nk: int, conv_kernel, k_splits, scale, causal, out_dtype, what: str):
+    B, H, r, d = Q.shape
+    c_q, c_k = conv_kernel.shape[1], conv_kernel.shape[2]
+    W = _weights(conv_kernel, H, c_q - 1, (c_k - 1) // 2, Q.device)
+    if not k_splits:
+        k_splits = default_k_splits(B, H, Nk)
+    if out_dtype not in _DT:
+        raise RuntimeError("out_dtype must be bfloat16 or float32")
+    desc = _lib.Desc(B, H, r, Nk, d, c_q, c_k, float(scale), int(bool(causal)), _DT[Q.dtype], _DT[out_dtype],
+                     int(k_splits), 0)
+    lib = _lib.load()
+    rc = lib.convattn_validate(C.byref(desc), _lib.OP_DECODE)
+    if rc == _lib.ERR_QROWS:
+        raise ValueError(f"Q sequence length must be <= 16 for inference, got {r}")
+    _lib.check(rc, what)
+    O_part = torch.empty((B, H, k_splits, d), dtype=torch.float32, device=Q.device)
+    M_part = torch.empty((B, H, k_splits), dtype=torch.float32, device=Q.device)
+    L_part = torch.empty((B, H, k_splits), dtype=torch.float32, device=Q.device)
+    O = torch.empty((B, H, 1, d), dtype=out_dtype, device=Q.device)
+    M = torch.empty((B, H, 1), dtype=torch.float32, device=Q.device)
+    L = torch.empty((B, H, 1), dtype=torch.float32, device=Q.device)
+    st = _stream(Q)
+    _lib.check(lib.convattn_decode_kv(C.byref(desc), _ptr(Q), _ptr(K), _ptr(V), C.byref(layout), _ptr(W),
+                                      _ptr(O_part), _ptr(M_part), _ptr(L_part), st), what)
+    _lib.check(lib.convattn_decode_combine(C.byref(desc), _ptr(O_part), _ptr(M_part), _ptr(L_part), _ptr(O),
+                                           _ptr(M), _ptr(L), st), what + " (combine)")
+    return O, M, L, (O_part, M_part, L_part)
+
+
+def _seq_lens(seq_lens, B: int, device):
+    if seq_lens is None:
+        return None
+    if seq_lens.dtype != torch.int32 or seq_lens.shape != (B,) or not seq_lens.is_cuda or not seq_lens.is_contiguous():
+        raise RuntimeError("seq_lens must be a contiguous int32 CUDA tensor [batch]")
+    return seq_lens
+
+
+def decode_gqa(Q, K, V, conv_kernel, k_splits, scale, causal=False, out_dtype=torch.float32, seq_lens=None):
+    """Decode step with shared KV heads: Q [B,H,r,d], K and V [B,H_kv,Nk,d] (or views
+    ``cache[:, :, :Nk]`` of a longer cache), H a multiple of H_kv; query head h reads KV head
+    h // (H // H_kv), the window weights stay per query head.  ``seq_lens`` (int32 [B] on the device,
+    each 1..Nk) gives every batch entry its own number of keys.  -> (O [B,H,1,d], M, L, partials).
+    bf16 only (the streaming decode kernel)."""
+    for t, n in ((Q, "Q"), (K, "K"), (V, "V")):
+        if t.dim() != 4:
+            raise RuntimeError(f"{n} must be [batch, heads, seq_len, d_head]")
+        if not t.is_cuda:
+            raise RuntimeError(f"{n} must be a CUDA tensor")
+    if not Q.is_contiguous():
+        raise RuntimeError("Q must be contiguous")
+    if not (K.is_contiguous() or _is_cache_view(K)) or K.stride() != V.stride() or K.shape != V.shape:
+        raise RuntimeError("K and V must be [batch, kv_heads, seq_len, d_head] tensors (or views of a longer cache) "
+                           "with the same shape and strides")
+    B, H, r, d = Q.shape
+    H_kv, Nk = K.shape[1], K.shape[2]
+    if K.shape[0] != B or K.shape[3] != d or H % H_kv != 0 or K.dtype != Q.dtype:
+        raise RuntimeError("K / V must match Q in batch, head dim and dtype, and their head count must divide Q's")
+    bs, hs = (H_kv * Nk * d, Nk * d) if K.is_contiguous() else (K.stride(0), K.stride(1))
+    sl = _seq_lens(seq_lens, B, Q.device)
+    layout = _lib.KvLayout(H_kv, 0, bs, hs, 0, None, 0, 0, _ptr(sl) if sl is not None else None)
+    return _decode_kv(Q, K, V, layout, Nk, conv_kernel, k_splits, scale, causal, out_dtype, "conv_attn.decode_gqa")
+
+
+def decode_paged(Q, k_pool, v_pool, block_table, seq_lens, max_seq_len, conv_kernel, k_splits, scale,
+                 causal=False, out_dtype=torch.float32):
+    """Decode step over a paged KV cache: pools [n_pages, H_kv, page_size, d] (page_size a power
+    of two >= 16), ``block_table`` int32 [B, pages per sequence] on the device (keys
+    [i*page_size, (i+1)*page_size) of entry b live in page block_table[b, i]), ``seq_lens`` int32
+    [B] on the device or None (then every entry has ``max_seq_len`` keys); ``max_seq_len`` is a host
+    integer (no device synchronisation).  H may be a multiple of H_kv.
+    -> (O [B,H,1,d], M, L, partials).  bf16 only (the streaming decode kernel)."""
+    if k_pool.dim() != 4 or k_pool.shape != v_pool.shape or not k_pool.is_contiguous() or not v_pool.is_contiguous():
+        raise RuntimeError("k_pool and v_pool must be contiguous [n_pages, kv_heads, page_size, d_head] tensors of one shape")
+    if Q.dim() != 4 or not Q.is_contiguous() or not Q.is_cuda or not k_pool.is_cuda:
+        raise RuntimeError("Q must be a contiguous CUDA tensor [batch, heads, rows, d_head]")
+    B, H, r, d = Q.shape
+    _, H_kv, ps, dk = k_pool.shape
+    if dk != d or H % H_kv != 0 or k_pool.dtype != Q.dtype:
+        raise RuntimeError("the pools must match Q in head dim and dtype, and their head count must divide Q's")
+    if (block_table.dtype != torch.int32 or block_table.dim() != 2 or block_table.shape[0] != B
+            or not block_table.is_cuda or not block_table.is_contiguous()):
+        raise RuntimeError("block_table must be a contiguous int32 CUDA tensor [batch, pages per sequence]")
+    if block_table.shape[1] * ps < max_seq_len:
+        raise RuntimeError("block_table has fewer pages than max_seq_len needs")
+    sl = _seq_lens(seq_lens, B, Q.device)
+    layout = _lib.KvLayout(H_kv, ps, 0, ps * d, H_kv * ps * d, _ptr(block_table), block_table.shape[1], 0,
+                           _ptr(sl) if sl is not None else None)
+    return _decode_kv(Q, k_pool, v_pool, layout, int(max_seq_len), conv_kernel, k_splits, scale, causal, out_dtype,
+                      "conv_attn.decode_paged")
+
+
 def forward_inference(Q, K, V, conv_kernel, k_splits, scale, pad_q, pad_k, causal,
                       num_k_blocks=None):
     """Reference-shaped decode op -> (O [B,H,k_splits,d], M, L [B,H,k_splits]) fp32

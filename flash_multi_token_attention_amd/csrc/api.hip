@@ -116,6 +116,7 @@ const char *convattn_strerror(int code) {
         case CONVATTN_ERR_CAUSAL_SHAPE: return "causal conv-attention needs seq_len_q == seq_len_k";
         case CONVATTN_ERR_LDS: return "convolution window too large for the 160 KB of LDS at this head dimension";
         case CONVATTN_ERR_TOO_LARGE: return "batch or head count too large for one launch";
+        case CONVATTN_ERR_KV_LAYOUT: return "KV layout rejected: H must be a multiple of H_kv, page_size a power of two >= 16, strides multiples of 8 that cover a page / a sequence, the block table long enough, and the descriptor one of the streaming decode kernel (bf16, d 64 or 128, c_k <= 17)";
         case CONVATTN_ERR_SCRATCH: return "the split partials of this decode step do not fit the library's built-in scratch (convattn_decode_noalloc): use fewer splits or convattn_decode";
         default: break;
     }
@@ -340,6 +341,44 @@ int convattn_decode_strided(const convattn_desc *desc, const void *q, const void
     if (pick_path(desc, p, CONVATTN_OP_DECODE) == 1)
         return (int)decode_stream(p, q, k, v, w, o_part, m_part, l_part, s);
     return (int)generic_decode(p, desc->in_dtype, q, k, v, w, o_part, m_part, l_part, s);
+}
+
+int convattn_decode_kv(const convattn_desc *desc, const void *q, const void *k, const void *v,
+                       const convattn_kv_layout *kv, const float *w, float *o_part, float *m_part,
+                       float *l_part, void *stream) {
+    Problem p;
+    int rc = validate(desc, CONVATTN_OP_DECODE, &p);
+    if (rc) return rc;
+    if (!kv) return CONVATTN_ERR_NULL;
+    if (pick_path(desc, p, CONVATTN_OP_DECODE) != 1) return CONVATTN_ERR_KV_LAYOUT;
+    const int h_kv = kv->H_kv > 0 ? kv->H_kv : p.H;
+    if (h_kv > p.H || p.H % h_kv != 0 || kv->reserved != 0) return CONVATTN_ERR_KV_LAYOUT;
+    KvArgs a = {};
+    a.group = p.H / h_kv;
+    a.seq_lens = kv->seq_lens;
+    const long long row = p.d;
+    if (kv->page_size == 0) {
+        // contiguous rows per (batch, KV head); KV heads and batches must not overlap
+        if (kv->head_stride < (long long)p.Nk * row || kv->head_stride % 8 != 0 || kv->batch_stride % 8 != 0 ||
+            (p.B > 1 && kv->batch_stride < (long long)p.Nk * row))
+            return CONVATTN_ERR_KV_LAYOUT;
+        p.kv_bstride = kv->batch_stride;
+    } else {
+        const int ps = kv->page_size;
+        if (ps < 16 || (ps & (ps - 1)) != 0 || !kv->block_table || kv->head_stride < (long long)ps * row ||
+            kv->head_stride % 8 != 0 || kv->page_stride % 8 != 0 || kv->page_stride < (long long)ps * row ||
+            (long long)kv->table_stride * ps < p.Nk)
+            return CONVATTN_ERR_KV_LAYOUT;
+        a.table = kv->block_table;
+        a.table_stride = kv->table_stride;
+        a.page_stride = kv->page_stride;
+        a.page_shift = __builtin_ctz((unsigned)ps);
+        p.kv_bstride = 0;
+    }
+    p.kv_hstride = kv->head_stride;
+    REQUIRE_PTR(q); REQUIRE_PTR(k); REQUIRE_PTR(v); REQUIRE_PTR(w);
+    REQUIRE_PTR(o_part); REQUIRE_PTR(m_part); REQUIRE_PTR(l_part);
+    return (int)decode_stream_kv(p, a, q, k, v, w, o_part, m_part, l_part, static_cast<hipStream_t>(stream));
 }
 
 size_t convattn_decode_noalloc_bytes(const convattn_desc *desc) {

@@ -19,19 +19,19 @@
 //     window and softmax of this iteration are computed.
 // The 4 waves merge their (m, l, o) in LDS and store one un-normalised partial
 // per split; convattn_decode_combine merges the splits.
+//
+// Where the rows live is a parameter of the kernel (KvArgs): query heads may share KV heads
+// (head h reads KV head h / group), the rows of a (batch, KV head) may be contiguous or come in
+// pages named by a block table (PAGED instance: one table lookup per row load; the lookups of the
+// rows a lane loads next are independent of everything else in the iteration), and every batch
+// entry may have its own number of keys.
 #include "mfma_common.hpp"
 
 namespace convattn {
 namespace {
 
-// 8 bf16 of the row nearest to `row` inside [0, N), as a non-temporal load: every K / V row is
-// read exactly once, and keeping it out of the caches' replacement order is worth 10 % of the
-// stream's bandwidth here.
-template <int D>
-__device__ __forceinline__ u32x4 load_row16_stream(const bf16_t *__restrict__ base, int row, int N, int col) {
-    const int rr = min(max(row, 0), N - 1);
-    return __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base + (size_t)rr * D + col));
-}
+// Non-temporal loads below: every K / V row is read exactly once, and keeping it out of the
+// caches' replacement order is worth 10 % of the stream's bandwidth here.
 
 constexpr int NW = 4;
 constexpr int IT = 64;             // keys per wave iteration
@@ -41,9 +41,9 @@ constexpr int SROW = SW + 4;       // floats per strip row (84)
 __device__ __forceinline__ float bf16_lo(unsigned int w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float bf16_hi(unsigned int w) { return __uint_as_float(w & 0xffff0000u); }
 
-template <int D>
+template <int D, bool PAGED>
 __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(
-    Problem p, const bf16_t *__restrict__ Q, const bf16_t *__restrict__ K,
+    Problem p, KvArgs kv, const bf16_t *__restrict__ Q, const bf16_t *__restrict__ K,
     const bf16_t *__restrict__ V, const float *__restrict__ W, float *__restrict__ O_part,
     float *__restrict__ M_part, float *__restrict__ L_part) {
     constexpr int KS = D / 32;
@@ -63,8 +63,21 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(
     const int cq = p.c_q, ck = p.c_k, pk = p.pk;
     const size_t bh = (size_t)b * p.H + h;
     const bf16_t *Qb = Q + bh * p.Nq * D;
-    const bf16_t *Kb = K + b * p.kv_bstride + h * p.kv_hstride;
-    const bf16_t *Vb = V + b * p.kv_bstride + h * p.kv_hstride;
+    const int hk = h / kv.group;
+    const int Nk = kv.seq_lens ? min(max(kv.seq_lens[b], 0), p.Nk) : p.Nk;   // keys of this batch entry
+    const bf16_t *Kb = K + (PAGED ? 0 : b * p.kv_bstride) + hk * p.kv_hstride;
+    const bf16_t *Vb = V + (PAGED ? 0 : b * p.kv_bstride) + hk * p.kv_hstride;
+    const int *tbl = PAGED ? kv.table + (size_t)b * kv.table_stride : nullptr;
+    // 8 bf16 at column `col` of the row nearest to `row` inside [0, Nk)
+    auto load_row = [&](const bf16_t *base, int row, int col) -> u32x4 {
+        const int rr = min(max(row, 0), Nk - 1);
+        const bf16_t *src;
+        if constexpr (PAGED)
+            src = base + (size_t)tbl[rr >> kv.page_shift] * kv.page_stride + (size_t)(rr & ((1 << kv.page_shift) - 1)) * D;
+        else
+            src = base + (size_t)rr * D;
+        return __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + col));
+    };
     float *strip = s_strip[wave];
 
     for (int i = tid; i < cq * ck; i += NW * 64) s_w[i] = W[(size_t)h * cq * ck + i];
@@ -82,11 +95,11 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(
         }
     }
     // Causal variant: tap row a sits at position Nk - c_q + a and sees no later key.
-    const int row_pos = p.causal ? p.Nk - cq + n : 0x7fffffff;
+    const int row_pos = p.causal ? Nk - cq + n : 0x7fffffff;
 
     // Key range of this wave: the split's chunk cut into 4 runs of whole iterations.
-    const int chunk = (p.Nk + p.n_splits - 1) / p.n_splits;
-    const int s_lo = sp * chunk, s_hi = min(p.Nk, s_lo + chunk);
+    const int chunk = (Nk + p.n_splits - 1) / p.n_splits;
+    const int s_lo = sp * chunk, s_hi = min(Nk, s_lo + chunk);
     const int per_wave = ((chunk + NW - 1) / NW + IT - 1) / IT * IT;
     const int lo = s_lo + wave * per_wave, hi = min(s_hi, lo + per_wave);
 
@@ -104,8 +117,11 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(
             f32x4 a4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                bf16x8 kf = __builtin_bit_cast(bf16x8, load_row16_nb<D>(Kb, lo - 8 + n, p.Nk, ks * 32 + g * 8));
-                a4 = mfma_bf16(kf, qf[ks], a4);
+                // (keys before the first or after the last one score zero: the window's padding)
+                const int row = lo - 8 + n;
+                u32x4 raw = load_row(Kb, row, ks * 32 + g * 8);
+                if (row < 0 || row >= Nk) raw = (u32x4){0u, 0u, 0u, 0u};
+                a4 = mfma_bf16(__builtin_bit_cast(bf16x8, raw), qf[ks], a4);
             }
             if (n < cq) {
 #pragma unroll
@@ -122,13 +138,13 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(
         for (int blk = 0; blk < 4; ++blk)
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks)
-                kreg[blk][ks] = load_row16_stream<D>(Kb, lo + 8 + blk * 16 + n, p.Nk, ks * 32 + g * 8);
+                kreg[blk][ks] = load_row(Kb, lo + 8 + blk * 16 + n, ks * 32 + g * 8);
 
         for (int j0 = lo; j0 < hi; j0 += IT) {
             // V of this iteration: keys j0 .. j0+63
             u32x4 vreg[VT];
 #pragma unroll
-            for (int t = 0; t < VT; ++t) vreg[t] = load_row16_stream<D>(Vb, j0 + RPI * t + gph, p.Nk, cc * 8);
+            for (int t = 0; t < VT; ++t) vreg[t] = load_row(Vb, j0 + RPI * t + gph, cc * 8);
 
             // scores of keys j0+8 .. j0+71 -> strip columns 16 .. 79
 #pragma unroll
@@ -143,10 +159,10 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(
                         const int key = j0 + 8 + blk * 16 + 4 * g + r;
                         a4[r] = (key > row_pos) ? 0.f : a4[r] * scale;
                     }
-                    if (j0 + IT + 8 > p.Nk) {  // keys past the end of the cache score zero (K rows were clamped)
+                    if (j0 + IT + 8 > Nk) {  // keys past the end of the cache score zero (K rows were clamped)
 #pragma unroll
                         for (int r = 0; r < 4; ++r)
-                            if (j0 + 8 + blk * 16 + 4 * g + r >= p.Nk) a4[r] = 0.f;
+                            if (j0 + 8 + blk * 16 + 4 * g + r >= Nk) a4[r] = 0.f;
                     }
                     *reinterpret_cast<f32x4 *>(strip + n * SROW + 16 + blk * 16 + 4 * g) = a4;
                 }
@@ -157,7 +173,7 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(
                 for (int blk = 0; blk < 4; ++blk)
 #pragma unroll
                     for (int ks = 0; ks < KS; ++ks)
-                        kreg[blk][ks] = load_row16_stream<D>(Kb, j0 + IT + 8 + blk * 16 + n, p.Nk, ks * 32 + g * 8);
+                        kreg[blk][ks] = load_row(Kb, j0 + IT + 8 + blk * 16 + n, ks * 32 + g * 8);
             }
             __builtin_amdgcn_wave_barrier();
 
@@ -246,16 +262,28 @@ bool decode_stream_ok(const Problem &p, int in_dt, unsigned flags) {
            p.pk <= 8 && p.c_q <= 16;
 }
 
+hipError_t decode_stream_kv(const Problem &p, const KvArgs &kv, const void *q, const void *k, const void *v,
+                            const float *w, float *o_part, float *m_part, float *l_part, hipStream_t s) {
+    dim3 grid(p.n_splits, p.H, p.B);
+#define CONVATTN_DECODE_LAUNCH(DD, PG)                                                                       \
+    decode_stream_kernel<DD, PG><<<grid, NW * 64, 0, s>>>(p, kv, (const bf16_t *)q, (const bf16_t *)k,         \
+                                                         (const bf16_t *)v, w, o_part, m_part, l_part)
+    if (p.d == 128) {
+        if (kv.table) CONVATTN_DECODE_LAUNCH(128, true);
+        else CONVATTN_DECODE_LAUNCH(128, false);
+    } else {
+        if (kv.table) CONVATTN_DECODE_LAUNCH(64, true);
+        else CONVATTN_DECODE_LAUNCH(64, false);
+    }
+#undef CONVATTN_DECODE_LAUNCH
+    return hipGetLastError();
+}
+
 hipError_t decode_stream(const Problem &p, const void *q, const void *k, const void *v, const float *w,
                          float *o_part, float *m_part, float *l_part, hipStream_t s) {
-    dim3 grid(p.n_splits, p.H, p.B);
-    if (p.d == 128)
-        decode_stream_kernel<128><<<grid, NW * 64, 0, s>>>(p, (const bf16_t *)q, (const bf16_t *)k,
-                                                            (const bf16_t *)v, w, o_part, m_part, l_part);
-    else
-        decode_stream_kernel<64><<<grid, NW * 64, 0, s>>>(p, (const bf16_t *)q, (const bf16_t *)k,
-                                                           (const bf16_t *)v, w, o_part, m_part, l_part);
-    return hipGetLastError();
+    KvArgs kv = {};
+    kv.group = 1;
+    return decode_stream_kv(p, kv, q, k, v, w, o_part, m_part, l_part, s);
 }
 
 }  // namespace convattn

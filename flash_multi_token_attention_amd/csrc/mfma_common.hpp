@@ -258,6 +258,17 @@ hipError_t mfma_dq_from_rows(const Problem &p, int out_dt, const void *k, const 
 
 // ---- decode as an HBM stream (decode_stream.hip) ----
 bool decode_stream_ok(const Problem &p, int in_dt, unsigned flags);
+// Where the decode kernel finds K and V rows beyond Problem's batch / head strides.
+struct KvArgs {
+    const int *table;       // block table [B][table_stride] of page numbers, or null: contiguous rows
+    const int *seq_lens;    // keys per batch entry [B] (clamped to Problem::Nk), or null: Nk for all
+    long long page_stride;  // elements between pages of the pool
+    int table_stride;
+    int page_shift;         // log2 of the keys per page
+    int group;              // query heads per KV head (>= 1)
+};
+hipError_t decode_stream_kv(const Problem &p, const KvArgs &kv, const void *q, const void *k, const void *v,
+                            const float *w, float *o_part, float *m_part, float *l_part, hipStream_t s);
 hipError_t decode_stream(const Problem &p, const void *q, const void *k, const void *v, const float *w,
                          float *o_part, float *m_part, float *l_part, hipStream_t s);
 

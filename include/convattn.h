@@ -62,7 +62,9 @@ typedef enum convattn_status {
     CONVATTN_ERR_CAUSAL_SHAPE = -10, /* causal training pass needs Nq == Nk */
     CONVATTN_ERR_LDS = -11,        /* the window needs more LDS than a CU has */
     CONVATTN_ERR_TOO_LARGE = -12,  /* a launch dimension would overflow */
-    CONVATTN_ERR_SCRATCH = -13     /* convattn_decode_noalloc: partials larger than the built-in scratch */
+    CONVATTN_ERR_SCRATCH = -13,    /* convattn_decode_noalloc: partials larger than the built-in scratch */
+    CONVATTN_ERR_KV_LAYOUT = -14   /* convattn_decode_kv: bad KV-head count, page size, stride or table, or a
+                                      descriptor outside the streaming decode kernel (bf16, d 64 / 128, c_k <= 17) */
 } convattn_status;
 
 /* Flags for convattn_desc.flags */
@@ -213,6 +215,42 @@ int convattn_decode(const convattn_desc *desc, const void *q, const void *k, con
 int convattn_decode_strided(const convattn_desc *desc, const void *q, const void *k, const void *v,
                             const float *w, long long kv_batch_stride, long long kv_head_stride,
                             float *o_part, float *m_part, float *l_part, void *stream);
+
+/*
+ * Where K and V of a decode step live, beyond the dense and strided [B,H,Nk,d] forms above: shared
+ * KV heads (grouped-query attention), a paged cache and per-sequence lengths.  The reference has
+ * none of the three (its shim takes dense [B,H,Nk,d] tensors, conv_attn/
+ * flash_conv_attention_inference.py:33-93); this is the widening of its decode entry for serving.
+ *   H_kv          KV heads (0 = H).  H % H_kv == 0; query head h reads KV head h / (H / H_kv).  W stays
+ *                 per query head.
+ *   page_size     0: the rows of one (batch, KV head) are contiguous, batches batch_stride and KV heads
+ *                 head_stride elements apart (as in convattn_decode_strided).
+ *                 > 0 (a power of two >= 16): k and v are pools of pages; page p of KV head g starts at
+ *                 p * page_stride + g * head_stride and holds page_size rows of d elements; keys
+ *                 [i * page_size, (i+1) * page_size) of batch entry b are page block_table[b * table_stride + i]
+ *                 (device memory, int32).  A pool laid out [n_pages][H_kv][page_size][d] has
+ *                 page_stride = H_kv*page_size*d and head_stride = page_size*d.
+ *   seq_lens      optional device int32 [B]: number of keys of every batch entry (1 .. desc->Nk); NULL =
+ *                 desc->Nk for all.  desc->Nk is the longest sequence; splits cut every sequence evenly.
+ * Strides are multiples of 8 elements.  Only descriptors that run the streaming decode kernel are
+ * accepted (bf16 K and V, d 64 or 128, c_k <= 17: convattn_kernel_path(desc, CONVATTN_OP_DECODE) == 1).
+ */
+typedef struct convattn_kv_layout {
+    int32_t H_kv;
+    int32_t page_size;
+    int64_t batch_stride;
+    int64_t head_stride;
+    int64_t page_stride;
+    const int32_t *block_table;
+    int32_t table_stride;
+    int32_t reserved;          /* 0 */
+    const int32_t *seq_lens;
+} convattn_kv_layout;
+
+/* convattn_decode with K and V described by `kv`; partials and convattn_decode_combine as above. */
+int convattn_decode_kv(const convattn_desc *desc, const void *q, const void *k, const void *v,
+                       const convattn_kv_layout *kv, const float *w, float *o_part, float *m_part,
+                       float *l_part, void *stream);
 
 /*
  * Log-sum-exp merge of the split partials into O [B,H,1,d] (out_dtype), M, L

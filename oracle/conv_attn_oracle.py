@@ -169,6 +169,31 @@ def decode(Q_res, K, V, W, scale: Optional[float] = None, causal: bool = False):
     return torch.matmul(E / L.unsqueeze(-1), V), M, L
 
 
+def gather_paged(pool: torch.Tensor, block_table: torch.Tensor, seq_len: int, b: int) -> torch.Tensor:
+    """Dense [H_kv, seq_len, d] rows of batch entry ``b`` from a pool [n_pages, H_kv, page_size, d]:
+    keys [i*page_size, (i+1)*page_size) are page ``block_table[b, i]`` (the layout vLLM-style serving
+    caches use; the reference has no paged cache, so this only restates the indexing)."""
+    ps = pool.shape[2]
+    n = (seq_len + ps - 1) // ps
+    pages = pool[block_table[b, :n].long()]                     # [n, H_kv, ps, d]
+    return pages.permute(1, 0, 2, 3).reshape(pool.shape[1], n * ps, pool.shape[3])[:, :seq_len]
+
+
+def decode_kv(Q_res, K_of, V_of, W, seq_lens, scale: Optional[float] = None, causal: bool = False):
+    """Decode step over shared KV heads and per-sequence lengths, one batch entry at a time:
+    ``K_of(b)`` / ``V_of(b)`` return the dense [H_kv, seq_lens[b], d] rows of entry b; query head h
+    reads KV head h // (H // H_kv).  Returns O [B,H,1,d], M, L [B,H,1] (``decode`` per entry)."""
+    B, H = Q_res.shape[0], Q_res.shape[1]
+    outs = []
+    for b in range(B):
+        Kb, Vb = K_of(b), V_of(b)
+        rep = H // Kb.shape[0]
+        Kb = Kb.repeat_interleave(rep, dim=0).unsqueeze(0)
+        Vb = Vb.repeat_interleave(rep, dim=0).unsqueeze(0)
+        outs.append(decode(Q_res[b:b + 1], Kb[:, :, :seq_lens[b]], Vb[:, :, :seq_lens[b]], W, scale, causal))
+    return tuple(torch.cat([o[i] for o in outs], dim=0) for i in range(3))
+
+
 def combine_splits(O_part, M_part, L_part):
     """Merge per-split un-normalised partials: O_part [..., S, d], M_part,
     L_part [..., S] -> normalised O [..., d], M, L [...]."""

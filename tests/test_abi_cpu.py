@@ -189,3 +189,32 @@ def test_benchmark_tables_parse_and_plot(tmp_path):
     assert all(float(r["conv fwd"]) > 0 for r in rows)
     files = benchmarks.plot(train, decode, str(tmp_path))
     assert len(files) == 4 and all(os.path.getsize(f) > 10000 for f in files)
+
+
+def test_kv_layout_rejected_before_launch(lib):
+    # convattn_decode_kv checks the layout on the host: nothing below reaches a kernel launch
+    dd = desc(Nq=6, causal=0, n_splits=2, H=8, Nk=4096, d=128)
+    null, ok = C.c_void_p(0), C.c_void_p(4096)
+    row = dd.d
+
+    def call(layout, q=ok):
+        return lib.convattn_decode_kv(C.byref(dd), q, ok, ok, C.byref(layout), ok, ok, ok, ok, null)
+
+    dense = dict(H_kv=2, page_size=0, batch_stride=2 * dd.Nk * row, head_stride=dd.Nk * row, page_stride=0,
+                 block_table=None, table_stride=0, reserved=0, seq_lens=None)
+    assert call(_lib.KvLayout(**dense), q=null) == -1                                  # the layout is fine, q is NULL
+    assert call(_lib.KvLayout(**{**dense, "H_kv": 3})) == -14                          # 8 % 3 != 0
+    assert call(_lib.KvLayout(**{**dense, "head_stride": dd.Nk * row - 8})) == -14     # KV heads overlap
+    assert call(_lib.KvLayout(**{**dense, "reserved": 1})) == -14
+    paged = dict(H_kv=2, page_size=64, batch_stride=0, head_stride=64 * row, page_stride=2 * 64 * row,
+                 block_table=4096, table_stride=64, reserved=0, seq_lens=None)
+    assert call(_lib.KvLayout(**paged), q=null) == -1
+    assert call(_lib.KvLayout(**{**paged, "page_size": 48})) == -14                    # not a power of two
+    assert call(_lib.KvLayout(**{**paged, "page_size": 8, "head_stride": 8 * row, "page_stride": 16 * row})) == -14
+    assert call(_lib.KvLayout(**{**paged, "table_stride": 63})) == -14                 # 63 pages < 4096 keys
+    assert call(_lib.KvLayout(**{**paged, "block_table": None})) == -14
+    assert call(_lib.KvLayout(**{**paged, "page_stride": 64 * row - 8})) == -14
+    # fp32 inputs run the fp32-arithmetic decode kernel, which reads dense K / V only
+    dd32 = desc(Nq=6, causal=0, n_splits=2, H=8, Nk=4096, d=128, in_dtype=_lib.F32)
+    assert lib.convattn_decode_kv(C.byref(dd32), ok, ok, ok, C.byref(_lib.KvLayout(**dense)), ok, ok, ok, ok, null) == -14
+    assert b"KV layout" in lib.convattn_strerror(-14)
