@@ -285,7 +285,10 @@ int convattn_bwd_fused_dq(const convattn_desc *desc, const void *q, const void *
                                       static_cast<float *>(workspace), s);
     }
     const FusedWs lay = fused_ws(p);
-    if (!lay.chain) return (int)mfma_dq_from_ds(p, desc->out_dtype, k, workspace, dq, s);
+    if (!lay.chain) {
+        REQUIRE_PTR(D);
+        return (int)mfma_dq_from_ds(p, desc->out_dtype, k, workspace, D, dq, s);
+    }
     const float *scale = reinterpret_cast<const float *>(static_cast<const unsigned char *>(workspace) + lay.scale_off);
     return (int)mfma_dq_from_rows(p, desc->out_dtype, k, workspace, scale, dq, s);
 }

@@ -261,17 +261,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
         dcs = dc_scale[2 * bh];
         dcs_log2 = dc_scale[2 * bh + 1];
     } else {
-        float mx = 0.f;
-        for (int i = tid; i < p.Nq; i += NT) mx = fmaxf(mx, fabsf(dl_b[i]));
-        mx = wave_max(mx);
-        float *red = reinterpret_cast<float *>(smem + Lds::stat_off);
-        if (lane == 0) red[wave] = mx;
-        __syncthreads();
-        mx = 0.f;
-#pragma unroll
-        for (int w2 = 0; w2 < 2 * NP; ++w2) mx = fmaxf(mx, red[w2]);
-        __syncthreads();
-        dcs_log2 = (mx > 0.f && mx < 3e38f) ? fminf(fmaxf(floorf(8.f - __log2f(mx)), -100.f), 100.f) : 0.f;
+        dcs_log2 = dc_scale_log2_from_d(dl_b, p.Nq, tid, NT, reinterpret_cast<float *>(smem + Lds::stat_off));
         dcs = exp2f(dcs_log2);
     }
 

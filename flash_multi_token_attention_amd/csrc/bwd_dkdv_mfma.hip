@@ -95,6 +95,11 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
     const float *lse_b = LSE + bh * p.Nq;
     const float *dl_b = Dl + bh * p.Nq;
 
+    // dC is carried as fp16 times a power of two taken from D (dc_scale_log2_from_d): log2 of it comes
+    // off the staged LSE, its inverse goes onto dK and dV
+    const float dcs_log2 = dc_scale_log2_from_d(dl_b, p.Nq, tid, NW * 64, reinterpret_cast<float *>(smem));
+    const float dcs_inv = exp2f(-dcs_log2);
+
     f16x8 tf[CQT], tfl[CQT];
     load_bands<CQT>(tf, W + (size_t)h * cq * ck, cq, ck, pk, g, n, false, p.scale * kLog2e);
     load_bands<CQT>(tfl, W + (size_t)h * cq * ck, cq, ck, pk, g, n, true, p.scale);
@@ -143,7 +148,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
             gr[i] = load_row16_clamped<D>(dOb, r0 + row, p.Nq, cc * 8);
         }
         ls = 1e30f; dd = 0.f;  // rows past the end: exp2(C - LSE) = 0
-        if (tid < BR && r0 + tid < p.Nq) { ls = lse_b[r0 + tid] * kLog2e; dd = dl_b[r0 + tid]; }
+        if (tid < BR && r0 + tid < p.Nq) { ls = lse_b[r0 + tid] * kLog2e - dcs_log2; dd = dl_b[r0 + tid]; }
     };
     load_tile(r_begin);
     // One row tile.  EDGE tiles apply the causal / sequence-end masks; the others are far enough
@@ -446,10 +451,10 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                 if constexpr (sizeof(TO) == 2) {
                     bf16x4 ov;
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) ov[r] = (bf16_t)acc_k[m][db][r];
+                    for (int r = 0; r < 4; ++r) ov[r] = (bf16_t)(acc_k[m][db][r] * dcs_inv);
                     *reinterpret_cast<bf16x4 *>(dst) = ov;
                 } else {
-                    *reinterpret_cast<f32x4 *>(dst) = acc_k[m][db];
+                    *reinterpret_cast<f32x4 *>(dst) = acc_k[m][db] * dcs_inv;
                 }
             }
             if (key_v >= 0 && key_v < p.Nk) {
@@ -457,10 +462,10 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                 if constexpr (sizeof(TO) == 2) {
                     bf16x4 ov;
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) ov[r] = (bf16_t)acc_v[m][db][r];
+                    for (int r = 0; r < 4; ++r) ov[r] = (bf16_t)(acc_v[m][db][r] * dcs_inv);
                     *reinterpret_cast<bf16x4 *>(dst) = ov;
                 } else {
-                    *reinterpret_cast<f32x4 *>(dst) = acc_v[m][db];
+                    *reinterpret_cast<f32x4 *>(dst) = acc_v[m][db] * dcs_inv;
                 }
             }
         }

@@ -28,7 +28,8 @@ template <int D> struct GemmLds {
 
 template <int D, typename TO>
 __global__ __launch_bounds__(NW * 64) void dq_from_ds_kernel(Problem p, const bf16_t *__restrict__ K,
-                                                             const bf16_t *__restrict__ dS_ws, int n_kt,
+                                                             const bf16_t *__restrict__ dS_ws,
+                                                             const float *__restrict__ Dl, int n_kt,
                                                              int n_rt, TO *__restrict__ dQ) {
     using Lds = GemmLds<D>;
     constexpr int RST = Lds::RST;
@@ -49,6 +50,8 @@ __global__ __launch_bounds__(NW * 64) void dq_from_ds_kernel(Problem p, const bf
     const size_t bh = (size_t)b * p.H + h;
     const bf16_t *Kb = K + bh * p.Nk * D;
     const bf16_t *ws = dS_ws + bh * n_kt * n_rt * (size_t)BLK;
+    // the dS blocks carry the dC scale of their (batch, head): the same power of two, from the same D
+    const float dcs_inv = exp2f(-dc_scale_log2_from_d(Dl + bh * p.Nq, p.Nq, tid, NW * 64, reinterpret_cast<float *>(smem)));
 
     f32x4 acc[2][DB];
 #pragma unroll
@@ -138,10 +141,10 @@ __global__ __launch_bounds__(NW * 64) void dq_from_ds_kernel(Problem p, const bf
                 if constexpr (sizeof(TO) == 2) {
                     bf16x4 ov;
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) ov[r] = (bf16_t)acc[ob][db][r];
+                    for (int r = 0; r < 4; ++r) ov[r] = (bf16_t)(acc[ob][db][r] * dcs_inv);
                     *reinterpret_cast<bf16x4 *>(orow + col) = ov;
                 } else {
-                    *reinterpret_cast<f32x4 *>(orow + col) = acc[ob][db];
+                    *reinterpret_cast<f32x4 *>(orow + col) = acc[ob][db] * dcs_inv;
                 }
             }
         }
@@ -149,28 +152,28 @@ __global__ __launch_bounds__(NW * 64) void dq_from_ds_kernel(Problem p, const bf
 }
 
 template <int D, typename TO>
-hipError_t launch(const Problem &p, const void *k, const void *ds_ws, void *dq, hipStream_t s) {
+hipError_t launch(const Problem &p, const void *k, const void *ds_ws, const float *Dl, void *dq, hipStream_t s) {
     auto kern = dq_from_ds_kernel<D, TO>;
     constexpr int lds = GemmLds<D>::total;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return e;
     dim3 grid(p.H, p.B, (p.Nq + kDsRowShift + BQ - 1) / BQ);
-    kern<<<grid, NW * 64, lds, s>>>(p, (const bf16_t *)k, (const bf16_t *)ds_ws, mfma_ds_key_tiles(p),
+    kern<<<grid, NW * 64, lds, s>>>(p, (const bf16_t *)k, (const bf16_t *)ds_ws, Dl, mfma_ds_key_tiles(p),
                                     mfma_ds_row_tiles(p), (TO *)dq);
     return hipGetLastError();
 }
 
 }  // namespace
 
-hipError_t mfma_dq_from_ds(const Problem &p, int out_dt, const void *k, const void *ds_ws, void *dq,
-                           hipStream_t s) {
+hipError_t mfma_dq_from_ds(const Problem &p, int out_dt, const void *k, const void *ds_ws, const float *Dl,
+                           void *dq, hipStream_t s) {
     if (p.d == 128) {
-        if (out_dt == CONVATTN_BF16) return launch<128, bf16_t>(p, k, ds_ws, dq, s);
-        return launch<128, float>(p, k, ds_ws, dq, s);
+        if (out_dt == CONVATTN_BF16) return launch<128, bf16_t>(p, k, ds_ws, Dl, dq, s);
+        return launch<128, float>(p, k, ds_ws, Dl, dq, s);
     }
-    if (out_dt == CONVATTN_BF16) return launch<64, bf16_t>(p, k, ds_ws, dq, s);
-    return launch<64, float>(p, k, ds_ws, dq, s);
+    if (out_dt == CONVATTN_BF16) return launch<64, bf16_t>(p, k, ds_ws, Dl, dq, s);
+    return launch<64, float>(p, k, ds_ws, Dl, dq, s);
 }
 
 }  // namespace convattn

@@ -86,6 +86,10 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_mfma_kernel(
     load_bands<CQT>(tf, W + (size_t)h * cq * ck, cq, ck, pk, g, n, false, p.scale * kLog2e);
     load_bands<CQT>(tfl, W + (size_t)h * cq * ck, cq, ck, pk, g, n, true, p.scale);
 
+    // dC is carried as fp16 times a power of two taken from D (dc_scale_log2_from_d): log2 of it comes
+    // off LSE, its inverse goes onto dQ and the dW partial
+    const float dcs_log2 = dc_scale_log2_from_d(Dl + bh * p.Nq, p.Nq, tid, NW * 64, reinterpret_cast<float *>(smem));
+    const float dcs_inv = exp2f(-dcs_log2);
     bf16x8 qf[4][KS];   // Q rows r0-16 .. r0+47
     bf16x8 gf[3][KS];   // dO rows r0 .. r0+47
     float lse2[3], dl[3];
@@ -100,7 +104,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_mfma_kernel(
         for (int ks = 0; ks < KS; ++ks)
             gf[rb][ks] = __builtin_bit_cast(bf16x8, load_row16_nb<D>(dOb, r0 + rb * 16 + n, p.Nq, ks * 32 + g * 8));
         const int qpos = r0 + rb * 16 + n;
-        lse2[rb] = qpos < p.Nq ? LSE[bh * p.Nq + qpos] * kLog2e : 0.f;
+        lse2[rb] = qpos < p.Nq ? LSE[bh * p.Nq + qpos] * kLog2e - dcs_log2 : 0.f;
         dl[rb] = qpos < p.Nq ? Dl[bh * p.Nq + qpos] : 0.f;
     }
 
@@ -397,10 +401,10 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_mfma_kernel(
                 if constexpr (sizeof(TO) == 2) {
                     bf16x4 ov;
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) ov[r] = (bf16_t)acc_q[ob][db][r];
+                    for (int r = 0; r < 4; ++r) ov[r] = (bf16_t)(acc_q[ob][db][r] * dcs_inv);
                     *reinterpret_cast<bf16x4 *>(orow + col) = ov;
                 } else {
-                    *reinterpret_cast<f32x4 *>(orow + col) = acc_q[ob][db];
+                    *reinterpret_cast<f32x4 *>(orow + col) = acc_q[ob][db] * dcs_inv;
                 }
             }
         }
@@ -419,7 +423,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_mfma_kernel(
         float s = 0.f;
 #pragma unroll
         for (int w = 0; w < NW; ++w) s += red[(w * 16 + a) * 16 + bb];
-        dW_part[(bh * n_qt + qt) * ntap + tid] = s * p.scale;
+        dW_part[(bh * n_qt + qt) * ntap + tid] = s * p.scale * dcs_inv;
     }
 }
 

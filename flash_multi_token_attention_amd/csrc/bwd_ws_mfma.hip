@@ -111,6 +111,11 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
     const float *lse_b = LSE + bh * p.Nq;
     const float *dl_b = Dl + bh * p.Nq;
 
+    // dC is carried as fp16 times a power of two taken from D (dc_scale_log2_from_d): log2 of it comes
+    // off the staged LSE, its inverse goes onto dK, dV, the dW partial and (in the dQ product) dQ
+    const float dcs_log2 = dc_scale_log2_from_d(dl_b, p.Nq, tid, NT, reinterpret_cast<float *>(smem));
+    const float dcs_inv = exp2f(-dcs_log2);
+
     // no dC before the first tile, and nothing but zeros where a tile was skipped
     for (int c = tid; c < NP * Lds::pair_bytes / 16; c += NT)
         *reinterpret_cast<u32x4 *>(smem + Lds::stage_bytes + c * 16) = (u32x4){0u, 0u, 0u, 0u};
@@ -144,7 +149,7 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
             gr[i] = __builtin_amdgcn_raw_buffer_load_b128(g_rsrc, ((r0 + row) * D + cc * 8) * 2, 0, 0);
         }
         ls = 1e30f; dd = 0.f;  // rows past the end: exp2(C - LSE) = 0
-        if (tid < BR && r0 + tid < p.Nq) { ls = lse_b[r0 + tid] * kLog2e; dd = dl_b[r0 + tid]; }
+        if (tid < BR && r0 + tid < p.Nq) { ls = lse_b[r0 + tid] * kLog2e - dcs_log2; dd = dl_b[r0 + tid]; }
     };
     // Both roles: the registers of tile t into its Q blocks, dO slot and LSE / D slot.
     auto stage_tile = [&](int t) {
@@ -536,10 +541,10 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
                 if constexpr (sizeof(TO) == 2) {
                     bf16x4 ov;
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) ov[r] = (bf16_t)acc_k[m][db][r];
+                    for (int r = 0; r < 4; ++r) ov[r] = (bf16_t)(acc_k[m][db][r] * dcs_inv);
                     *reinterpret_cast<bf16x4 *>(dst) = ov;
                 } else {
-                    *reinterpret_cast<f32x4 *>(dst) = acc_k[m][db];
+                    *reinterpret_cast<f32x4 *>(dst) = acc_k[m][db] * dcs_inv;
                 }
             }
             if (key_v >= 0 && key_v < p.Nk) {
@@ -547,10 +552,10 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
                 if constexpr (sizeof(TO) == 2) {
                     bf16x4 ov;
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) ov[r] = (bf16_t)acc_v[m][db][r];
+                    for (int r = 0; r < 4; ++r) ov[r] = (bf16_t)(acc_v[m][db][r] * dcs_inv);
                     *reinterpret_cast<bf16x4 *>(dst) = ov;
                 } else {
-                    *reinterpret_cast<f32x4 *>(dst) = acc_v[m][db];
+                    *reinterpret_cast<f32x4 *>(dst) = acc_v[m][db] * dcs_inv;
                 }
             }
         }
@@ -588,7 +593,7 @@ __global__ __launch_bounds__(NT) void bwd_ws_mfma_kernel(
 #pragma unroll
         for (int w = 0; w < NP; ++w)
             sum += reinterpret_cast<const float *>(smem + Lds::stage_bytes + w * Lds::pair_bytes)[a * 16 + bb];
-        dW_part[(bh * gridDim.z + blockIdx.z) * ntap + tid] = sum * p.scale;
+        dW_part[(bh * gridDim.z + blockIdx.z) * ntap + tid] = sum * p.scale * dcs_inv;
     }
 }
 

@@ -41,6 +41,17 @@ constexpr float kMaxSlack = 6.f;  // log2 units a score may exceed its row's exp
 // window's halo, the other 33-CQT are its output rows.
 constexpr int wave_rows(int cqt) { return 33 - cqt; }
 
+#ifdef FWD_TS
+__device__ long long g_fwd_ts[4][64][8];
+#define FTS(i)                                                                                     \
+    do {                                                                                           \
+        if (lane == 0 && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == FWD_TS && u < 64)     \
+            g_fwd_ts[wave][u][i] = clock64();                                                      \
+    } while (0)
+#else
+#define FTS(i)
+#endif
+
 template <int D> struct FwdLds {
     static constexpr int KST = D * 2 + 16;  // bytes per K / V row (== 16 mod 256 for D = 128)
     static constexpr int k_bytes = BK * KST;
@@ -241,6 +252,7 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
 #pragma unroll
             for (int dw = 0; dw < 2; ++dw) carry[f][dw] = pd[1][f][dw];
 
+        FTS(3);
         // V^T fragments of the first two head-dim blocks: in flight during the softmax
         bf16x8 vf[3];
         auto load_vf = [&](int buf, int db) {
@@ -319,6 +331,7 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
         // ---- O^T += V^T P^T: V^T fragments through the LDS transpose read, P^T straight from
         //      the softmax registers (k slot 8g+e <-> key 4g+e of output block 0 for e < 4, of
         //      output block 1 for e >= 4) ----
+        FTS(4);
         __builtin_amdgcn_s_setprio(1);
         bf16x8 pf[2];
 #pragma unroll
@@ -338,6 +351,7 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
             for (int ob = 0; ob < 2; ++ob) acc_o[ob][db] = mfma_bf16(vf[db % 3], pf[ob], acc_o[ob][db]);
             SCHED_MFMA(2);
         }
+        FTS(5);
     };
 
     const int k_end = causal ? min(p.Nk, i0 + BQ) : p.Nk;
@@ -353,9 +367,12 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
         constexpr int KIND = decltype(kind)::value;
 #pragma unroll 1
         for (int u = ua; u < ub; ++u) {
+            FTS(0);
             __syncthreads();  // step u-1 is done everywhere: its buffer is free, and step u's is written
+            FTS(1);
             stage_step(u + 1);
             load_step(u + 2);
+            FTS(2);
             if constexpr (KIND != 2) step(u, std::integral_constant<bool, KIND == 1>{});
         }
     };
@@ -429,6 +446,12 @@ hipError_t pick_cq(const Problem &p, const void *q, const void *k, const void *v
 }
 
 }  // namespace
+
+#ifdef FWD_TS
+extern "C" int convattn_debug_fwd_ts(long long *host) {
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_fwd_ts), sizeof(long long) * 4 * 64 * 8);
+}
+#endif
 
 hipError_t mfma_fwd(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
                     const float *w, void *o, float *m, float *l, hipStream_t s) {

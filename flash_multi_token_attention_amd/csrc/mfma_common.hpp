@@ -182,6 +182,27 @@ inline bool mfma_bwd_shape_ok(const Problem &p, int in_dt, unsigned flags) {
            ((long long)p.Nq + 16 + 127) / 128 <= kMaxGridZ && ((long long)p.Nk + 8 + 127) / 128 <= kMaxGridZ;
 }
 
+#if defined(__HIPCC__)
+// log2 of the dC scale of one (batch, head), taken from D = rowsum(dO o O) of its rows: D is linear
+// in dO and of the magnitude of dP, so the power of two s with s |D|max ~ 2^8 keeps the fp16 dC
+// tiles (dC = P (dP - D), times s) in fp16's normal range whatever the magnitude of dO is, which
+// makes the backward linear in dO.  Every kernel of a backward pass derives the same s from the
+// same D.  Called by all `nthreads` threads of a workgroup; `red` is LDS room for one float per
+// wave that nothing else uses until the call returns (two barriers inside).
+__device__ __forceinline__ float dc_scale_log2_from_d(const float *__restrict__ dl_b, int Nq, int tid, int nthreads,
+                                                      float *red) {
+    float mx = 0.f;
+    for (int i = tid; i < Nq; i += nthreads) mx = fmaxf(mx, fabsf(dl_b[i]));
+    mx = wave_max(mx);
+    if ((tid & 63) == 0) red[tid >> 6] = mx;
+    __syncthreads();
+    mx = 0.f;
+    for (int w2 = 0; w2 < nthreads / 64; ++w2) mx = fmaxf(mx, red[w2]);
+    __syncthreads();
+    return (mx > 0.f && mx < 3e38f) ? fminf(fmaxf(floorf(8.f - __log2f(mx)), -100.f), 100.f) : 0.f;
+}
+#endif
+
 // ---- bf16 MFMA kernels ----
 hipError_t mfma_fwd(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
                     const float *w, void *o, float *m, float *l, hipStream_t s);
@@ -217,8 +238,8 @@ inline size_t mfma_ds_bytes(const Problem &p) {
 hipError_t mfma_bwd_fused_ws(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
                              const void *d_o, const float *Dl, const float *lse, const float *w, void *dk,
                              void *dv, void *ds_ws, float *dw_part, hipStream_t s);
-hipError_t mfma_dq_from_ds(const Problem &p, int out_dt, const void *k, const void *ds_ws, void *dq,
-                           hipStream_t s);
+hipError_t mfma_dq_from_ds(const Problem &p, int out_dt, const void *k, const void *ds_ws, const float *Dl,
+                           void *dq, hipStream_t s);
 
 // ---- whole backward with the score chain in registers (bwd_chain_mfma.hip, bwd_dq_rows.hip) ----
 // Windows of up to 6 query taps.  The key-stationary kernel's workgroups cover 128 keys each (+ 8:

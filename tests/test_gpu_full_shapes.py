@@ -109,22 +109,26 @@ def test_autograd_function_partial_gradients(need):
 
 
 @pytest.mark.parametrize("factor", [2.0 ** -20, 2.0 ** -10, 2.0 ** 10])
-@pytest.mark.parametrize("one_pass", [True, False])
-def test_backward_is_linear_in_dO_over_many_orders_of_magnitude(factor, one_pass):
-    # dC is carried as fp16 times a power of two chosen from the magnitudes of dO and V: gradients of
-    # dO * factor are factor times the gradients of dO, to the same tolerance as at factor 1 (a mean
-    # loss over many tokens in bf16 training gives dO of 1e-6 and less)
-    Q, K, V, dO, W = rand_case(2, 2, 300, 300, 128, 6, 11, torch.bfloat16, seed=5)
+@pytest.mark.parametrize("mode", ["one_pass", "two_pass", "low_memory"])
+@pytest.mark.parametrize("c_q", [6, 11])
+def test_backward_is_linear_in_dO_over_many_orders_of_magnitude(factor, mode, c_q):
+    # dC is carried as fp16 times a power of two chosen from the magnitude of the upstream gradient:
+    # gradients of dO * factor are factor times the gradients of dO, to the same tolerance as at
+    # factor 1 (a mean loss over many tokens in bf16 training gives dO of 1e-6 and less).  Windows of
+    # up to 6 query taps run the key-stationary kernel, wider ones and the low-memory dQ pass the
+    # kernels with the score tiles in LDS.
+    Q, K, V, dO, W = rand_case(2, 2, 300, 300, 128, c_q, 11, torch.bfloat16, seed=5)
     ref = oracle_bwd(Q, K, V, W, dO, True)
     g = [t.to(DEV) for t in (Q, K, V, dO, W)]
-    sc, pq, pk = scale_of(128), 5, 5
+    sc, pq, pk = scale_of(128), c_q - 1, 5
     O, M, L = ops.forward(g[0], g[1], g[2], g[4], sc, pq, pk, True, out_dtype=torch.bfloat16)
     dOs = (g[3].float() * factor).to(torch.bfloat16)     # a power of two: exact in bf16
     D, LSE = ops.bwd_preprocess(O, dOs, M, L)
-    if one_pass:
+    if mode == "one_pass":
         dQ, dK, dV, dW = ops.backward(g[0], g[1], g[2], dOs, D, LSE, g[4], sc, pq, pk, True, out_dtype=torch.float32)
     else:
-        dQ, dW = ops.dq_backward(g[0], g[1], g[2], dOs, D, LSE, g[4], sc, pq, pk, True, out_dtype=torch.float32)
+        dQ, dW = ops.dq_backward(g[0], g[1], g[2], dOs, D, LSE, g[4], sc, pq, pk, True, out_dtype=torch.float32,
+                                 low_memory=(mode == "low_memory"))
         dK, dV = ops.dkdv_backward(g[0], g[1], g[2], dOs, D, LSE, g[4], sc, pq, pk, True, out_dtype=torch.float32)
     assert max_abs(dQ / factor, ref[0]) <= TOL_BF16
     assert max_abs(dK / factor, ref[1]) <= TOL_BF16
