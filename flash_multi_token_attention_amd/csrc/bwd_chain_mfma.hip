@@ -929,13 +929,8 @@ hipError_t launch_chain(const Problem &p, const void *q, const void *k, const vo
     auto kern = bwd_chain_kernel<D, CQT, TO, WANT>;
     constexpr int lds = ChainLds<D, CQT>::total;
     static_assert(lds <= 160 * 1024, "LDS budget");
-    static bool attr_set = false;  // per kernel instantiation; the attribute is sticky
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    hipError_t e = set_max_lds_once<bwd_chain_kernel<D, CQT, TO, WANT>>(lds);
+    if (e != hipSuccess) return e;
     dim3 grid(p.H, p.B, mfma_kv_tiles(p));
     ChainArgs args{p, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, (const bf16_t *)d_o, Dl, lse, w,
                    dc_scale, dk, dv, (bf16_t *)ds_ws, dw_part, chain_row_tiles(p)};

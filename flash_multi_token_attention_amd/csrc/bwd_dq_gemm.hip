@@ -155,8 +155,7 @@ template <int D, typename TO>
 hipError_t launch(const Problem &p, const void *k, const void *ds_ws, const float *Dl, void *dq, hipStream_t s) {
     auto kern = dq_from_ds_kernel<D, TO>;
     constexpr int lds = GemmLds<D>::total;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    hipError_t e = set_max_lds_once<dq_from_ds_kernel<D, TO>>(lds);
     if (e != hipSuccess) return e;
     dim3 grid(p.H, p.B, (p.Nq + kDsRowShift + BQ - 1) / BQ);
     kern<<<grid, NW * 64, lds, s>>>(p, (const bf16_t *)k, (const bf16_t *)ds_ws, Dl, mfma_ds_key_tiles(p),

@@ -433,8 +433,7 @@ hipError_t launch_dq(const Problem &p, const void *q, const void *k, const void 
                      hipStream_t s) {
     auto kern = bwd_dq_mfma_kernel<D, CQT, TO>;
     constexpr int lds = DqLds<D>::total;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    hipError_t e = set_max_lds_once<bwd_dq_mfma_kernel<D, CQT, TO>>(lds);
     if (e != hipSuccess) return e;
     dim3 grid(p.H, p.B, mfma_dq_tiles(p));
     kern<<<grid, NW * 64, lds, s>>>(p, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v,

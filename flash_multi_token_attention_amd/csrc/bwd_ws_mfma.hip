@@ -604,8 +604,7 @@ hipError_t launch_ws(const Problem &p, const void *q, const void *k, const void 
     auto kern = bwd_ws_mfma_kernel<D, CQT, TO>;
     constexpr int lds = WsLds<D>::total;
     static_assert(lds <= 160 * 1024, "LDS budget");
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    hipError_t e = set_max_lds_once<bwd_ws_mfma_kernel<D, CQT, TO>>(lds);
     if (e != hipSuccess) return e;
     dim3 grid(p.H, p.B, mfma_kv_tiles(p));
     kern<<<grid, NT, lds, s>>>(p, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v,

@@ -425,8 +425,7 @@ hipError_t launch_fwd(const Problem &p, const void *q, const void *k, const void
     auto kern = fwd_reg_mfma_kernel<D, CQT, TO>;
     constexpr int lds = FwdLds<D>::total;
     if (lds > 64 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        hipError_t e = set_max_lds_once<fwd_reg_mfma_kernel<D, CQT, TO>>(lds);
         if (e != hipSuccess) return e;
     }
     constexpr int BQ = NW * wave_rows(CQT);

@@ -13,6 +13,7 @@
 // pad_k <= 8.  Scores are staged in LDS as fp16 (11-bit significand; bf16's 8
 // bits would cost ~1e-2 in the softmax argument).
 #pragma once
+#include <atomic>
 #include <type_traits>
 
 #include "common.hpp"
@@ -202,6 +203,21 @@ __device__ __forceinline__ float dc_scale_log2_from_d(const float *__restrict__ 
     return (mx > 0.f && mx < 3e38f) ? fminf(fmaxf(floorf(8.f - __log2f(mx)), -100.f), 100.f) : 0.f;
 }
 #endif
+
+// Raises a kernel's dynamic LDS limit once per device (the attribute is sticky; setting it on every
+// launch costs a driver call).  One instance, and one flag word, per kernel instantiation.
+template <auto Kern>
+inline hipError_t set_max_lds_once(int bytes) {
+    static std::atomic<unsigned long long> done{0};   // one bit per device ordinal (mod 64)
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const unsigned long long bit = 1ull << (dev & 63);
+    if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(Kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess) done.fetch_or(bit, std::memory_order_release);
+    return e;
+}
 
 // ---- bf16 MFMA kernels ----
 hipError_t mfma_fwd(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
