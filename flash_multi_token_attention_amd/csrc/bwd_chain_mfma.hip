@@ -152,6 +152,21 @@ __device__ __forceinline__ f16x8 band_frag(int t, const float *__restrict__ w_he
     return f;
 }
 
+#ifndef CHAIN_PF
+#define CHAIN_PF 3
+#endif
+#ifndef CHAIN_PRIO_P
+#define CHAIN_PRIO_P 1
+#endif
+#ifndef CHAIN_PRIO_C
+#define CHAIN_PRIO_C 1
+#endif
+#ifndef CHAIN_PRIO_TC
+#define CHAIN_PRIO_TC 2
+#endif
+#ifndef CHAIN_PRIO_CEND
+#define CHAIN_PRIO_CEND 0
+#endif
 #ifndef CHAIN_ABLATE
 #define CHAIN_ABLATE 0
 #endif
@@ -438,7 +453,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                 // row fragments: lane n of fragment f reads row 2n + f, 16 bytes at column 32 ks + 8 g
                 const unsigned char *Qs = smem + opaque((unsigned int)(q_slot(it) - smem) + 2 * n * RST + g * 16);
                 const unsigned char *Gs = smem + opaque((unsigned int)(g_slot(it) - smem) + 2 * n * RST + g * 16);
-                __builtin_amdgcn_s_setprio(1);
+                __builtin_amdgcn_s_setprio(CHAIN_PRIO_P);
                 // ---- dP^T = V dO^T - D: depends on the staged tile only, so it goes first and its
                 // MFMAs run back to back with those of S^T ----
                 f32x4 dp[NCB][2];
@@ -608,17 +623,26 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
             if (WANT_KV && u_ok && !(CHAIN_ABLATE & 4)) {
                 const unsigned char *Ps = smem + opaque((unsigned int)(p_stage(u) - smem) + tr_lane_off(PST, g, n));
                 const unsigned char *Gs = smem + opaque((unsigned int)(g_slot(u) - smem) + tr_lane_off(RST, g, n));
-                __builtin_amdgcn_s_setprio(1);
+                __builtin_amdgcn_s_setprio(CHAIN_PRIO_C);
                 // ---- dV^T += dO^T P (keys c0-8 .. c0+23) ----
-                bf16x8 pf[2];
+                // the dO^T fragment of head-dim block db + PF is read while block db is multiplied: the
+                // MFMAs of PF blocks cover the LDS latency
+                constexpr int PF = CHAIN_PF;
+                bf16x8 pf[2], gq[PF + 1];
 #pragma unroll
                 for (int cb = 0; cb < 2; ++cb) pf[cb] = read_tr(Ps, PST, cb * 16);
 #pragma unroll
-                for (int db = 0; db < DB; ++db) {
-                    const bf16x8 gt = read_tr(Gs, RST, db * 16);
+                for (int db = 0; db < PF && db < DB; ++db) gq[db] = read_tr(Gs, RST, db * 16);
+                static_for<DB>([&](auto DBI) {
+                    constexpr int db = decltype(DBI)::value;
+                    if constexpr (db + PF < DB) {
+                        gq[(db + PF) % (PF + 1)] = read_tr(Gs, RST, (db + PF) * 16);
+                        SCHED_DS_READ_ID(2, 60 + db);
+                    }
 #pragma unroll
-                    for (int cb = 0; cb < 2; ++cb) acc_v[cb][db] = mfma_bf16(gt, pf[cb], acc_v[cb][db]);
-                }
+                    for (int cb = 0; cb < 2; ++cb) acc_v[cb][db] = mfma_bf16(gq[db % (PF + 1)], pf[cb], acc_v[cb][db]);
+                    SCHED_MFMA_ID(2, 60 + db);
+                });
             }
             CHAIN_SCHED_BARRIER;
             TS(3);
@@ -637,21 +661,28 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                         cur_dc[cb][f][1] = t2[1];
                     }
             }
+            TS(7);
             if (v_ok && !(CHAIN_ABLATE & 512)) {
                 const bool edge = is_edge(r0v);
                 bf16_t *ds_blk = ds_pair + (size_t)(r0v / BR) * (WK * BR);
-                __builtin_amdgcn_s_setprio(1);
+                __builtin_amdgcn_s_setprio(CHAIN_PRIO_TC);
                 // ---- dS^T of tile v: rows below it come from tile v+1.  Operand of row offset
                 // e = parity + (CQT-1 - tap slot): fragment e & 1 shifted e >> 1 lanes up. ----
                 f32x4 ds[NDB][2];
 #pragma unroll
                 for (int sb = 0; sb < NDB; ++sb) ds[sb][0] = ds[sb][1] = (f32x4){0.f, 0.f, 0.f, 0.f};
-                f16x8 tb_prev = (f16x8)(_Float16)0.f;
+                // flipped bands: the fragment of step e + 2 is read during step e (two steps of MFMAs
+                // cover the LDS latency; read one step ahead, every step waited for its band)
+                auto band_of = [&](int e) { return *reinterpret_cast<const f16x8 *>(bands + (CQT - 1 - e) * 1024); };
+                f16x8 tbq[4];   // bands of steps e-1 .. e+2
+                tbq[0] = band_of(0);
+                tbq[1] = band_of(CQT >= 2 ? 1 : 0);
+                tbq[2] = tbq[3] = tbq[0];
                 static_for<(CHAIN_ABLATE & 2) ? 0 : CQT + 1>([&](auto E) {
                     constexpr int e = decltype(E)::value, f = e & 1, s = e >> 1;
                     // tap slot CQT-1-e for parity 0 (this step's band), CQT-e for parity 1 (the last step's)
-                    f16x8 tb_cur = tb_prev;
-                    if constexpr (e <= CQT - 1) tb_cur = *reinterpret_cast<const f16x8 *>(bands + (CQT - 1 - e) * 1024);
+                    if constexpr (e + 2 <= CQT - 1) tbq[(e + 2) % 4] = band_of(e + 2);
+                    const f16x8 tb_cur = tbq[e % 4], tb_prev = tbq[(e + 3) % 4];
                     unsigned int sh[NCB][2];
 #pragma unroll
                     for (int cb = 0; cb < NCB; ++cb)
@@ -663,8 +694,8 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                         if constexpr (e <= CQT - 1) ds[sb][0] = mfma_f16(tb_cur, __builtin_bit_cast(f16x8, bv), ds[sb][0]);
                         if constexpr (e >= 1) ds[sb][1] = mfma_f16(tb_prev, __builtin_bit_cast(f16x8, bv), ds[sb][1]);
                     }
-                    tb_prev = tb_cur;
                 });
+                TS(8);
 #pragma unroll
                 for (int sb = 0; sb < NDB; ++sb)
 #pragma unroll
@@ -682,6 +713,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                         if constexpr (WANT_QW) *reinterpret_cast<bf16x4 *>(ds_blk + ((ob * 2 + sb) * 16 + n) * 16 + 4 * g) = sv;
                         if constexpr (WANT_KV) *reinterpret_cast<bf16x4 *>(ds_tile + (2 * n + ob) * PST + (sb * 16 + 4 * g) * 2) = sv;
                     }
+                TS(9);
             }
 #pragma unroll
             for (int cb = 0; cb < NCB; ++cb)
@@ -771,23 +803,31 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                 const unsigned char *Dsl = smem + opaque((unsigned int)(ds_tile - smem) + tr_lane_off(PST, g, n));
                 asm volatile("" ::: "memory");
                 __builtin_amdgcn_wave_barrier();
-                __builtin_amdgcn_s_setprio(1);
+                __builtin_amdgcn_s_setprio(CHAIN_PRIO_C);
                 // ---- dK^T += Q^T dS ----
                 {
-                    bf16x8 sf[2];
+                    constexpr int PF = CHAIN_PF;
+                    bf16x8 sf[2], qq[PF + 1];
+                    // (Q^T does not depend on the dS tile: its first fragments are on their way first)
+#pragma unroll
+                    for (int db = 0; db < PF && db < DB; ++db) qq[db] = read_tr(Qs, RST, db * 16);
 #pragma unroll
                     for (int sb = 0; sb < 2; ++sb) sf[sb] = read_tr(Dsl, PST, sb * 16);
+                    static_for<DB>([&](auto DBI) {
+                        constexpr int db = decltype(DBI)::value;
+                        if constexpr (db + PF < DB) {
+                            qq[(db + PF) % (PF + 1)] = read_tr(Qs, RST, (db + PF) * 16);
+                            SCHED_DS_READ_ID(2, 70 + db);
+                        }
 #pragma unroll
-                    for (int db = 0; db < DB; ++db) {
-                        const bf16x8 qt = read_tr(Qs, RST, db * 16);
-#pragma unroll
-                        for (int sb = 0; sb < 2; ++sb) acc_k[sb][db] = mfma_bf16(qt, sf[sb], acc_k[sb][db]);
-                    }
+                        for (int sb = 0; sb < 2; ++sb) acc_k[sb][db] = mfma_bf16(qq[db % (PF + 1)], sf[sb], acc_k[sb][db]);
+                        SCHED_MFMA_ID(2, 70 + db);
+                    });
                 }
                 asm volatile("" ::: "memory");
                 __builtin_amdgcn_wave_barrier();
             }
-            __builtin_amdgcn_s_setprio(0);
+            __builtin_amdgcn_s_setprio(CHAIN_PRIO_CEND);
             TS(6);
         }
 
