@@ -41,6 +41,9 @@ constexpr float kMaxSlack = 6.f;  // log2 units a score may exceed its row's exp
 // window's halo, the other 33-CQT are its output rows.
 constexpr int wave_rows(int cqt) { return 33 - cqt; }
 
+#ifndef FWD_PFV
+#define FWD_PFV 2   // V^T fragments read ahead of their MFMAs in the P V phase
+#endif
 #ifdef FWD_TS
 __device__ long long g_fwd_ts[4][64][8];
 #define FTS(i)                                                                                     \
@@ -253,15 +256,16 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
             for (int dw = 0; dw < 2; ++dw) carry[f][dw] = pd[1][f][dw];
 
         FTS(3);
-        // V^T fragments of the first two head-dim blocks: in flight during the softmax
-        bf16x8 vf[3];
+        // V^T fragments of the first FWD_PFV head-dim blocks: in flight during the softmax
+        constexpr int PFV = FWD_PFV < DB ? FWD_PFV : DB;
+        bf16x8 vf[PFV + 1];
         auto load_vf = [&](int buf, int db) {
             bf16x4 lo = lds_read_tr4x16(Vs, KST, 4 * g, db * 16, n);
             bf16x4 hi = lds_read_tr4x16(Vs, KST, 16 + 4 * g, db * 16, n);
             vf[buf] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
         };
-        load_vf(0, 0);
-        load_vf(1, 1);
+#pragma unroll
+        for (int db = 0; db < PFV; ++db) load_vf(db, db);
         // The two waves of a SIMD are at different places of their steps: the one in an MFMA
         // phase (P V, S^T, the convolution) gets the issue slot first, the one in the softmax
         // arithmetic fills the gaps (measured: 1.5 % over equal priorities; the reverse is slower).
@@ -343,12 +347,12 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
             }
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
-            if (db + 2 < DB) {
-                load_vf((db + 2) % 3, db + 2);
+            if (db + PFV < DB) {
+                load_vf((db + PFV) % (PFV + 1), db + PFV);
                 SCHED_DS_READ(2);
             }
 #pragma unroll
-            for (int ob = 0; ob < 2; ++ob) acc_o[ob][db] = mfma_bf16(vf[db % 3], pf[ob], acc_o[ob][db]);
+            for (int ob = 0; ob < 2; ++ob) acc_o[ob][db] = mfma_bf16(vf[db % (PFV + 1)], pf[ob], acc_o[ob][db]);
             SCHED_MFMA(2);
         }
         FTS(5);
