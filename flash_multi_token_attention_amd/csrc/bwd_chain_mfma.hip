@@ -454,31 +454,9 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                 const unsigned char *Qs = smem + opaque((unsigned int)(q_slot(it) - smem) + 2 * n * RST + g * 16);
                 const unsigned char *Gs = smem + opaque((unsigned int)(g_slot(it) - smem) + 2 * n * RST + g * 16);
                 __builtin_amdgcn_s_setprio(CHAIN_PRIO_P);
-                // ---- dP^T = V dO^T - D: depends on the staged tile only, so it goes first and its
-                // MFMAs run back to back with those of S^T ----
                 f32x4 dp[NCB][2];
                 float2 l2 = {0.f, 0.f};
-                if constexpr (FULL && !(CHAIN_ABLATE & 32)) {
-                    const float *st = stat_slot(it);
-                    l2 = *reinterpret_cast<const float2 *>(st + 2 * n);
-                    const float2 d2 = *reinterpret_cast<const float2 *>(st + BR + 2 * n);
-#pragma unroll
-                    for (int cb = 0; cb < NCB; ++cb) {
-                        dp[cb][0] = (f32x4){-d2.x, -d2.x, -d2.x, -d2.x};
-                        dp[cb][1] = (f32x4){-d2.y, -d2.y, -d2.y, -d2.y};
-                    }
-#pragma unroll
-                    for (int ks = 0; ks < KS; ++ks) {
-                        bf16x8 gf[2];
-#pragma unroll
-                        for (int f = 0; f < 2; ++f)
-                            gf[f] = *reinterpret_cast<const bf16x8 *>(Gs + f * RST + ks * 64);
-#pragma unroll
-                        for (int cb = 0; cb < NCB; ++cb)
-#pragma unroll
-                            for (int f = 0; f < 2; ++f) dp[cb][f] = mfma_bf16(vf[cb][ks], gf[f], dp[cb][f]);
-                    }
-                }
+                if constexpr (FULL) l2 = *reinterpret_cast<const float2 *>(stat_slot(it) + 2 * n);
                 TS(4);
                 // ---- S^T ----
                 unsigned int pd[NSB][2][2];
@@ -523,6 +501,27 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                     for (int kb = 0; kb < NSB; ++kb)
 #pragma unroll
                         for (int f = 0; f < 2; ++f) { prev_pd[kb][f][0] = pd[kb][f][0]; prev_pd[kb][f][1] = pd[kb][f][1]; }
+                    // ---- dP^T = V dO^T - D, after the convolution: the shifted score windows are no
+                    // longer live then (with dP first, some instances of the kernel needed scratch) ----
+                    if constexpr (!(CHAIN_ABLATE & 32)) {
+                        const float2 d2 = *reinterpret_cast<const float2 *>(stat_slot(it) + BR + 2 * n);
+#pragma unroll
+                        for (int cb = 0; cb < NCB; ++cb) {
+                            dp[cb][0] = (f32x4){-d2.x, -d2.x, -d2.x, -d2.x};
+                            dp[cb][1] = (f32x4){-d2.y, -d2.y, -d2.y, -d2.y};
+                        }
+#pragma unroll
+                        for (int ks = 0; ks < KS; ++ks) {
+                            bf16x8 gf[2];
+#pragma unroll
+                            for (int f = 0; f < 2; ++f)
+                                gf[f] = *reinterpret_cast<const bf16x8 *>(Gs + f * RST + ks * 64);
+#pragma unroll
+                            for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+                                for (int f = 0; f < 2; ++f) dp[cb][f] = mfma_bf16(vf[cb][ks], gf[f], dp[cb][f]);
+                        }
+                    }
                     CHAIN_SCHED_BARRIER;
                     TS(5);
                     // ---- P = exp2(C - LSE) (times the dC scale), dC = P dP ----
