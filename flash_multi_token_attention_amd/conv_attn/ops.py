@@ -321,7 +321,10 @@ def _decode_kv(Q, K, V, layout: "_lib.KvLayout", Nk: int, conv_kernel, k_splits,
     c_q, c_k = conv_kernel.shape[1], conv_kernel.shape[2]
     W = _weights(conv_kernel, H, c_q - 1, (c_k - 1) // 2, Q.device)
     if not k_splits:
-        k_splits = default_k_splits(B, H, Nk)
+        # a workgroup takes 4 or 2 query heads of one KV head when the window has at most 8 query taps
+        group = H // max(1, layout.H_kv or H)
+        heads_per_wg = 1 if c_q > 8 else 4 if group % 4 == 0 else 2 if group % 2 == 0 else 1
+        k_splits = default_k_splits(B, H // heads_per_wg, Nk)
     if out_dtype not in _DT:
         raise RuntimeError("out_dtype must be bfloat16 or float32")
     desc = _lib.Desc(B, H, r, Nk, d, c_q, c_k, float(scale), int(bool(causal)), _DT[Q.dtype], _DT[out_dtype],

@@ -24,7 +24,10 @@
 // (head h reads KV head h / group), the rows of a (batch, KV head) may be contiguous or come in
 // pages named by a block table (PAGED instance: one table lookup per row load; the lookups of the
 // rows a lane loads next are independent of everything else in the iteration), and every batch
-// entry may have its own number of keys.
+// entry may have its own number of keys.  With shared KV heads a workgroup takes HG = 2 or 4 query
+// heads of one KV head (windows of up to 8 query taps): two heads' tap rows fill one 16-row MFMA
+// (rows 0..7 and 8..15), so the K / V stream of the KV head is read once for all of them, and only
+// the window, the softmax and P.V are repeated per head.
 #include "mfma_common.hpp"
 
 namespace convattn {
@@ -41,7 +44,7 @@ constexpr int SROW = SW + 4;       // floats per strip row (84)
 __device__ __forceinline__ float bf16_lo(unsigned int w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float bf16_hi(unsigned int w) { return __uint_as_float(w & 0xffff0000u); }
 
-template <int D, bool PAGED>
+template <int D, bool PAGED, int HG>
 __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(
     Problem p, KvArgs kv, const bf16_t *__restrict__ Q, const bf16_t *__restrict__ K,
     const bf16_t *__restrict__ V, const float *__restrict__ W, float *__restrict__ O_part,
@@ -50,20 +53,24 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(
     constexpr int CPR = D / 8;       // 16-byte chunks per K/V row
     constexpr int RPI = 64 / CPR;    // V rows one load instruction of the wave covers
     constexpr int VT = IT / RPI;     // V loads per lane per iteration
-    __shared__ __attribute__((aligned(16))) float s_strip[NW][16 * SROW];
-    __shared__ __attribute__((aligned(16))) float s_p[NW][IT];
-    __shared__ float s_w[kMaxCq * 17];
-    __shared__ __attribute__((aligned(16))) float s_o[NW][D];
-    __shared__ float s_ml[NW][2];
+    constexpr int MG = (HG + 1) / 2;   // 16-row MFMA groups: one head (HG = 1) or two heads each
+    __shared__ __attribute__((aligned(16))) float s_strip[NW][MG][16 * SROW];
+    __shared__ __attribute__((aligned(16))) float s_p[NW][HG][IT];
+    // window weights, one row of 20 floats per tap row: key tap b sits at column 8 - pk + b of the
+    // 17 columns around a key (zeros elsewhere), so that the window loop has a fixed trip count
+    __shared__ __attribute__((aligned(16))) float s_w[HG][kMaxCq][20];
+    __shared__ __attribute__((aligned(16))) float s_o[NW][HG][D];
+    __shared__ float s_ml[NW][HG][2];
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     const int g = lane >> 4, n = lane & 15;
-    const int sp = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int sp = blockIdx.x, h = blockIdx.y * HG, b = blockIdx.z;   // h: first query head of the workgroup
     const int cq = p.c_q, ck = p.c_k, pk = p.pk;
     const size_t bh = (size_t)b * p.H + h;
-    const bf16_t *Qb = Q + bh * p.Nq * D;
     const int hk = h / kv.group;
+    // MFMA row n of a group: tap row_tap of head 2 m + row_head of the workgroup
+    const int row_head = HG == 1 ? 0 : (n >> 3), row_tap = HG == 1 ? n : (n & 7);
     const int Nk = kv.seq_lens ? min(max(kv.seq_lens[b], 0), p.Nk) : p.Nk;   // keys of this batch entry
     const bf16_t *Kb = K + (PAGED ? 0 : b * p.kv_bstride) + hk * p.kv_hstride;
     const bf16_t *Vb = V + (PAGED ? 0 : b * p.kv_bstride) + hk * p.kv_hstride;
@@ -78,24 +85,27 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(
             src = base + (size_t)rr * D;
         return __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + col));
     };
-    float *strip = s_strip[wave];
-
-    for (int i = tid; i < cq * ck; i += NW * 64) s_w[i] = W[(size_t)h * cq * ck + i];
+    for (int i = tid; i < HG * kMaxCq * 20; i += NW * 64) {
+        const int hh = i / (kMaxCq * 20), a = i / 20 % kMaxCq, bb = i % 20 - (8 - pk);
+        s_w[hh][a][i % 20] = (a < cq && bb >= 0 && bb < ck) ? W[((size_t)(h + hh) * cq + a) * ck + bb] : 0.f;
+    }
 
     // Tap row a reads resident row Nq - c_q + a (zero row if it does not exist).
-    bf16x8 qf[KS];
-    {
-        const int ri = p.Nq - cq + n;
-        const bool ok = n < cq && ri >= 0;
+    bf16x8 qf[MG][KS];
+#pragma unroll
+    for (int m = 0; m < MG; ++m) {
+        const int ri = p.Nq - cq + row_tap, hh = 2 * m + row_head;
+        const bool ok = row_tap < cq && ri >= 0 && hh < HG;
+        const bf16_t *Qb = Q + (bh + hh) * p.Nq * D;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             u32x4 raw = {0u, 0u, 0u, 0u};
             if (ok) raw = *reinterpret_cast<const u32x4 *>(Qb + (size_t)ri * D + ks * 32 + g * 8);
-            qf[ks] = __builtin_bit_cast(bf16x8, raw);
+            qf[m][ks] = __builtin_bit_cast(bf16x8, raw);
         }
     }
     // Causal variant: tap row a sits at position Nk - c_q + a and sees no later key.
-    const int row_pos = p.causal ? Nk - cq + n : 0x7fffffff;
+    const int row_pos = p.causal ? Nk - cq + row_tap : 0x7fffffff;
 
     // Key range of this wave: the split's chunk cut into 4 runs of whole iterations.
     const int chunk = (Nk + p.n_splits - 1) / p.n_splits;
@@ -104,32 +114,42 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(
     const int lo = s_lo + wave * per_wave, hi = min(s_hi, lo + per_wave);
 
     const int cc = lane % CPR, gph = lane / CPR;  // this lane's V column chunk and key phase
-    float acc[8];
+    float acc[HG][8], m_run[HG], l_run[HG];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-    float m_run = kNegInf, l_run = 0.f;
+    for (int hh = 0; hh < HG; ++hh) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[hh][e] = 0.f;
+        m_run[hh] = kNegInf;
+        l_run[hh] = 0.f;
+    }
     const float scale = p.scale;
     __syncthreads();  // s_w
 
     if (lo < hi) {
         // strip columns 0..15 <- scores of keys lo-8 .. lo+7
         {
-            f32x4 a4 = {0.f, 0.f, 0.f, 0.f};
+            f32x4 a4[MG];
+#pragma unroll
+            for (int m = 0; m < MG; ++m) a4[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 // (keys before the first or after the last one score zero: the window's padding)
                 const int row = lo - 8 + n;
                 u32x4 raw = load_row(Kb, row, ks * 32 + g * 8);
                 if (row < 0 || row >= Nk) raw = (u32x4){0u, 0u, 0u, 0u};
-                a4 = mfma_bf16(__builtin_bit_cast(bf16x8, raw), qf[ks], a4);
-            }
-            if (n < cq) {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int key = lo - 8 + 4 * g + r;
-                    a4[r] = (key > row_pos) ? 0.f : a4[r] * scale;
+                for (int m = 0; m < MG; ++m) a4[m] = mfma_bf16(__builtin_bit_cast(bf16x8, raw), qf[m][ks], a4[m]);
+            }
+            if (row_tap < cq) {
+#pragma unroll
+                for (int m = 0; m < MG; ++m) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int key = lo - 8 + 4 * g + r;
+                        a4[m][r] = (key > row_pos) ? 0.f : a4[m][r] * scale;
+                    }
+                    *reinterpret_cast<f32x4 *>(s_strip[wave][m] + n * SROW + 4 * g) = a4[m];
                 }
-                *reinterpret_cast<f32x4 *>(strip + n * SROW + 4 * g) = a4;
             }
         }
         // K of the first iteration: keys lo+8 .. lo+71
@@ -149,22 +169,25 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(
             // scores of keys j0+8 .. j0+71 -> strip columns 16 .. 79
 #pragma unroll
             for (int blk = 0; blk < 4; ++blk) {
-                f32x4 a4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks)
-                    a4 = mfma_bf16(__builtin_bit_cast(bf16x8, kreg[blk][ks]), qf[ks], a4);
-                if (n < cq) {
+                for (int m = 0; m < MG; ++m) {
+                    f32x4 a4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const int key = j0 + 8 + blk * 16 + 4 * g + r;
-                        a4[r] = (key > row_pos) ? 0.f : a4[r] * scale;
+                    for (int ks = 0; ks < KS; ++ks)
+                        a4 = mfma_bf16(__builtin_bit_cast(bf16x8, kreg[blk][ks]), qf[m][ks], a4);
+                    if (row_tap < cq) {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            const int key = j0 + 8 + blk * 16 + 4 * g + r;
+                            a4[r] = (key > row_pos) ? 0.f : a4[r] * scale;
+                        }
+                        if (j0 + IT + 8 > Nk) {  // keys past the end of the cache score zero (K rows were clamped)
+#pragma unroll
+                            for (int r = 0; r < 4; ++r)
+                                if (j0 + 8 + blk * 16 + 4 * g + r >= Nk) a4[r] = 0.f;
+                        }
+                        *reinterpret_cast<f32x4 *>(s_strip[wave][m] + n * SROW + 16 + blk * 16 + 4 * g) = a4;
                     }
-                    if (j0 + IT + 8 > Nk) {  // keys past the end of the cache score zero (K rows were clamped)
-#pragma unroll
-                        for (int r = 0; r < 4; ++r)
-                            if (j0 + 8 + blk * 16 + 4 * g + r >= Nk) a4[r] = 0.f;
-                    }
-                    *reinterpret_cast<f32x4 *>(strip + n * SROW + 16 + blk * 16 + 4 * g) = a4;
                 }
             }
             // K of the next iteration (zeros past the cache end)
@@ -178,80 +201,113 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(
             __builtin_amdgcn_wave_barrier();
 
             // window: lane j -> key j0 + j; strip column of key x is x - (j0 - 8)
-            float c = 0.f;
-            {
-                const float *srow = strip + lane + 8 - pk;
-                for (int a = 0; a < cq; ++a) {
-                    const float *wr = s_w + a * ck;
-                    for (int bb = 0; bb < ck; ++bb) c = fmaf(wr[bb], srow[bb], c);
-                    srow += SROW;
+            float alpha[HG];
+#pragma unroll
+            for (int hh = 0; hh < HG; ++hh) {
+                // (17 columns around the key whatever c_k is: the reads of a tap row are independent
+                // of each other and issued together; with run-time bounds every tap waited for its own)
+                float c = 0.f;
+                {
+                    const float *srow = s_strip[wave][hh >> 1] + (HG == 1 ? 0 : 8 * (hh & 1)) * SROW + lane;
+                    for (int a = 0; a < cq; ++a) {
+                        float wv[20], sv[17];
+#pragma unroll
+                        for (int q4 = 0; q4 < 5; ++q4)
+                            *reinterpret_cast<f32x4 *>(wv + 4 * q4) = *reinterpret_cast<const f32x4 *>(&s_w[hh][a][4 * q4]);
+#pragma unroll
+                        for (int bb = 0; bb < 17; ++bb) sv[bb] = srow[bb];
+                        float c0 = 0.f, c1 = 0.f;
+#pragma unroll
+                        for (int bb = 0; bb < 16; bb += 2) { c0 = fmaf(wv[bb], sv[bb], c0); c1 = fmaf(wv[bb + 1], sv[bb + 1], c1); }
+                        c += c0 + fmaf(wv[16], sv[16], c1);
+                        srow += SROW;
+                    }
                 }
+                if (j0 + lane >= hi) c = kNegInf;
+                const float m_new = fmaxf(m_run[hh], wave_max(c));
+                const float e = (c == kNegInf) ? 0.f : __expf(c - m_new);
+                alpha[hh] = (m_run[hh] == kNegInf) ? 0.f : __expf(m_run[hh] - m_new);
+                m_run[hh] = m_new;
+                l_run[hh] = l_run[hh] * alpha[hh] + e;
+                // hand p to the lanes that own each key's V row: phase-major order
+                s_p[wave][hh][(lane % RPI) * VT + lane / RPI] = e;
             }
-            if (j0 + lane >= hi) c = kNegInf;
-            const float m_new = fmaxf(m_run, wave_max(c));
-            const float e = (c == kNegInf) ? 0.f : __expf(c - m_new);
-            const float alpha = (m_run == kNegInf) ? 0.f : __expf(m_run - m_new);
-            m_run = m_new;
-            l_run = l_run * alpha + e;
-            // hand p to the lanes that own each key's V row: phase-major order
-            s_p[wave][(lane % RPI) * VT + lane / RPI] = e;
             __builtin_amdgcn_wave_barrier();
             // carry the last 16 score columns to the front for the next iteration
             if (lane < 16) {
-                for (int a = 0; a < cq; ++a) strip[a * SROW + lane] = strip[a * SROW + IT + lane];
+#pragma unroll
+                for (int m = 0; m < MG; ++m) {
+                    float cv[16];
+#pragma unroll
+                    for (int a = 0; a < 16; ++a) cv[a] = s_strip[wave][m][a * SROW + IT + lane];
+#pragma unroll
+                    for (int a = 0; a < 16; ++a) s_strip[wave][m][a * SROW + lane] = cv[a];
+                }
             }
-            float pv[VT];
 #pragma unroll
-            for (int t = 0; t < VT; t += 4) {
-                f32x4 p4 = *reinterpret_cast<const f32x4 *>(&s_p[wave][gph * VT + t]);
-                pv[t] = p4[0]; pv[t + 1] = p4[1]; pv[t + 2] = p4[2]; pv[t + 3] = p4[3];
-            }
+            for (int hh = 0; hh < HG; ++hh) {
+                float pv[VT];
 #pragma unroll
-            for (int e8 = 0; e8 < 8; ++e8) acc[e8] *= alpha;
+                for (int t = 0; t < VT; t += 4) {
+                    f32x4 p4 = *reinterpret_cast<const f32x4 *>(&s_p[wave][hh][gph * VT + t]);
+                    pv[t] = p4[0]; pv[t + 1] = p4[1]; pv[t + 2] = p4[2]; pv[t + 3] = p4[3];
+                }
 #pragma unroll
-            for (int t = 0; t < VT; ++t) {
+                for (int e8 = 0; e8 < 8; ++e8) acc[hh][e8] *= alpha[hh];
 #pragma unroll
-                for (int w2 = 0; w2 < 4; ++w2) {
-                    acc[2 * w2] = fmaf(pv[t], bf16_lo(vreg[t][w2]), acc[2 * w2]);
-                    acc[2 * w2 + 1] = fmaf(pv[t], bf16_hi(vreg[t][w2]), acc[2 * w2 + 1]);
+                for (int t = 0; t < VT; ++t) {
+#pragma unroll
+                    for (int w2 = 0; w2 < 4; ++w2) {
+                        acc[hh][2 * w2] = fmaf(pv[t], bf16_lo(vreg[t][w2]), acc[hh][2 * w2]);
+                        acc[hh][2 * w2 + 1] = fmaf(pv[t], bf16_hi(vreg[t][w2]), acc[hh][2 * w2 + 1]);
+                    }
                 }
             }
             __builtin_amdgcn_wave_barrier();
         }
         // sum the key phases (lanes with the same column chunk) and the row sums
 #pragma unroll
-        for (int o = CPR; o < 64; o <<= 1) {
+        for (int hh = 0; hh < HG; ++hh) {
 #pragma unroll
-            for (int e8 = 0; e8 < 8; ++e8) acc[e8] += __shfl_xor(acc[e8], o, kWave);
+            for (int o = CPR; o < 64; o <<= 1) {
+#pragma unroll
+                for (int e8 = 0; e8 < 8; ++e8) acc[hh][e8] += __shfl_xor(acc[hh][e8], o, kWave);
+            }
+            l_run[hh] = wave_sum(l_run[hh]);
         }
-        l_run = wave_sum(l_run);
     }
 
     // merge the 4 waves: o = sum o_w e^{m_w - m}, l = sum l_w e^{m_w - m}
-    if (lane < CPR) {
 #pragma unroll
-        for (int e8 = 0; e8 < 8; ++e8) s_o[wave][lane * 8 + e8] = acc[e8];
+    for (int hh = 0; hh < HG; ++hh) {
+        if (lane < CPR) {
+#pragma unroll
+            for (int e8 = 0; e8 < 8; ++e8) s_o[wave][hh][lane * 8 + e8] = acc[hh][e8];
+        }
+        if (lane == 0) { s_ml[wave][hh][0] = m_run[hh]; s_ml[wave][hh][1] = l_run[hh]; }
     }
-    if (lane == 0) { s_ml[wave][0] = m_run; s_ml[wave][1] = l_run; }
     __syncthreads();
-    float m = kNegInf;
 #pragma unroll
-    for (int w = 0; w < NW; ++w) m = fmaxf(m, s_ml[w][0]);
-    const size_t slot = bh * p.n_splits + sp;
-    if (tid < D) {
-        float o = 0.f;
+    for (int hh = 0; hh < HG; ++hh) {
+        float m = kNegInf;
 #pragma unroll
-        for (int w = 0; w < NW; ++w)
-            if (s_ml[w][0] != kNegInf) o = fmaf(s_o[w][tid], __expf(s_ml[w][0] - m), o);
-        O_part[slot * D + tid] = o;
-    }
-    if (tid == 0) {
-        float l = 0.f;
+        for (int w = 0; w < NW; ++w) m = fmaxf(m, s_ml[w][hh][0]);
+        const size_t slot = (bh + hh) * p.n_splits + sp;
+        if (tid < D) {
+            float o = 0.f;
 #pragma unroll
-        for (int w = 0; w < NW; ++w)
-            if (s_ml[w][0] != kNegInf) l = fmaf(s_ml[w][1], __expf(s_ml[w][0] - m), l);
-        M_part[slot] = m;
-        L_part[slot] = l;
+            for (int w = 0; w < NW; ++w)
+                if (s_ml[w][hh][0] != kNegInf) o = fmaf(s_o[w][hh][tid], __expf(s_ml[w][hh][0] - m), o);
+            O_part[slot * D + tid] = o;
+        }
+        if (tid == 0) {
+            float l = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w)
+                if (s_ml[w][hh][0] != kNegInf) l = fmaf(s_ml[w][hh][1], __expf(s_ml[w][hh][0] - m), l);
+            M_part[slot] = m;
+            L_part[slot] = l;
+        }
     }
 }
 
@@ -262,19 +318,34 @@ bool decode_stream_ok(const Problem &p, int in_dt, unsigned flags) {
            p.pk <= 8 && p.c_q <= 16;
 }
 
+// Query heads a workgroup takes together: 4 or 2 heads of one KV head when the window's query taps
+// fit half an MFMA (8 rows), else 1.
+int decode_heads_per_wg(const Problem &p, int group) {
+    if (p.c_q > 8) return 1;
+    return group % 4 == 0 ? 4 : group % 2 == 0 ? 2 : 1;
+}
+
 hipError_t decode_stream_kv(const Problem &p, const KvArgs &kv, const void *q, const void *k, const void *v,
                             const float *w, float *o_part, float *m_part, float *l_part, hipStream_t s) {
-    dim3 grid(p.n_splits, p.H, p.B);
-#define CONVATTN_DECODE_LAUNCH(DD, PG)                                                                       \
-    decode_stream_kernel<DD, PG><<<grid, NW * 64, 0, s>>>(p, kv, (const bf16_t *)q, (const bf16_t *)k,         \
-                                                         (const bf16_t *)v, w, o_part, m_part, l_part)
+    const int hg = decode_heads_per_wg(p, kv.group);
+    dim3 grid(p.n_splits, p.H / hg, p.B);
+#define CONVATTN_DECODE_LAUNCH(DD, PG, HH)                                                                   \
+    decode_stream_kernel<DD, PG, HH><<<grid, NW * 64, 0, s>>>(p, kv, (const bf16_t *)q, (const bf16_t *)k,     \
+                                                             (const bf16_t *)v, w, o_part, m_part, l_part)
+#define CONVATTN_DECODE_PICK_HG(DD, PG)                                                                      \
+    do {                                                                                                     \
+        if (hg == 4) CONVATTN_DECODE_LAUNCH(DD, PG, 4);                                                       \
+        else if (hg == 2) CONVATTN_DECODE_LAUNCH(DD, PG, 2);                                                  \
+        else CONVATTN_DECODE_LAUNCH(DD, PG, 1);                                                               \
+    } while (0)
     if (p.d == 128) {
-        if (kv.table) CONVATTN_DECODE_LAUNCH(128, true);
-        else CONVATTN_DECODE_LAUNCH(128, false);
+        if (kv.table) CONVATTN_DECODE_PICK_HG(128, true);
+        else CONVATTN_DECODE_PICK_HG(128, false);
     } else {
-        if (kv.table) CONVATTN_DECODE_LAUNCH(64, true);
-        else CONVATTN_DECODE_LAUNCH(64, false);
+        if (kv.table) CONVATTN_DECODE_PICK_HG(64, true);
+        else CONVATTN_DECODE_PICK_HG(64, false);
     }
+#undef CONVATTN_DECODE_PICK_HG
 #undef CONVATTN_DECODE_LAUNCH
     return hipGetLastError();
 }

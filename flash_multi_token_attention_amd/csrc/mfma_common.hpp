@@ -304,6 +304,7 @@ struct KvArgs {
     int page_shift;         // log2 of the keys per page
     int group;              // query heads per KV head (>= 1)
 };
+int decode_heads_per_wg(const Problem &p, int group);
 hipError_t decode_stream_kv(const Problem &p, const KvArgs &kv, const void *q, const void *k, const void *v,
                             const float *w, float *o_part, float *m_part, float *l_part, hipStream_t s);
 hipError_t decode_stream(const Problem &p, const void *q, const void *k, const void *v, const float *w,

@@ -27,11 +27,13 @@ def _check(out, ref):
     assert max_abs(M + torch.log(L), ref[1] + torch.log(ref[2])) <= 2e-2
 
 
-@pytest.mark.parametrize("H,H_kv", [(8, 8), (8, 2), (6, 1)])
+@pytest.mark.parametrize("H,H_kv,c_q", [(8, 8, 6), (8, 2, 6), (6, 1, 6), (8, 1, 8), (4, 2, 3), (8, 2, 11), (16, 2, 1)])
 @pytest.mark.parametrize("causal", [False, True])
-def test_gqa_dense_and_cache_view(H, H_kv, causal):
-    B, Nk, d, c_q, c_k = 2, 700, 128, 6, 11
-    Q, K, V, W = _case(B, H, H_kv, Nk, d, c_q, c_k, seed=H * 10 + H_kv)
+def test_gqa_dense_and_cache_view(H, H_kv, c_q, causal):
+    # (groups of 4 and 2 query heads share one K / V stream when the window has at most 8 query taps;
+    # 11 taps and odd groups run one head per workgroup)
+    B, Nk, d, c_k = 2, 700, 128, 11
+    Q, K, V, W = _case(B, H, H_kv, Nk, d, c_q, c_k, seed=H * 10 + H_kv + c_q)
     sc = scale_of(d)
     ref = orc.decode_kv(Q.float(), lambda b: K[b].float(), lambda b: V[b].float(), W, [Nk] * B, sc, causal)
     g = [t.to(DEV) for t in (Q, K, V, W)]
