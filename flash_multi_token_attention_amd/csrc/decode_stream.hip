@@ -22,8 +22,9 @@
 //
 // Where the rows live is a parameter of the kernel (KvArgs): query heads may share KV heads
 // (head h reads KV head h / group), the rows of a (batch, KV head) may be contiguous or come in
-// pages named by a block table (PAGED instance: one table lookup per row load; the lookups of the
-// rows a lane loads next are independent of everything else in the iteration), and every batch
+// pages named by a block table (PAGED instance: the page numbers of the 80 rows around a 64-key
+// iteration are fetched by scalar loads one iteration ahead and handed to the lanes through LDS,
+// so the lookups do not sit in the vector-load queue between the K / V loads), and every batch
 // entry may have its own number of keys.  With shared KV heads a workgroup takes HG = 2 or 4 query
 // heads of one KV head (windows of up to 8 query taps): two heads' tap rows fill one 16-row MFMA
 // (rows 0..7 and 8..15), so the K / V stream of the KV head is read once for all of them, and only
@@ -61,9 +62,10 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(
     __shared__ __attribute__((aligned(16))) float s_w[HG][kMaxCq][20];
     __shared__ __attribute__((aligned(16))) float s_o[NW][HG][D];
     __shared__ float s_ml[NW][HG][2];
+    __shared__ int s_pid[NW][2][8];   // PAGED: page numbers of the row windows of two iterations
 
     const int tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int g = lane >> 4, n = lane & 15;
     const int sp = blockIdx.x, h = blockIdx.y * HG, b = blockIdx.z;   // h: first query head of the workgroup
     const int cq = p.c_q, ck = p.c_k, pk = p.pk;
@@ -74,15 +76,41 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(
     const int Nk = kv.seq_lens ? min(max(kv.seq_lens[b], 0), p.Nk) : p.Nk;   // keys of this batch entry
     const bf16_t *Kb = K + (PAGED ? 0 : b * p.kv_bstride) + hk * p.kv_hstride;
     const bf16_t *Vb = V + (PAGED ? 0 : b * p.kv_bstride) + hk * p.kv_hstride;
-    const int *tbl = PAGED ? kv.table + (size_t)b * kv.table_stride : nullptr;
+    // PAGED: the window of a 64-key iteration starting at key w0 (a multiple of 64) is rows
+    // w0-8 .. w0+71: at most 6 pages of 16 or more keys.  fetch_pages(w0) reads their numbers with
+    // scalar loads (the table is read-only: constant address space) and leaves them in the wave's
+    // slot (w0 / 64) & 1; load_row(w0, ...) looks a row's page up there.
+#if defined(__HIP_DEVICE_COMPILE__)
+    typedef const __attribute__((address_space(4))) int *tbl_ptr_t;
+#else
+    typedef const int *tbl_ptr_t;
+#endif
+    tbl_ptr_t tbl = PAGED ? (tbl_ptr_t)(kv.table + (size_t)b * kv.table_stride) : (tbl_ptr_t) nullptr;
+    auto fetch_pages = [&](int w0) {
+        if constexpr (PAGED) {
+            const int first = max(w0 - 8, 0) >> kv.page_shift, last = (Nk - 1) >> kv.page_shift;
+            int mine = 0;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int id = tbl[min(first + i, last)];
+                mine = lane == i ? id : mine;
+            }
+            if (lane < 8) s_pid[wave][(w0 >> 6) & 1][lane] = mine;
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_wave_barrier();
+        }
+    };
     // 8 bf16 at column `col` of the row nearest to `row` inside [0, Nk)
-    auto load_row = [&](const bf16_t *base, int row, int col) -> u32x4 {
+    auto load_row = [&](int w0, const bf16_t *base, int row, int col) -> u32x4 {
         const int rr = min(max(row, 0), Nk - 1);
         const bf16_t *src;
-        if constexpr (PAGED)
-            src = base + (size_t)tbl[rr >> kv.page_shift] * kv.page_stride + (size_t)(rr & ((1 << kv.page_shift) - 1)) * D;
-        else
+        if constexpr (PAGED) {
+            const int first = max(w0 - 8, 0) >> kv.page_shift;
+            const int page = s_pid[wave][(w0 >> 6) & 1][(rr >> kv.page_shift) - first];
+            src = base + (size_t)page * kv.page_stride + (size_t)(rr & ((1 << kv.page_shift) - 1)) * D;
+        } else {
             src = base + (size_t)rr * D;
+        }
         return __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + col));
     };
     for (int i = tid; i < HG * kMaxCq * 20; i += NW * 64) {
@@ -108,7 +136,8 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(
     const int row_pos = p.causal ? Nk - cq + row_tap : 0x7fffffff;
 
     // Key range of this wave: the split's chunk cut into 4 runs of whole iterations.
-    const int chunk = (Nk + p.n_splits - 1) / p.n_splits;
+    // (PAGED: splits start at multiples of 64 keys, so that an iteration's rows are a fixed window)
+    const int chunk = PAGED ? ((Nk + p.n_splits - 1) / p.n_splits + IT - 1) / IT * IT : (Nk + p.n_splits - 1) / p.n_splits;
     const int s_lo = sp * chunk, s_hi = min(Nk, s_lo + chunk);
     const int per_wave = ((chunk + NW - 1) / NW + IT - 1) / IT * IT;
     const int lo = s_lo + wave * per_wave, hi = min(s_hi, lo + per_wave);
@@ -126,6 +155,7 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(
     __syncthreads();  // s_w
 
     if (lo < hi) {
+        fetch_pages(lo);
         // strip columns 0..15 <- scores of keys lo-8 .. lo+7
         {
             f32x4 a4[MG];
@@ -135,7 +165,7 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(
             for (int ks = 0; ks < KS; ++ks) {
                 // (keys before the first or after the last one score zero: the window's padding)
                 const int row = lo - 8 + n;
-                u32x4 raw = load_row(Kb, row, ks * 32 + g * 8);
+                u32x4 raw = load_row(lo, Kb, row, ks * 32 + g * 8);
                 if (row < 0 || row >= Nk) raw = (u32x4){0u, 0u, 0u, 0u};
 #pragma unroll
                 for (int m = 0; m < MG; ++m) a4[m] = mfma_bf16(__builtin_bit_cast(bf16x8, raw), qf[m][ks], a4[m]);
@@ -158,13 +188,14 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(
         for (int blk = 0; blk < 4; ++blk)
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks)
-                kreg[blk][ks] = load_row(Kb, lo + 8 + blk * 16 + n, ks * 32 + g * 8);
+                kreg[blk][ks] = load_row(lo, Kb, lo + 8 + blk * 16 + n, ks * 32 + g * 8);
 
         for (int j0 = lo; j0 < hi; j0 += IT) {
             // V of this iteration: keys j0 .. j0+63
             u32x4 vreg[VT];
 #pragma unroll
-            for (int t = 0; t < VT; ++t) vreg[t] = load_row(Vb, j0 + RPI * t + gph, cc * 8);
+            for (int t = 0; t < VT; ++t) vreg[t] = load_row(j0, Vb, j0 + RPI * t + gph, cc * 8);
+            if (j0 + IT < hi) fetch_pages(j0 + IT);   // for the K loads below and the next iteration's V loads
 
             // scores of keys j0+8 .. j0+71 -> strip columns 16 .. 79
 #pragma unroll
@@ -196,7 +227,7 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(
                 for (int blk = 0; blk < 4; ++blk)
 #pragma unroll
                     for (int ks = 0; ks < KS; ++ks)
-                        kreg[blk][ks] = load_row(Kb, j0 + IT + 8 + blk * 16 + n, ks * 32 + g * 8);
+                        kreg[blk][ks] = load_row(j0 + IT, Kb, j0 + IT + 8 + blk * 16 + n, ks * 32 + g * 8);
             }
             __builtin_amdgcn_wave_barrier();
 
