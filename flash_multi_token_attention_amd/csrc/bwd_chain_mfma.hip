@@ -291,6 +291,16 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
 
     // Staging registers: this thread's 16-byte chunks of the next Q / dO tile and its LSE / D entry.
     u32x4 qr[LD], gr[LD];
+#ifndef CHAIN_STAGE_C
+#define CHAIN_STAGE_C 3
+#endif
+    // D = 128: a tile is four units of 256 chunks (dO rows 0-15, Q rows 0-15, Q rows 16-31, dO rows
+    // 16-31); the producers stage the first 4 - SPLIT of them, the consumers the rest
+    constexpr int SPLIT = D == 128 ? CHAIN_STAGE_C : 2;
+    constexpr int U0 = producer ? 0 : 4 - SPLIT, NU = producer ? 4 - SPLIT : SPLIT;
+    u32x4 sr[NU > 0 ? NU : 1];
+    auto unit_is_q = [](int i) { return i == 1 || i == 2; };
+    auto unit_chunk0 = [](int i) { return i >= 2 ? 256 : 0; };
     float ls = 0.f, dd = 0.f;
     // Buffer loads: rows before the first or after the last query row are outside the descriptor's
     // range and read as zeros.
@@ -301,11 +311,19 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
     auto load_tile = [&](int r0) {
         if (CHAIN_ABLATE & 256) return;
         const int tt = (int)opaque((unsigned int)tid);
+        if constexpr (SPLIT != 2) {
+#pragma unroll
+            for (int i = 0; i < NU; ++i) {
+                const int c = unit_chunk0(U0 + i) + (tt & 255), row = c / CPR, cc = c % CPR;
+                sr[i] = __builtin_amdgcn_raw_buffer_load_b128(unit_is_q(U0 + i) ? q_rsrc : g_rsrc, ((r0 + row) * D + cc * 8) * 2, 0, 0);
+            }
+        } else {
 #pragma unroll
         for (int i = 0; i < LD; ++i) {
             const int c = min(tt + i * NT, CH - 1), row = c / CPR, cc = c % CPR;
             qr[i] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, ((r0 + row) * D + cc * 8) * 2, 0, 0);
             gr[i] = __builtin_amdgcn_raw_buffer_load_b128(g_rsrc, ((r0 + row) * D + cc * 8) * 2, 0, 0);
+        }
         }
         if constexpr (producer) {
             // raw values: arithmetic on them here would wait for the loads in this iteration
@@ -317,6 +335,13 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
         if (CHAIN_ABLATE & 256) return;
         const int tt = (int)opaque((unsigned int)tid);
         unsigned char *Qs = q_slot(t), *Gs = g_slot(t);
+        if constexpr (SPLIT != 2) {
+#pragma unroll
+            for (int i = 0; i < NU; ++i) {
+                const int c = unit_chunk0(U0 + i) + (tt & 255), row = c / CPR, cc = c % CPR;
+                *reinterpret_cast<u32x4 *>((unit_is_q(U0 + i) ? Qs : Gs) + row * RST + cc * 16) = sr[i];
+            }
+        } else {
 #pragma unroll
         for (int i = 0; i < LD; ++i) {
             const int c = tt + i * NT, row = c / CPR, cc = c % CPR;
@@ -324,6 +349,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                 *reinterpret_cast<u32x4 *>(Qs + row * RST + cc * 16) = qr[i];
                 *reinterpret_cast<u32x4 *>(Gs + row * RST + cc * 16) = gr[i];
             }
+        }
         }
         if constexpr (producer) {
             float *st = stat_slot(t);

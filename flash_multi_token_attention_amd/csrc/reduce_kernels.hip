@@ -50,18 +50,32 @@ __global__ __launch_bounds__(256) void preprocess_kernel(size_t rows, int d, con
     }
 }
 
-// dW[h][tap] = sum over (batch, tile) of the partials, in index order.
-__global__ void dw_reduce_kernel(int B, int H, int n_tiles, int ntap, const float *__restrict__ part,
-                                 float *__restrict__ dW) {
-    const int h = blockIdx.x;
-    for (int tap = threadIdx.x; tap < ntap; tap += blockDim.x) {
-        float s = 0.f;
-        for (int b = 0; b < B; ++b) {
-            const float *src = part + ((size_t)b * H + h) * n_tiles * ntap + tap;
-            for (int t = 0; t < n_tiles; ++t) s += src[(size_t)t * ntap];
+// dW[h][tap] = sum over (batch, tile) of the partials, in a fixed order: a workgroup takes 64 taps
+// of one head (lane = tap, so a partial is read with contiguous loads); wave w adds the partials
+// w, w+4, ... in four independent chains, and the four waves' sums are added in wave order.
+__global__ __launch_bounds__(256) void dw_reduce_kernel(int B, int H, int n_tiles, int ntap,
+                                                        const float *__restrict__ part, float *__restrict__ dW) {
+    __shared__ float red[4][64];
+    const int h = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int tap = blockIdx.y * 64 + lane;
+    const int n = B * n_tiles;
+    float s[4] = {0.f, 0.f, 0.f, 0.f};
+    if (tap < ntap) {
+        auto at = [&](int q) {
+            const int b = q / n_tiles, t = q - b * n_tiles;
+            return part[(((size_t)b * H + h) * n_tiles + t) * ntap + tap];
+        };
+        int q = wave;
+        for (; q + 12 < n; q += 16) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) s[c] += at(q + 4 * c);
         }
-        dW[(size_t)h * ntap + tap] = s;
+        for (int c = 0; q < n; q += 4, ++c) s[c] += at(q);
     }
+    red[wave][lane] = (s[0] + s[1]) + (s[2] + s[3]);
+    __syncthreads();
+    if (wave == 0 && tap < ntap)
+        dW[(size_t)h * ntap + tap] = (red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]);
 }
 
 // One workgroup per (batch, head): m = max m_s, l = sum l_s e^{m_s - m},
@@ -103,7 +117,7 @@ hipError_t bwd_preprocess(const Problem &p, int in_dt, int out_dt, const void *o
 }
 
 hipError_t dw_reduce(const Problem &p, int n_tiles, const float *dw_part, float *dw, hipStream_t s) {
-    dw_reduce_kernel<<<p.H, 256, 0, s>>>(p.B, p.H, n_tiles, p.c_q * p.c_k, dw_part, dw);
+    dw_reduce_kernel<<<dim3(p.H, (p.c_q * p.c_k + 63) / 64), 256, 0, s>>>(p.B, p.H, n_tiles, p.c_q * p.c_k, dw_part, dw);
     return hipGetLastError();
 }
 
