@@ -137,18 +137,20 @@ template <int CQT>
 __device__ __forceinline__ f16x8 band_frag(int t, const float *__restrict__ w_head, int c_q, int c_k, int pk,
                                            int g, int n, bool flip, float mul) {
     const int a = t - (CQT - c_q);
-    f16x8 f = (f16x8)(_Float16)0.f;
-    if (a >= 0) {
+    // (unconditional loads from clamped indices: the eight of a fragment are in flight together)
+    const float *row = w_head + max(a, 0) * c_k;
+    float v[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const int kappa = e < 4 ? 4 * g + e : 16 + 4 * g + e - 4;
-            const int off = kappa - kKeyHalo - n;
-            const int bb = flip ? pk - off : pk + off;
-            float v = 0.f;
-            if (bb >= 0 && bb < c_k) v = w_head[a * c_k + bb] * mul;
-            f[e] = (_Float16)v;
-        }
+    for (int e = 0; e < 8; ++e) {
+        const int kappa = e < 4 ? 4 * g + e : 16 + 4 * g + e - 4;
+        const int off = kappa - kKeyHalo - n;
+        const int bb = flip ? pk - off : pk + off;
+        v[e] = row[min(max(bb, 0), c_k - 1)];
+        if (a < 0 || bb < 0 || bb >= c_k) v[e] = 0.f;
     }
+    f16x8 f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f[e] = (_Float16)(v[e] * mul);
     return f;
 }
 
@@ -189,8 +191,14 @@ __device__ long long g_chain_ts[8][64][12];
         if (lane == 0 && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == CHAIN_TS && it < 64) \
             g_chain_ts[wave][it][i] = clock64();                                                  \
     } while (0)
+#define TSX(a, b)                                                                          \
+    do {                                                                                   \
+        if (lane == 0 && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == CHAIN_TS)     \
+            g_chain_ts[wave][a][b] = clock64();                                            \
+    } while (0)
 #else
 #define TS(i)
+#define TSX(a, b)
 #endif
 
 // Kernel arguments as one block: each role reads them from the kernel argument segment with
@@ -248,6 +256,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
     constexpr bool producer = ROLE == 0;
     constexpr bool WANT_KV = (WANT & 1) != 0, WANT_QW = (WANT & 2) != 0;
     const int pr = wave & (NP - 1);
+    TSX(0, 10);
 
     auto q_slot = [&](int t) { return smem + Lds::q_off + (t & 3) * Lds::tile_bytes; };
     auto g_slot = [&](int t) { return smem + Lds::g_off + (t % 3) * Lds::tile_bytes; };
@@ -357,24 +366,20 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
         }
     };
 
+    // Set-up: every global load of it is issued before the first wait (the first tile, K / V
+    // fragments, the rows above the first tile, the window's weights), so that it costs one round
+    // trip to memory instead of several.
     load_tile(r_begin);
-    stage_tile(0);
-    load_tile(r_begin + BR);
 
     if constexpr (producer) {
         // ================================ producer ================================
         const bf16_t *Kb = K + bh * p.Nk * D;
         const bf16_t *Vb = V + bh * p.Nk * D;
         // bands (times scale * log2 e: the convolved scores come out in log2 units) in LDS, one KB
-        // per tap slot, written by one wave; the first barrier of the tile loop publishes them
+        // per tap slot, the slots dealt out to the four waves; the first barrier of the tile loop
+        // publishes them
         // lane's 16 bytes of a band: the tap slot is a constant offset from one address register
         const unsigned char *bands = smem + opaque((unsigned int)Lds::band_off + lane * 16);
-        if (pr == 0) {
-#pragma unroll
-            for (int t = 0; t < CQT; ++t)
-                *reinterpret_cast<f16x8 *>(smem + Lds::band_off + t * 1024 + lane * 16) =
-                    band_frag<CQT>(t, W + (size_t)h * cq * ck, cq, ck, pk, g, n, false, p.scale * kLog2e);
-        }
         bf16x8 kf[NSB][KS];  // K rows c0-16 .. c0+47
         bf16x8 vf[NCB][KS];  // V rows c0-8 .. c0+39
 #pragma unroll
@@ -387,6 +392,19 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks)
                 vf[kb][ks] = __builtin_bit_cast(bf16x8, load_row16_nb<D>(Vb, c0 - 8 + kb * 16 + n, p.Nk, ks * 32 + g * 8));
+
+        // Q rows of the 32 rows above the first tile
+        bf16x8 q_above[2][KS];
+#pragma unroll
+        for (int f = 0; f < 2; ++f)
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+                q_above[f][ks] = __builtin_bit_cast(bf16x8, load_row16_nb<D>(Qb, r_begin - BR + 2 * n + f, p.Nq, ks * 32 + g * 8));
+        for (int t = pr; t < CQT; t += NP)
+            *reinterpret_cast<f16x8 *>(smem + Lds::band_off + t * 1024 + lane * 16) =
+                band_frag<CQT>(t, W + (size_t)h * cq * ck, cq, ck, pk, g, n, false, p.scale * kLog2e);
+        stage_tile(0);
+        load_tile(r_begin + BR);
 
         // packed fp16 scores of the previous tile: [block][fragment][dword]
         unsigned int prev_pd[NSB][2][2];
@@ -441,12 +459,10 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
 
         // the 32 rows above the first tile: their scores are the window's halo for tile 0
         {
-            const int rp = r_begin - BR;
-            s_phase(rp, 0, prev_pd, std::true_type{}, [&](int f, int ks) {
-                return __builtin_bit_cast(bf16x8, load_row16_nb<D>(Qb, rp + 2 * n + f, p.Nq, ks * 32 + g * 8));
-            });
+            s_phase(r_begin - BR, 0, prev_pd, std::true_type{}, [&](int f, int ks) { return q_above[f][ks]; });
         }
 
+        TSX(0, 11);
         for (int it = 0; it <= n_tiles + 1; ++it) {
             const int r0 = r_begin + it * BR;
             TS(0);
@@ -593,17 +609,40 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
             else ptile(std::false_type{}, std::true_type{});
             TS(6);
         }
+        TSX(1, 10);
         __syncthreads();  // the consumers' barrier before they hand over their dW accumulators
+        __syncthreads();  // ... and the one after it
+        // ---- dW partial of this workgroup: G[m][n] of half x belongs to key tap b = n - m + 16 x - 8 + pk;
+        // the sum runs over the pair groups, the halves and the diagonals' elements in a fixed order.
+        // S was raw, so * scale; dC was scaled, so / dcs. ----
+        static_assert(2 * CQT * 2 * 1024 <= NP * ChainLds<D, CQT>::pair_bytes, "room for the dW accumulators");
+        // Four lanes per tap (pair group, half), each adds its diagonal's elements in index order; the
+        // four sums are added as (0 + 1) + (2 + 3).
+        const int ntap = cq * ck;
+        for (int q = tid; WANT_QW && (q >> 2) < ntap; q += NT / 2) {
+            const int tap = q >> 2, a = tap / ck, bb = tap - a * ck, t = a + CQT - cq;
+            const int pgi = (q >> 1) & 1, x = q & 1;
+            const float *red = reinterpret_cast<const float *>(smem + Lds::pair_off) + ((pgi * CQT + t) * 2 + x) * 256;
+            float sum = 0.f;
+#pragma unroll
+            for (int m = 0; m < 16; ++m) {
+                const int nn = bb + m - 16 * x + 8 - pk;
+                const float val = red[m * 16 + min(max(nn, 0), 15)];
+                if (nn >= 0 && nn < 16) sum += val;
+            }
+            sum += __shfl_xor(sum, 1);
+            sum += __shfl_xor(sum, 2);
+            if ((q & 3) == 0) dW_part[(bh * gridDim.z + blockIdx.z) * ntap + tap] = sum * p.scale / dcs;
+        }
     } else {
         // ================================ consumer ================================
         const float *w_head = W + (size_t)h * cq * ck;
-        // flipped bands (times the softmax scale) in LDS, one KB per tap slot, written by one wave
+        // flipped bands (times the softmax scale) in LDS, one KB per tap slot, dealt out to the four waves
         unsigned char *bands = smem + opaque((unsigned int)Lds::band_off + CQT * 1024 + lane * 16);
-        if (pr == 0) {
-#pragma unroll
-            for (int t = 0; t < CQT; ++t)
-                *reinterpret_cast<f16x8 *>(bands + t * 1024) = band_frag<CQT>(t, w_head, cq, ck, pk, g, n, true, p.scale);
-        }
+        for (int t = pr; t < CQT; t += NP)
+            *reinterpret_cast<f16x8 *>(bands + t * 1024) = band_frag<CQT>(t, w_head, cq, ck, pk, g, n, true, p.scale);
+        stage_tile(0);
+        load_tile(r_begin + BR);
         // dW: this wave takes the key blocks of two pairs (pg) and half of the tap slots (t_lo ..)
         constexpr int TH = (CQT + 1) / 2;
         const int pg = pr >> 1, t_lo = (pr & 1) * TH;
@@ -626,6 +665,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
         const int n_kt = gridDim.z * NP, kt = blockIdx.z * NP + pr;
         bf16_t *ds_pair = dS_ws + (bh * n_kt + kt) * (size_t)n_rt * (WK * BR);
 
+        TSX(0, 11);
         for (int it = 0; it <= n_tiles + 1; ++it) {
             TS(0);
             __syncthreads();
@@ -856,6 +896,21 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
             TS(6);
         }
 
+        TSX(1, 10);
+        // ---- dW accumulators of this wave to LDS as [pair group][tap slot][x][m][n], once every
+        // wave is done with the tiles ----
+        __syncthreads();
+        float *red = reinterpret_cast<float *>(smem + Lds::pair_off);
+#pragma unroll
+        for (int tt = 0; tt < TH; ++tt)
+#pragma unroll
+            for (int x = 0; x < 2; ++x)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (WANT_QW && t_lo + tt < CQT)
+                        red[(((pg * CQT + t_lo + tt) * 2 + x) * 16 + 4 * g + r) * 16 + n] = acc_w[tt][x][r];
+        __syncthreads();  // the producers add the dW partial up while the consumers store dK and dV
+
         // ---- stores: lane = key, 4 consecutive head-dim columns per block ----
         const float inv = 1.f / dcs;
 #pragma unroll
@@ -890,38 +945,9 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
             }
         }
 
-        // ---- dW accumulators of this wave to LDS as [pair group][tap slot][x][m][n], once every
-        // wave is done with the tiles ----
-        __syncthreads();
-        float *red = reinterpret_cast<float *>(smem + Lds::pair_off);
-#pragma unroll
-        for (int tt = 0; tt < TH; ++tt)
-#pragma unroll
-            for (int x = 0; x < 2; ++x)
-#pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    if (WANT_QW && t_lo + tt < CQT)
-                        red[(((pg * CQT + t_lo + tt) * 2 + x) * 16 + 4 * g + r) * 16 + n] = acc_w[tt][x][r];
     }  // consumer
 
-    // ---- dW partial of this workgroup: G[m][n] of half x belongs to key tap b = n - m + 16 x - 8 + pk;
-    // the sum runs over the pair groups, the halves and the diagonals' elements in a fixed order.
-    // S was raw, so * scale; dC was scaled, so / dcs. ----
-    static_assert(2 * CQT * 2 * 1024 <= NP * ChainLds<D, CQT>::pair_bytes, "room for the dW accumulators");
-    __syncthreads();
-    const int ntap = cq * ck;
-    if (WANT_QW && tid < ntap) {
-        const int a = tid / ck, bb = tid - a * ck, t = a + CQT - cq;
-        const float *red = reinterpret_cast<const float *>(smem + Lds::pair_off);
-        float sum = 0.f;
-        for (int pgi = 0; pgi < 2; ++pgi)
-            for (int x = 0; x < 2; ++x)
-                for (int m = 0; m < 16; ++m) {
-                    const int nn = bb + m - 16 * x + 8 - pk;
-                    if (nn >= 0 && nn < 16) sum += red[(((pgi * CQT + t) * 2 + x) * 16 + m) * 16 + nn];
-                }
-        dW_part[(bh * gridDim.z + blockIdx.z) * ntap + tid] = sum * p.scale / dcs;
-    }
+    TSX(1, 11);
 }
 
 template <int D, int CQT, typename TO, int WANT>
