@@ -51,8 +51,14 @@ __device__ long long g_fwd_ts[4][64][8];
         if (lane == 0 && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == FWD_TS && u < 64)     \
             g_fwd_ts[wave][u][i] = clock64();                                                      \
     } while (0)
+#define FTSX(a, b)                                                                        \
+    do {                                                                                  \
+        if (lane == 0 && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == FWD_TS)      \
+            g_fwd_ts[wave][a][b] = clock64();                                             \
+    } while (0)
 #else
 #define FTS(i)
+#define FTSX(a, b)
 #endif
 
 template <int D> struct FwdLds {
@@ -80,6 +86,7 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;  // wave-uniform for the compiler too
     const int g = lane >> 4, n = lane & 15;
+    FTSX(0, 6);
 
     // x = head, y = batch, z = query tile: the dispatcher hands out every (batch, head) of the
     // longest (causal) tiles first, so the tail of the launch is made of short tiles
@@ -100,21 +107,27 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
     f16x8 tf[CQT];
     {
         const float *w_head = W + (size_t)h * cq * p.c_k;
+        // (unconditional loads from clamped indices, all in flight together; the select happens on the values)
+        float wv[CQT][8];
 #pragma unroll
         for (int t = 0; t < CQT; ++t) {
             const int a = t - (CQT - cq);
-            f16x8 f = (f16x8)(_Float16)0.f;
-            if (a >= 0) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const int kappa = e < 4 ? 4 * g + e : 16 + 4 * g + e - 4;
-                    const int bb = kappa - kKeyHalo - n + pk;
-                    float v = 0.f;
-                    if (bb >= 0 && bb < p.c_k) v = w_head[a * p.c_k + bb] * (p.scale * kLog2e);
-                    f[e] = (_Float16)v;
-                }
+            for (int e = 0; e < 8; ++e) {
+                const int kappa = e < 4 ? 4 * g + e : 16 + 4 * g + e - 4;
+                const int bb = kappa - kKeyHalo - n + pk;
+                wv[t][e] = w_head[max(a, 0) * p.c_k + min(max(bb, 0), p.c_k - 1)];
             }
-            tf[t] = f;
+        }
+#pragma unroll
+        for (int t = 0; t < CQT; ++t) {
+            const int a = t - (CQT - cq);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int kappa = e < 4 ? 4 * g + e : 16 + 4 * g + e - 4;
+                const int bb = kappa - kKeyHalo - n + pk;
+                tf[t][e] = (_Float16)((a >= 0 && bb >= 0 && bb < p.c_k) ? wv[t][e] * (p.scale * kLog2e) : 0.f);
+            }
         }
     }
 
@@ -384,11 +397,13 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
     const int u_tail = p.Nk < 24 ? 1 : (p.Nk - 24) / 32 + 1;    // first u >= 1 with 32u + 24 > Nk
     const int u1 = min(causal ? min(u_diag, u_tail) : u_tail, n_steps);
     const int u2 = max(u1, causal ? min((i0w + WR + 15) / 32 + 1, n_steps) : n_steps);  // 32u - 16 > i0w + WR - 1
+    FTSX(0, 7);
     run(0, 1, std::integral_constant<int, 1>{});
     run(1, u1, std::integral_constant<int, 0>{});
     run(u1, u2, std::integral_constant<int, 1>{});
     run(u2, n_steps, std::integral_constant<int, 2>{});
 
+    FTSX(1, 6);
     // ---- epilogue: finish the row sums and maxima, normalise, store O, M, L ----
 #pragma unroll
     for (int ob = 0; ob < 2; ++ob) {
@@ -421,6 +436,7 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
             }
         }
     }
+    FTSX(1, 7);
 }
 
 template <int D, int CQT, typename TO>
