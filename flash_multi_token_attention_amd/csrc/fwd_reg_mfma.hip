@@ -4,8 +4,10 @@
 // (the first CQT-1 of them only as the window's halo above its 33-CQT output rows) and keeps
 // O^T, the row sums and the softmax bases of its rows in registers for the whole key loop.
 // Lane n of score fragment f holds row base + 2n + f.  Per 32-key step:
-//   1. all waves write the K / V rows they loaded during the previous step to the LDS buffer
-//      of the next step and issue the loads for the step after it (one barrier per step);
+//   1. all waves issue the loads of the next step's K / V rows, which go from global memory
+//      straight into the LDS buffer the step before this one has just left (buffer loads with the
+//      LDS modifier: no staging registers, no LDS writes by the waves; rows are dense and their
+//      16-byte chunks XOR-swizzled with the row index; one barrier per step);
 //   2. S^T = K Q^T for two 16-key blocks; the accumulator layout (lane = query row, 4 keys per
 //      lane group) is, packed to fp16 after the causal pre-mask, already the B operand layout of
 //      the convolution MFMA: k slots 0..3 of a lane group come from one block, 4..7 from the next
@@ -32,6 +34,16 @@ typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 template <int CTRL>
 __device__ __forceinline__ unsigned int dpp_zero(unsigned int src) {
     return (unsigned int)__builtin_amdgcn_update_dpp(0, (int)src, CTRL, 0xf, 0xf, true);
+}
+
+__device__ __forceinline__ unsigned int opaque_u32(unsigned int x) {
+    asm volatile("" : "+v"(x));
+    return x;
+}
+__device__ __forceinline__ bf16x4 lds_tr64(const unsigned char *ptr) {
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(ptr));
+    return __builtin_bit_cast(bf16x4, v);
 }
 
 constexpr int NW = 4;             // waves per workgroup
@@ -61,11 +73,30 @@ __device__ long long g_fwd_ts[4][64][8];
 #define FTSX(a, b)
 #endif
 
+#ifndef FWD_DMA
+#define FWD_DMA 1
+#endif
+#ifndef FWD_NBUF
+#define FWD_NBUF 2
+#endif
 template <int D> struct FwdLds {
+#if FWD_DMA
+    // K / V rows go from global memory straight into LDS (buffer loads with the LDS modifier: the
+    // 64 lanes of a load fill 1 KB of consecutive LDS, which rules out padded rows), so the rows are
+    // dense and the 16-byte chunk c of row r sits at chunk position c ^ (r mod chunks per row):
+    // a fragment read (16 rows, one column) then touches 16 different bank groups.
+    static constexpr int KST = D * 2;
+#else
     static constexpr int KST = D * 2 + 16;  // bytes per K / V row (== 16 mod 256 for D = 128)
+#endif
     static constexpr int k_bytes = BK * KST;
     static constexpr int buf_bytes = 2 * k_bytes;  // K rows, then V rows
-    static constexpr int total = 2 * buf_bytes;    // double-buffered
+#if FWD_DMA
+    static constexpr int n_buf = FWD_NBUF;         // steps u, u+1 (and u+2) resident or on their way
+#else
+    static constexpr int n_buf = 2;
+#endif
+    static constexpr int total = n_buf * buf_bytes;
 };
 
 template <int D, int CQT, typename TO>
@@ -81,7 +112,7 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
     constexpr int WR = wave_rows(CQT), BQ = NW * WR;
     constexpr int N_LD = BK * CPR / (NW * 64);  // 16-byte chunks per thread and matrix
     static_assert(BK * CPR % (NW * 64) == 0 && (NW * 64) % CPR == 0, "whole chunks per thread, whole rows per pass");
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;  // wave-uniform for the compiler too
@@ -161,13 +192,57 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
     // are carried from the previous step.
     // Staging registers: every thread holds its 16-byte chunks of the K / V rows of step u+2
     // while step u is computed.
+#if !FWD_DMA
     u32x4 kr[N_LD], vr[N_LD];
+#endif
     // Buffer loads: rows before the first or after the last key are outside the descriptor's
     // range and read as zeros, which is what the window's zero padding asks for.
     const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)Kb, 0, p.Nk * D * 2, 0x00020000);
     const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)Vb, 0, p.Nk * D * 2, 0x00020000);
     const int ld_off = ((tid / CPR) * D + (tid % CPR) * 8) * 2;  // byte offset of this thread's first chunk in a step
     constexpr int kChunkStep = (NW * 64 / CPR) * D * 2;         // and from one of its chunks to the next
+#if FWD_DMA
+    // Load i of a wave fills rows RPL (i NW + wave) .. + RPL - 1 of a tile (RPL = rows per KB): lane l
+    // writes chunk position l % CPR of row l / CPR and therefore reads chunk (l % CPR) ^ (row % CPR).
+    constexpr int RPL = 1024 / (D * 2);
+    static_assert(N_LD * NW * RPL == BK, "whole tiles");
+    const int dma_off = ((lane / CPR) * D + ((lane % CPR) ^ ((lane / CPR + RPL * wave) % CPR)) * 8) * 2 + wave * 1024;
+    // rows of step u: issued right after the barrier that ends step u - 1 (their buffer is free then),
+    // landed by the barrier that starts step u (the barrier waits for the wave's loads)
+    // (issued as inline assembly: for the builtin the compiler makes every later LDS read wait for the
+    // load, since it cannot tell the two buffers apart; the wait is written out before the barrier instead)
+    typedef int i32x4 __attribute__((ext_vector_type(4)));
+    auto dma_rsrc = [&](const bf16_t *ptr) {
+        const unsigned long long a = reinterpret_cast<unsigned long long>(ptr);
+        return (i32x4){(int)(unsigned int)a, (int)(unsigned int)(a >> 32), p.Nk * D * 2, 0x00020000};
+    };
+    const i32x4 k_dma = dma_rsrc(Kb), v_dma = dma_rsrc(Vb);
+    const unsigned int lds_base =
+        (unsigned int)(unsigned long long)(__attribute__((address_space(3))) unsigned char *)smem + wave * 1024;
+    auto dma16 = [&](const i32x4 &rsrc, unsigned int lds_addr, int voffset) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                     :: "s"(lds_addr), "v"(voffset), "s"(rsrc) : "memory");
+    };
+    auto fetch_step = [&](int u) {
+        const unsigned int Ks = lds_base + (u % Lds::n_buf) * Lds::buf_bytes, Vs = Ks + Lds::k_bytes;
+        const int k0 = (32 * u - 8) * D * 2 + dma_off, v0 = (32 * u - 16) * D * 2 + dma_off;
+#pragma unroll
+        for (int i = 0; i < N_LD; ++i) {
+            dma16(k_dma, Ks + i * NW * 1024, k0 + i * NW * 1024);
+            dma16(v_dma, Vs + i * NW * 1024, v0 + i * NW * 1024);
+        }
+    };
+    // lane addresses of the fragment reads inside a tile: chunk c of row r at r KST + ((c ^ (r % CPR)) << 4);
+    // row blocks of 16 and the buffers are constant offsets on top
+    unsigned int ka[KS], va[DB];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) ka[ks] = opaque_u32(n * KST + (((ks * 4 + g) ^ (n % CPR)) << 4));
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+        const int r = 4 * g + (n >> 2);
+        va[db] = opaque_u32(r * KST + (((db * 2 + ((n >> 1) & 1)) ^ (r % CPR)) << 4) + (n & 1) * 8);
+    }
+#else
     auto load_step = [&](int u) {
         const int k0 = (32 * u - 8) * D * 2 + ld_off, v0 = (32 * u - 16) * D * 2 + ld_off;
 #pragma unroll
@@ -185,6 +260,7 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
             *reinterpret_cast<u32x4 *>(Vs + row * KST + cc * 16) = vr[i];
         }
     };
+#endif
 
     // packed fp16 scores of the last score block of the previous step:
     // carry[f][dword] = row base + 2n + f, keys 4g .. 4g+3 of the block
@@ -194,7 +270,13 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
     // (wave-uniform), only then are the masks evaluated.
     auto step = [&](int u, auto edge_tag) {
         constexpr bool EDGE = decltype(edge_tag)::value;
+#if FWD_DMA
+        // (the address registers ka / va point into the buffer of the step: they are moved to the
+        // other buffer at the end of every step)
+        const unsigned char *Ks = smem, *Vs = Ks + Lds::k_bytes;
+#else
         const unsigned char *Ks = smem + (u & 1) * Lds::buf_bytes, *Vs = Ks + Lds::k_bytes;
+#endif
         const int jk = 32 * u - 8, jv = 32 * u - 16;
         f32x4 c[2][2];
         bf16x8 kf[KS];  // K fragments of one score block; the second block's are read during the first's convolution
@@ -202,7 +284,11 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
         auto load_kf = [&](int blk) {
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks)
+#if FWD_DMA
+                kf[ks] = *reinterpret_cast<const bf16x8 *>(Ks + ka[ks] + blk * 16 * KST);
+#else
                 kf[ks] = *reinterpret_cast<const bf16x8 *>(Ks + (blk * 16 + n) * KST + (ks * 32 + g * 8) * 2);
+#endif
         };
         load_kf(0);
         static_for<2>([&](auto BL) {
@@ -273,8 +359,13 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
         constexpr int PFV = FWD_PFV < DB ? FWD_PFV : DB;
         bf16x8 vf[PFV + 1];
         auto load_vf = [&](int buf, int db) {
+#if FWD_DMA
+            bf16x4 lo = lds_tr64(Vs + va[db]);
+            bf16x4 hi = lds_tr64(Vs + va[db] + 16 * KST);
+#else
             bf16x4 lo = lds_read_tr4x16(Vs, KST, 4 * g, db * 16, n);
             bf16x4 hi = lds_read_tr4x16(Vs, KST, 16 + 4 * g, db * 16, n);
+#endif
             vf[buf] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
         };
 #pragma unroll
@@ -373,9 +464,14 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
 
     const int k_end = causal ? min(p.Nk, i0 + BQ) : p.Nk;
     const int n_steps = (k_end + 16 + BK - 1) / BK;
+#if FWD_DMA
+    fetch_step(0);
+    if constexpr (Lds::n_buf == 3) fetch_step(1);
+#else
     load_step(0);
     stage_step(0);
     load_step(1);
+#endif
     // Along the keys a wave's steps are: step 0 (keys before the first one to mask), steps whose
     // keys all lie at or before its first score row (no masks), steps on the diagonal or at the
     // end of the keys (masks), and steps entirely after its rows (it only takes part in the
@@ -385,12 +481,28 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
 #pragma unroll 1
         for (int u = ua; u < ub; ++u) {
             FTS(0);
+#if FWD_DMA
+            // this wave's rows of step u have landed (with three buffers those of step u + 1 may be on their way)
+            if constexpr (Lds::n_buf == 3) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * N_LD) : "memory");
+            else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#endif
             __syncthreads();  // step u-1 is done everywhere: its buffer is free, and step u's is written
             FTS(1);
+#if FWD_DMA
+            fetch_step(u + Lds::n_buf - 1);
+            FTS(2);
+            if constexpr (KIND != 2) step(u, std::integral_constant<bool, KIND == 1>{});
+            const int to_other = (u % Lds::n_buf == Lds::n_buf - 1) ? -(Lds::n_buf - 1) * Lds::buf_bytes : Lds::buf_bytes;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) ka[ks] += to_other;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) va[db] += to_other;
+#else
             stage_step(u + 1);
             load_step(u + 2);
             FTS(2);
             if constexpr (KIND != 2) step(u, std::integral_constant<bool, KIND == 1>{});
+#endif
         }
     };
     const int u_diag = base < 23 ? 1 : (base - 23) / 32 + 1;    // first u >= 1 with 32u + 23 > base
