@@ -14,8 +14,9 @@
 //       packed dC^T (rows below a tile come from the next tile, hence the extra tile of delay),
 //       dS -> workspace (bf16 blocks of 32 rows x 32 keys in the order the lanes hold them) and
 //       -> LDS, dK^T += Q^T dS.
-// One workgroup barrier per tile; Q and dO tiles are staged row-major with rows padded by 16 bytes
-// (row fragments are 128-bit reads, the transposed operands of dV / dK 64-bit transpose reads).
+// One workgroup barrier per tile; Q and dO tiles go from global memory straight into LDS (buffer
+// loads with the LDS modifier, one tile ahead), in a layout that serves both the 128-bit row
+// fragment reads of the producers and the 64-bit transpose reads of dV / dK (see ChainLds).
 //
 // dW[a][b] = sum_i sum_j dC[i][j] S_m[i+a-pq][j+b-pk] is computed as G_a = dC^T S(rows shifted by
 // a), a [key j] x [key j'] product contracted over the rows on the matrix cores; only its
@@ -50,7 +51,13 @@ constexpr int PST = 72;          // bytes per row of the P and dS tiles (32 keys
 static_assert(BKW == kKvKeysPerWg && WK == kChainKeys && BR == kChainRows, "dS workspace layout");
 
 template <int D, int CQT> struct ChainLds {
-    static constexpr int RST = D * 2 + 16;                          // bytes per staged Q / dO row
+    // Q / dO tiles are filled by buffer loads with the LDS modifier (64 lanes = 1 KB of consecutive
+    // LDS), which rules out padded rows.  A tile of 32 rows is kept as [k-step ks][row parity f]
+    // [row pair n][64 bytes]: the 4 chunks of 16 bytes that row 2n + f holds of head-dim columns
+    // 32 ks .. 32 ks + 31, chunk c at position c ^ (n / 4 mod 4).  Row fragments (lane n reads row
+    // 2n + f) and transposed fragments then touch every bank equally often, and k-step, parity and
+    // head-dim block are constant offsets from one lane address.
+    static constexpr int RST = D * 2;                               // bytes per Q / dO row
     static constexpr int tile_bytes = BR * RST;
     static constexpr int q_off = 0, q_slots = 4;                    // tiles it-2 .. it+1
     static constexpr int g_off = q_off + q_slots * tile_bytes, g_slots = 3;  // tiles it-1 .. it+1
@@ -246,9 +253,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
     const int n_rt = args.n_rt;
     using Lds = ChainLds<D, CQT>;
     constexpr int KS = D / 32, DB = D / 16, CPR = D / 8, RST = Lds::RST;
-    constexpr int CH = BR * CPR;                 // 16-byte chunks of a staged tile
-    constexpr int LD = (CH + NT - 1) / NT;       // per thread
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
@@ -298,78 +303,79 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
     // no (row, key) pair of the tile is visible: only its scores are needed, by the tile below
     auto is_skipped = [&](int r0) { return causal && r0 + BR - 1 < c0 - 8; };
 
-    // Staging registers: this thread's 16-byte chunks of the next Q / dO tile and its LSE / D entry.
-    u32x4 qr[LD], gr[LD];
-#ifndef CHAIN_STAGE_C
-#define CHAIN_STAGE_C 3
-#endif
-    // D = 128: a tile is four units of 256 chunks (dO rows 0-15, Q rows 0-15, Q rows 16-31, dO rows
-    // 16-31); the producers stage the first 4 - SPLIT of them, the consumers the rest
-    constexpr int SPLIT = D == 128 ? CHAIN_STAGE_C : 2;
-    constexpr int U0 = producer ? 0 : 4 - SPLIT, NU = producer ? 4 - SPLIT : SPLIT;
-    u32x4 sr[NU > 0 ? NU : 1];
-    auto unit_is_q = [](int i) { return i == 1 || i == 2; };
-    auto unit_chunk0 = [](int i) { return i >= 2 ? 256 : 0; };
-    float ls = 0.f, dd = 0.f;
-    // Buffer loads: rows before the first or after the last query row are outside the descriptor's
-    // range and read as zeros.
-    const __amdgpu_buffer_rsrc_t q_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)Qb, 0, p.Nq * D * 2, 0x00020000);
-    const __amdgpu_buffer_rsrc_t g_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)dOb, 0, p.Nq * D * 2, 0x00020000);
-    // (the thread's chunk coordinates are recomputed from an opaque copy of its index at every use:
-    // kept in registers across the tile loop they are what the register allocator spills first)
-    auto load_tile = [&](int r0) {
+    // Q / dO tiles: global memory -> LDS without passing through registers.  A tile is 2 KBT units
+    // of 1 KB (KBT of Q, then KBT of dO; unit 2 ks + f = the 16 row pairs of one k-step and parity);
+    // wave w issues the units w, w + 8, ...  Lane l of a load fills chunk position l % 4 of row pair
+    // l / 4.  Rows after the last query row are outside the descriptor's range and arrive as zeros.
+    // (Inline assembly: for the builtin the compiler makes every later LDS read wait for the load,
+    // as it cannot tell the tile slots apart; the wait is written out before the barrier instead.)
+    typedef int i32x4 __attribute__((ext_vector_type(4)));
+    constexpr int KBT = Lds::tile_bytes / 1024;
+    static_assert(KBT == 2 * KS, "one unit per k-step and row parity");
+    auto dma_rsrc = [&](const bf16_t *ptr) {
+        const unsigned long long a = reinterpret_cast<unsigned long long>(ptr);
+        return (i32x4){(int)(unsigned int)a, (int)(unsigned int)(a >> 32), p.Nq * D * 2, 0x00020000};
+    };
+    const i32x4 q_dma = dma_rsrc(Qb), g_dma = dma_rsrc(dOb);
+    const unsigned int lds0 = (unsigned int)(unsigned long long)(__attribute__((address_space(3))) unsigned char *)smem;
+    auto fetch_tile = [&](int t) {
         if (CHAIN_ABLATE & 256) return;
-        const int tt = (int)opaque((unsigned int)tid);
-        if constexpr (SPLIT != 2) {
+        const int ln = (int)opaque((unsigned int)lane);
 #pragma unroll
-            for (int i = 0; i < NU; ++i) {
-                const int c = unit_chunk0(U0 + i) + (tt & 255), row = c / CPR, cc = c % CPR;
-                sr[i] = __builtin_amdgcn_raw_buffer_load_b128(unit_is_q(U0 + i) ? q_rsrc : g_rsrc, ((r0 + row) * D + cc * 8) * 2, 0, 0);
-            }
-        } else {
-#pragma unroll
-        for (int i = 0; i < LD; ++i) {
-            const int c = min(tt + i * NT, CH - 1), row = c / CPR, cc = c % CPR;
-            qr[i] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, ((r0 + row) * D + cc * 8) * 2, 0, 0);
-            gr[i] = __builtin_amdgcn_raw_buffer_load_b128(g_rsrc, ((r0 + row) * D + cc * 8) * 2, 0, 0);
+        for (int j0 = 0; j0 < 2 * KBT; j0 += 2 * NP) {
+            const int j = j0 + wave, m = j / KBT, kb = j - m * KBT;
+            const int row = 2 * (ln >> 2) + (kb & 1), chunk = (kb >> 1) * 4 + ((ln & 3) ^ ((ln >> 4) & 3));
+            const int voff = ((r_begin + t * BR + row) * D + chunk * 8) * 2;
+            const unsigned int dst = lds0 + (m ? Lds::g_off + (t % 3) * Lds::tile_bytes : Lds::q_off + (t & 3) * Lds::tile_bytes) + kb * 1024;
+            const i32x4 rsrc = m ? g_dma : q_dma;
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                         :: "s"(dst), "v"(voff), "s"(rsrc) : "memory");
         }
-        }
+    };
+    // Every tile this wave has asked for is in LDS (to be followed by the workgroup barrier).  Vector
+    // memory operations complete in the order of their issue: `younger` = the global stores the wave
+    // has issued since the tile loads (the dS block of an iteration: NDB * 2), which need not be waited for.
+    auto tiles_landed = [&](bool younger) {
+        if (younger) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(NDB * 2) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    };
+    static_assert((2 * KBT) % (2 * NP) == 0, "whole units per wave");
+    // LSE and D of a tile: loaded by the first 32 threads one iteration before they are written to LDS
+    float ls = 0.f, dd = 0.f;
+    auto load_stats = [&](int r0) {
         if constexpr (producer) {
             // raw values: arithmetic on them here would wait for the loads in this iteration
+            const int tt = (int)opaque((unsigned int)tid);
             ls = 1e30f; dd = 0.f;  // rows past the end: exp2(C - LSE) = 0
             if (tt < BR && r0 + tt < p.Nq) { ls = lse_b[r0 + tt]; dd = dl_b[r0 + tt]; }
         }
     };
-    auto stage_tile = [&](int t) {
-        if (CHAIN_ABLATE & 256) return;
-        const int tt = (int)opaque((unsigned int)tid);
-        unsigned char *Qs = q_slot(t), *Gs = g_slot(t);
-        if constexpr (SPLIT != 2) {
-#pragma unroll
-            for (int i = 0; i < NU; ++i) {
-                const int c = unit_chunk0(U0 + i) + (tt & 255), row = c / CPR, cc = c % CPR;
-                *reinterpret_cast<u32x4 *>((unit_is_q(U0 + i) ? Qs : Gs) + row * RST + cc * 16) = sr[i];
-            }
-        } else {
-#pragma unroll
-        for (int i = 0; i < LD; ++i) {
-            const int c = tt + i * NT, row = c / CPR, cc = c % CPR;
-            if (c < CH) {
-                *reinterpret_cast<u32x4 *>(Qs + row * RST + cc * 16) = qr[i];
-                *reinterpret_cast<u32x4 *>(Gs + row * RST + cc * 16) = gr[i];
-            }
-        }
-        }
+    auto stage_stats = [&](int t) {
         if constexpr (producer) {
+            const int tt = (int)opaque((unsigned int)tid);
             float *st = stat_slot(t);
             if (tt < BR) { st[tt] = ls * kLog2e - dcs_log2; st[BR + tt] = dd; }
         }
+    };
+    // Lane parts of the fragment addresses inside a tile.  Row fragment (producers): row 2n + f,
+    // chunk 4 ks + g: + f KB + 2 ks KB.  Transposed fragment (consumers): rows 4g + n/4 (+ 16 hi),
+    // 8 bytes at byte column 32 db + 8 (n % 4): see read_tr_t for the constant part.
+    auto row_frag_off = [&] { return (unsigned int)(n * 64 + ((g ^ ((n >> 2) & 3)) << 4)); };
+    auto tr_frag_off = [&] {
+        return (unsigned int)(((n >> 2) & 1) * 1024 + (2 * g + (n >> 3)) * 64 + ((((n >> 1) & 1) ^ (g >> 1)) << 4) + (n & 1) * 8);
+    };
+    auto read_tr_t = [&](const unsigned char *lane_ptr, int db) {   // (db: a constant after unrolling)
+        // rows + 16: row pair + 8, whose chunk positions are those of this one with bit 1 flipped
+        bf16x4 lo = lds_tr64(lane_ptr + (db >> 1) * 2048 + ((db & 1) << 5));
+        bf16x4 hi = lds_tr64(lane_ptr + (db >> 1) * 2048 + (((db & 1) ^ 1) << 5) + 512);
+        return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
     };
 
     // Set-up: every global load of it is issued before the first wait (the first tile, K / V
     // fragments, the rows above the first tile, the window's weights), so that it costs one round
     // trip to memory instead of several.
-    load_tile(r_begin);
+    fetch_tile(0);
+    load_stats(r_begin);
 
     if constexpr (producer) {
         // ================================ producer ================================
@@ -403,8 +409,8 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
         for (int t = pr; t < CQT; t += NP)
             *reinterpret_cast<f16x8 *>(smem + Lds::band_off + t * 1024 + lane * 16) =
                 band_frag<CQT>(t, W + (size_t)h * cq * ck, cq, ck, pk, g, n, false, p.scale * kLog2e);
-        stage_tile(0);
-        load_tile(r_begin + BR);
+        stage_stats(0);
+        load_stats(r_begin + BR);
 
         // packed fp16 scores of the previous tile: [block][fragment][dword]
         unsigned int prev_pd[NSB][2][2];
@@ -466,10 +472,13 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
         for (int it = 0; it <= n_tiles + 1; ++it) {
             const int r0 = r_begin + it * BR;
             TS(0);
+            tiles_landed(false);
             __syncthreads();
             TS(1);
-            if (it + 1 < n_tiles) stage_tile(it + 1);
-            load_tile(r0 + 2 * BR);
+            // (the LSE / D loads before the tile loads: the wait above is for the youngest loads of the wave)
+            if (it + 1 < n_tiles) stage_stats(it + 1);
+            load_stats(r0 + 2 * BR);
+            if (it + 1 < n_tiles) fetch_tile(it + 1);
             TS(2);
             // dC of a tile that has none (entirely above the diagonal, or the one after the last):
             // zeros, so that the consumers read every tile alike
@@ -493,8 +502,8 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                 constexpr bool EDGE = decltype(edge_tag)::value;
                 constexpr bool FULL = decltype(full_tag)::value;
                 // row fragments: lane n of fragment f reads row 2n + f, 16 bytes at column 32 ks + 8 g
-                const unsigned char *Qs = smem + opaque((unsigned int)(q_slot(it) - smem) + 2 * n * RST + g * 16);
-                const unsigned char *Gs = smem + opaque((unsigned int)(g_slot(it) - smem) + 2 * n * RST + g * 16);
+                const unsigned char *Qs = smem + opaque((unsigned int)(q_slot(it) - smem) + row_frag_off());
+                const unsigned char *Gs = smem + opaque((unsigned int)(g_slot(it) - smem) + row_frag_off());
                 __builtin_amdgcn_s_setprio(CHAIN_PRIO_P);
                 f32x4 dp[NCB][2];
                 float2 l2 = {0.f, 0.f};
@@ -503,7 +512,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                 // ---- S^T ----
                 unsigned int pd[NSB][2][2];
                 s_phase(r0, it + 1, pd, edge_tag, [&](int f, int ks) {
-                    return *reinterpret_cast<const bf16x8 *>(Qs + f * RST + ks * 64);
+                    return *reinterpret_cast<const bf16x8 *>(Qs + f * 1024 + ks * 2048);
                 });
                 CHAIN_SCHED_BARRIER;
                 TS(3);
@@ -557,7 +566,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                             bf16x8 gf[2];
 #pragma unroll
                             for (int f = 0; f < 2; ++f)
-                                gf[f] = *reinterpret_cast<const bf16x8 *>(Gs + f * RST + ks * 64);
+                                gf[f] = *reinterpret_cast<const bf16x8 *>(Gs + f * 1024 + ks * 2048);
 #pragma unroll
                             for (int cb = 0; cb < NCB; ++cb)
 #pragma unroll
@@ -641,8 +650,6 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
         unsigned char *bands = smem + opaque((unsigned int)Lds::band_off + CQT * 1024 + lane * 16);
         for (int t = pr; t < CQT; t += NP)
             *reinterpret_cast<f16x8 *>(bands + t * 1024) = band_frag<CQT>(t, w_head, cq, ck, pk, g, n, true, p.scale);
-        stage_tile(0);
-        load_tile(r_begin + BR);
         // dW: this wave takes the key blocks of two pairs (pg) and half of the tap slots (t_lo ..)
         constexpr int TH = (CQT + 1) / 2;
         const int pg = pr >> 1, t_lo = (pr & 1) * TH;
@@ -666,12 +673,14 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
         bf16_t *ds_pair = dS_ws + (bh * n_kt + kt) * (size_t)n_rt * (WK * BR);
 
         TSX(0, 11);
+        bool ds_stored = false;  // the last iteration stored a dS block (after its tile loads)
         for (int it = 0; it <= n_tiles + 1; ++it) {
             TS(0);
+            tiles_landed(ds_stored);
+            ds_stored = false;
             __syncthreads();
             TS(1);
-            if (it + 1 < n_tiles) stage_tile(it + 1);
-            load_tile(r_begin + (it + 2) * BR);
+            if (it + 1 < n_tiles) fetch_tile(it + 1);
             TS(2);
             const int u = it - 1, v = it - 2;
             const int r0u = r_begin + u * BR, r0v = r_begin + v * BR;
@@ -687,7 +696,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
             // the round trip of dS through LDS), dK.
             if (WANT_KV && u_ok && !(CHAIN_ABLATE & 4)) {
                 const unsigned char *Ps = smem + opaque((unsigned int)(p_stage(u) - smem) + tr_lane_off(PST, g, n));
-                const unsigned char *Gs = smem + opaque((unsigned int)(g_slot(u) - smem) + tr_lane_off(RST, g, n));
+                const unsigned char *Gs = smem + opaque((unsigned int)(g_slot(u) - smem) + tr_frag_off());
                 __builtin_amdgcn_s_setprio(CHAIN_PRIO_C);
                 // ---- dV^T += dO^T P (keys c0-8 .. c0+23) ----
                 // the dO^T fragment of head-dim block db + PF is read while block db is multiplied: the
@@ -697,11 +706,11 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
 #pragma unroll
                 for (int cb = 0; cb < 2; ++cb) pf[cb] = read_tr(Ps, PST, cb * 16);
 #pragma unroll
-                for (int db = 0; db < PF && db < DB; ++db) gq[db] = read_tr(Gs, RST, db * 16);
+                for (int db = 0; db < PF && db < DB; ++db) gq[db] = read_tr_t(Gs, db);
                 static_for<DB>([&](auto DBI) {
                     constexpr int db = decltype(DBI)::value;
                     if constexpr (db + PF < DB) {
-                        gq[(db + PF) % (PF + 1)] = read_tr(Gs, RST, (db + PF) * 16);
+                        gq[(db + PF) % (PF + 1)] = read_tr_t(Gs, db + PF);
                         SCHED_DS_READ_ID(2, 60 + db);
                     }
 #pragma unroll
@@ -775,7 +784,10 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                         for (int r = 0; r < 4; ++r) sv[r] = (bf16_t)ds[sb][ob][r];
                         // block layout [row parity][key half][16 row pairs][16 keys]: the 64 lanes of a store
                         // write 512 contiguous bytes
-                        if constexpr (WANT_QW) *reinterpret_cast<bf16x4 *>(ds_blk + ((ob * 2 + sb) * 16 + n) * 16 + 4 * g) = sv;
+                        if constexpr (WANT_QW) {
+                            *reinterpret_cast<bf16x4 *>(ds_blk + ((ob * 2 + sb) * 16 + n) * 16 + 4 * g) = sv;
+                            ds_stored = true;
+                        }
                         if constexpr (WANT_KV) *reinterpret_cast<bf16x4 *>(ds_tile + (2 * n + ob) * PST + (sb * 16 + 4 * g) * 2) = sv;
                     }
                 TS(9);
@@ -864,7 +876,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
             CHAIN_SCHED_BARRIER;
             TS(5);
             if (WANT_KV && v_ok && !(CHAIN_ABLATE & 8)) {
-                const unsigned char *Qs = smem + opaque((unsigned int)(q_slot(v) - smem) + tr_lane_off(RST, g, n));
+                const unsigned char *Qs = smem + opaque((unsigned int)(q_slot(v) - smem) + tr_frag_off());
                 const unsigned char *Dsl = smem + opaque((unsigned int)(ds_tile - smem) + tr_lane_off(PST, g, n));
                 asm volatile("" ::: "memory");
                 __builtin_amdgcn_wave_barrier();
@@ -875,13 +887,13 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                     bf16x8 sf[2], qq[PF + 1];
                     // (Q^T does not depend on the dS tile: its first fragments are on their way first)
 #pragma unroll
-                    for (int db = 0; db < PF && db < DB; ++db) qq[db] = read_tr(Qs, RST, db * 16);
+                    for (int db = 0; db < PF && db < DB; ++db) qq[db] = read_tr_t(Qs, db);
 #pragma unroll
                     for (int sb = 0; sb < 2; ++sb) sf[sb] = read_tr(Dsl, PST, sb * 16);
                     static_for<DB>([&](auto DBI) {
                         constexpr int db = decltype(DBI)::value;
                         if constexpr (db + PF < DB) {
-                            qq[(db + PF) % (PF + 1)] = read_tr(Qs, RST, (db + PF) * 16);
+                            qq[(db + PF) % (PF + 1)] = read_tr_t(Qs, db + PF);
                             SCHED_DS_READ_ID(2, 70 + db);
                         }
 #pragma unroll
