@@ -1,0 +1,3 @@
+"""Alias of ``flash_multi_token_attention_amd.head_conv_attn.bwd_dk_dv`` under the reference's module path."""
+from flash_multi_token_attention_amd.head_conv_attn.bwd_dk_dv import *  # noqa: F401,F403
+from flash_multi_token_attention_amd.head_conv_attn.bwd_dk_dv import __all__  # noqa: F401

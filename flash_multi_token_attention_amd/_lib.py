@@ -39,8 +39,18 @@ class KvLayout(C.Structure):
     ]
 
 
+class HeadmixDesc(C.Structure):
+    """struct convattn_headmix_desc of include/convattn.h."""
+    _fields_ = [
+        ("B", C.c_int32), ("H", C.c_int32), ("N", C.c_int32), ("d", C.c_int32),
+        ("scale", C.c_float), ("causal", C.c_int32),
+        ("in_dtype", C.c_int32), ("out_dtype", C.c_int32),
+    ]
+
+
 _P = C.c_void_p
 _D = C.POINTER(Desc)
+_HD = C.POINTER(HeadmixDesc)
 _SIGNATURES = {
     "convattn_version": (C.c_int, []),
     "convattn_strerror": (C.c_char_p, [C.c_int]),
@@ -64,6 +74,11 @@ _SIGNATURES = {
     "convattn_decode_combine": (C.c_int, [_D] + [_P] * 7),
     "convattn_decode_noalloc_bytes": (C.c_size_t, [_D]),
     "convattn_decode_noalloc": (C.c_int, [_D] + [_P] * 4 + [C.c_longlong] * 2 + [_P] * 4),
+    "convattn_headmix_validate": (C.c_int, [_HD]),
+    "convattn_headmix_fwd": (C.c_int, [_HD] + [_P] * 8),
+    "convattn_headmix_bwd_workspace_bytes": (C.c_size_t, [_HD]),
+    "convattn_headmix_bwd_dq_dw": (C.c_int, [_HD] + [_P] * 12),
+    "convattn_headmix_bwd_dkdv": (C.c_int, [_HD] + [_P] * 12),
 }
 EXPORTS = tuple(_SIGNATURES)
 

@@ -42,6 +42,7 @@ UNITS = [
     ("bwd_chain_mfma.hip", "bwd_chain_mfma_qw", ["-DCONVATTN_CHAIN_UNIT=2"]),
     ("bwd_dq_rows.hip", "bwd_dq_rows", []),
     ("decode_stream.hip", "decode_stream", []),
+    ("headmix_attn.hip", "headmix_attn", []),
 ]
 SOURCES = sorted({u[0] for u in UNITS})
 

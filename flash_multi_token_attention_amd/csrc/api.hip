@@ -117,6 +117,7 @@ const char *convattn_strerror(int code) {
         case CONVATTN_ERR_LDS: return "convolution window too large for the 160 KB of LDS at this head dimension";
         case CONVATTN_ERR_TOO_LARGE: return "batch or head count too large for one launch";
         case CONVATTN_ERR_KV_LAYOUT: return "KV layout rejected: H must be a multiple of H_kv, page_size a power of two >= 16, strides multiples of 8 that cover a page / a sequence, the block table long enough, and the descriptor one of the streaming decode kernel (bf16, d 64 or 128, c_k <= 17)";
+        case CONVATTN_ERR_HEADMIX: return "head-mixing attention: n_heads must be 16 or 32, d_model 32, 64 or 128, inputs bf16";
         case CONVATTN_ERR_SCRATCH: return "the split partials of this decode step do not fit the library's built-in scratch (convattn_decode_noalloc): use fewer splits or convattn_decode";
         default: break;
     }
@@ -422,6 +423,86 @@ int convattn_decode_combine(const convattn_desc *desc, const float *o_part, cons
     REQUIRE_PTR(o); REQUIRE_PTR(m); REQUIRE_PTR(l);
     return (int)decode_combine(p, desc->out_dtype, o_part, m_part, l_part, o, m, l,
                                static_cast<hipStream_t>(stream));
+}
+
+// ---- head-mixing attention ----
+static int headmix_check(const convattn_headmix_desc *d) {
+    if (!d) return CONVATTN_ERR_NULL;
+    if (d->B <= 0 || d->N <= 0) return CONVATTN_ERR_SHAPE;
+    if ((d->H != 16 && d->H != 32) || (d->d != 32 && d->d != 64 && d->d != 128)) return CONVATTN_ERR_HEADMIX;
+    if (d->in_dtype != CONVATTN_BF16) return CONVATTN_ERR_HEADMIX;
+    if (d->out_dtype != CONVATTN_BF16 && d->out_dtype != CONVATTN_F32) return CONVATTN_ERR_DTYPE;
+    if (!(d->scale == d->scale) || d->scale - d->scale != 0.f) return CONVATTN_ERR_SCALE;
+    if ((long long)d->B > 65535) return CONVATTN_ERR_TOO_LARGE;
+    return 0;
+}
+struct HeadmixWs {
+    size_t stat_bytes, part_off, total;
+};
+static HeadmixWs headmix_ws(const convattn_headmix_desc *d) {
+    HeadmixWs w;
+    w.stat_bytes = align256((size_t)d->B * d->H * d->N * sizeof(float));
+    w.part_off = 2 * w.stat_bytes;
+    w.total = w.part_off + align256((size_t)d->B * headmix_row_tiles(d->N) * d->H * d->H * sizeof(float));
+    return w;
+}
+// D = rowsum(dO o O) and LSE = M + log L of every row into the workspace
+static int headmix_prepare(const convattn_headmix_desc *d, const void *o, const void *d_o, const float *l, const float *m,
+                           void *workspace, hipStream_t s) {
+    Problem p{};
+    p.B = d->B; p.H = d->H; p.Nq = p.Nk = d->N; p.d = d->d;
+    float *Dl = static_cast<float *>(workspace);
+    float *lse = reinterpret_cast<float *>(static_cast<unsigned char *>(workspace) + headmix_ws(d).stat_bytes);
+    return (int)bwd_preprocess(p, d->in_dtype, d->out_dtype, o, d_o, m, l, Dl, lse, s);
+}
+
+int convattn_headmix_validate(const convattn_headmix_desc *desc) { return headmix_check(desc); }
+
+int convattn_headmix_fwd(const convattn_headmix_desc *desc, const void *q, const void *k, const void *v,
+                         const float *w, void *o, float *l, float *m, void *stream) {
+    int rc = headmix_check(desc);
+    if (rc) return rc;
+    REQUIRE_PTR(q); REQUIRE_PTR(k); REQUIRE_PTR(v); REQUIRE_PTR(w); REQUIRE_PTR(o); REQUIRE_PTR(l); REQUIRE_PTR(m);
+    return (int)headmix_fwd(desc->B, desc->H, desc->N, desc->d, desc->scale, desc->causal, desc->out_dtype, q, k, v, w, o,
+                            l, m, static_cast<hipStream_t>(stream));
+}
+
+size_t convattn_headmix_bwd_workspace_bytes(const convattn_headmix_desc *desc) {
+    return headmix_check(desc) ? 0 : headmix_ws(desc).total;
+}
+
+int convattn_headmix_bwd_dq_dw(const convattn_headmix_desc *desc, const void *q, const void *k, const void *v,
+                               const float *w, const void *o, const void *d_o, const float *l, const float *m,
+                               void *workspace, float *dq, float *dw, void *stream) {
+    int rc = headmix_check(desc);
+    if (rc) return rc;
+    REQUIRE_PTR(q); REQUIRE_PTR(k); REQUIRE_PTR(v); REQUIRE_PTR(w); REQUIRE_PTR(o); REQUIRE_PTR(d_o);
+    REQUIRE_PTR(l); REQUIRE_PTR(m); REQUIRE_PTR(workspace); REQUIRE_PTR(dq); REQUIRE_PTR(dw);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    rc = headmix_prepare(desc, o, d_o, l, m, workspace, s);
+    if (rc) return rc;
+    const HeadmixWs ws = headmix_ws(desc);
+    unsigned char *base = static_cast<unsigned char *>(workspace);
+    return (int)headmix_bwd_dq_dw(desc->B, desc->H, desc->N, desc->d, desc->scale, desc->causal, q, k, v, w, d_o,
+                                  reinterpret_cast<const float *>(base + ws.stat_bytes), reinterpret_cast<const float *>(base),
+                                  dq, reinterpret_cast<float *>(base + ws.part_off), dw, s);
+}
+
+int convattn_headmix_bwd_dkdv(const convattn_headmix_desc *desc, const void *q, const void *k, const void *v,
+                              const float *w, const void *o, const void *d_o, const float *l, const float *m,
+                              void *workspace, float *dk, float *dv, void *stream) {
+    int rc = headmix_check(desc);
+    if (rc) return rc;
+    REQUIRE_PTR(q); REQUIRE_PTR(k); REQUIRE_PTR(v); REQUIRE_PTR(w); REQUIRE_PTR(o); REQUIRE_PTR(d_o);
+    REQUIRE_PTR(l); REQUIRE_PTR(m); REQUIRE_PTR(workspace); REQUIRE_PTR(dk); REQUIRE_PTR(dv);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    rc = headmix_prepare(desc, o, d_o, l, m, workspace, s);
+    if (rc) return rc;
+    const HeadmixWs ws = headmix_ws(desc);
+    unsigned char *base = static_cast<unsigned char *>(workspace);
+    return (int)headmix_bwd_dkdv(desc->B, desc->H, desc->N, desc->d, desc->scale, desc->causal, q, k, v, w, d_o,
+                                 reinterpret_cast<const float *>(base + ws.stat_bytes), reinterpret_cast<const float *>(base),
+                                 dk, dv, s);
 }
 
 }  // extern "C"

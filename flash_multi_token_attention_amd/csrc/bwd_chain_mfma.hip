@@ -252,7 +252,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
     float *__restrict__ dW_part = args.dW_part;
     const int n_rt = args.n_rt;
     using Lds = ChainLds<D, CQT>;
-    constexpr int KS = D / 32, DB = D / 16, CPR = D / 8, RST = Lds::RST;
+    constexpr int KS = D / 32, DB = D / 16;
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
     const int tid = threadIdx.x;

@@ -76,4 +76,15 @@ hipError_t dw_reduce(const Problem &p, int n_tiles, const float *dw_part, float 
 hipError_t decode_combine(const Problem &p, int out_dt, const float *o_part, const float *m_part,
                           const float *l_part, void *o, float *m, float *l, hipStream_t s);
 
+// ---- head-mixing attention (headmix_attn.hip) ----
+hipError_t headmix_fwd(int B, int H, int N, int d, float scale, int causal, int out_dt, const void *q, const void *k,
+                       const void *v, const float *w, void *o, float *l, float *m, hipStream_t s);
+hipError_t headmix_bwd_dq_dw(int B, int H, int N, int d, float scale, int causal, const void *q, const void *k,
+                             const void *v, const float *w, const void *d_o, const float *lse, const float *Dl, float *dq,
+                             float *dw_part, float *dw, hipStream_t s);
+hipError_t headmix_bwd_dkdv(int B, int H, int N, int d, float scale, int causal, const void *q, const void *k,
+                            const void *v, const float *w, const void *d_o, const float *lse, const float *Dl, float *dk,
+                            float *dv, hipStream_t s);
+int headmix_row_tiles(int N);
+
 }  // namespace convattn

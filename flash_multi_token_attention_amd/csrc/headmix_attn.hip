@@ -1,0 +1,568 @@
+// Head-mixing attention ("head_conv_attn" of the reference) on fp32 MFMA (gfx950).
+//
+//   S_h' = scale Q_h' K_h'^T,   Z_h = sum_h' w[h][h'] S_h',   P_h = softmax_j(Z_h + causal mask),
+//   O_h = P_h V_h.
+// The heads of a (batch, row, key) triple are coupled before the softmax, so a workgroup handles
+// ALL heads of 16 query rows (forward, dQ + dW) or of 16 keys (dK / dV) of one batch entry and
+// walks the other axis in tiles of 16.  Every product runs on v_mfma_f32_16x16x4_f32 with fp32
+// accumulation; bf16 inputs are widened to fp32 operands, scores and probabilities stay fp32.
+//
+// Per 16 x 16 tile (8 waves):
+//   1. waves take heads: S_h' from Q / K row fragments read straight from global memory
+//      (the contraction index is permuted so that one 16-byte load feeds 8 MFMA steps)  -> LDS;
+//   2. waves take rows: Z = W S as a product over the head index (A = W, B = the scores of one
+//      row across the heads), mask, softmax (or P = exp(Z - LSE) in the backward)        -> LDS;
+//   3. waves take heads again: P V (forward), dP = dO V^T, dV += P^T dO, dZ = P (dP - D);
+//   4. (backward) waves take rows: dW += dZ S^T over the tile's elements, dS = W^T dZ in place;
+//   5. (backward) waves take heads: dQ += dS K or dK += dS^T Q.
+// Operands that are read along their rows (V, K, Q, dO as the right-hand side) are staged per wave
+// in a 16-row bf16 tile.  Accumulators (O, dQ, dK / dV of up to 4 heads per wave) stay in registers
+// for the whole loop; nothing is accumulated through global memory and there are no atomics
+// (the reference's Triton kernels read-modify-write O per key block, fwd_kernel.py:214-250, and add
+// dW with tl.atomic_add, bwd_dq_dw.py:370): dW partials are summed in a fixed order.
+#include "common.hpp"
+
+namespace convattn {
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int HW = 8;            // waves per workgroup
+constexpr int HT = 16;           // rows / keys per tile
+constexpr int SST = 20;          // floats per row of a score tile in LDS
+constexpr int HST = HT * SST + 16;   // floats per head of a score array (== 16 mod 32: see the reads in phase 2)
+
+__device__ __forceinline__ f32x4 mfma4(float a, float b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+}
+
+struct HmArgs {
+    int B, H, N, causal;
+    float scale;
+};
+
+template <int H, int D> struct HmLds {
+    static constexpr int WST = H + 4;                       // floats per row of W
+    static constexpr int XST = D * 2 + 32;                  // bytes per row of a staged bf16 tile
+    static constexpr int arr_bytes = H * HST * 4;           // one score array
+    static constexpr int s_off = 0;                         // S (forward: then P in place)
+    static constexpr int p_off = s_off + arr_bytes;         // backward: P, then dZ, then dS
+    static constexpr int w_off = p_off + arr_bytes;
+    static constexpr int x_off = w_off + H * WST * 4;       // per-wave staging tiles
+    static constexpr int stat_off = x_off + HW * HT * XST;  // three [H][16] float arrays
+    static constexpr int total = stat_off + 3 * H * HT * 4;
+};
+
+// 8 consecutive bf16 of row `row` at column `col` as floats; zeros for rows outside [0, N)
+template <int D>
+__device__ __forceinline__ void row_frag(const bf16_t *__restrict__ base, int row, int N, int col, float (&f)[8]) {
+    u32x4 raw = {0u, 0u, 0u, 0u};
+    if (row >= 0 && row < N) raw = *reinterpret_cast<const u32x4 *>(base + (size_t)row * D + col);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        f[2 * i] = __uint_as_float(raw[i] << 16);
+        f[2 * i + 1] = __uint_as_float(raw[i] & 0xffff0000u);
+    }
+}
+
+// C[16 x 16] (lane (g, n): rows 4g .. 4g+3, column n) = X Y^T for two row-major bf16 matrices in global
+// memory: rows x0 + n of X against rows y0 + n of Y.  Contraction index of lane group g at step s of
+// block blk: 32 blk + 8 g + s, the same for both operands.
+template <int D>
+__device__ __forceinline__ f32x4 rows_times_rows(const bf16_t *__restrict__ X, int x0, const bf16_t *__restrict__ Y,
+                                                 int y0, int N, int g, int n) {
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int blk = 0; blk < D / 32; ++blk) {
+        float a[8], b[8];
+        row_frag<D>(X, x0 + n, N, blk * 32 + 8 * g, a);
+        row_frag<D>(Y, y0 + n, N, blk * 32 + 8 * g, b);
+#pragma unroll
+        for (int s = 0; s < 8; ++s) acc = mfma4(a[s], b[s], acc);
+    }
+    return acc;
+}
+
+// Rows r0 .. r0+15 of a [N][D] bf16 matrix into this wave's staging tile (zeros outside [0, N)).
+template <int D>
+__device__ __forceinline__ void stage_rows(unsigned char *xt, int xst, const bf16_t *__restrict__ base, int r0, int N,
+                                           int lane) {
+    constexpr int CPR = D / 8;
+#pragma unroll
+    for (int c = lane; c < HT * CPR; c += 64) {
+        const int row = c / CPR, cc = c % CPR;
+        u32x4 raw = {0u, 0u, 0u, 0u};
+        if (r0 + row >= 0 && r0 + row < N) raw = *reinterpret_cast<const u32x4 *>(base + (size_t)(r0 + row) * D + cc * 8);
+        *reinterpret_cast<u32x4 *>(xt + row * xst + cc * 16) = raw;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+__device__ __forceinline__ float staged(const unsigned char *xt, int xst, int row, int col) {
+    return __uint_as_float((unsigned int)*reinterpret_cast<const unsigned short *>(xt + row * xst + col * 2) << 16);
+}
+
+// acc[db] (lane (g, n): tile row 4g .. 4g+3, head-dim column 16 db + n) += A X, with A a 16 x 16 fp32 tile
+// in LDS (element (m, k) at a[m * a_rs + k * a_cs]) and X this wave's staged 16-row tile.
+template <int D>
+__device__ __forceinline__ void tile_times_staged(f32x4 (&acc)[D / 16], const float *a, int a_rs, int a_cs,
+                                                  const unsigned char *xt, int xst, int g, int n) {
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+        const float av = a[n * a_rs + (4 * s + g) * a_cs];
+#pragma unroll
+        for (int db = 0; db < D / 16; ++db) acc[db] = mfma4(av, staged(xt, xst, 4 * s + g, db * 16 + n), acc[db]);
+    }
+}
+
+// Max / sum over the 16 lanes of a lane group (all of them get the result).
+__device__ __forceinline__ float row16_max(float v) {
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 16));
+    return v;
+}
+__device__ __forceinline__ float row16_sum(float v) {
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, 16);
+    return v;
+}
+
+template <int H> __device__ __forceinline__ void load_w(float *Wl, int wst, const float *__restrict__ W, int tid) {
+    for (int i = tid; i < H * H; i += HW * 64) Wl[(i / H) * wst + (i % H)] = W[i];
+}
+
+// Phase 1: scaled scores of the heads wave, wave + 8, ... for rows i0.. and keys j0.. -> S[h'][i][j]
+template <int H, int D>
+__device__ __forceinline__ void scores_phase(float *S, const HmArgs &a, const bf16_t *__restrict__ Qb,
+                                             const bf16_t *__restrict__ Kb, int i0, int j0, int wave, int g, int n) {
+#pragma unroll
+    for (int t = 0; t < H / HW; ++t) {
+        const int h = wave + t * HW;
+        const f32x4 acc = rows_times_rows<D>(Qb + (size_t)h * a.N * D, i0, Kb + (size_t)h * a.N * D, j0, a.N, g, n);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) S[h * HST + (4 * g + r) * SST + n] = acc[r] * a.scale;
+    }
+}
+
+// Z (or its transpose-weighted counterpart) of tile row i for every head: out[hb] (lane (g, n): head
+// 16 hb + 4g + r, key n) = sum_k Wt(16 hb + m, k) X[k][i][n], Wt(m, k) = Wl[m * w_rs + k * w_cs].
+template <int H>
+__device__ __forceinline__ void mix_row(f32x4 (&out)[H / 16], const float *Wl, int w_rs, int w_cs, const float *X,
+                                        int i, int g, int n) {
+#pragma unroll
+    for (int hb = 0; hb < H / 16; ++hb) out[hb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int k0 = 0; k0 < H; k0 += 4) {
+        const float b = X[(k0 + g) * HST + i * SST + n];
+#pragma unroll
+        for (int hb = 0; hb < H / 16; ++hb) out[hb] = mfma4(Wl[(hb * 16 + n) * w_rs + (k0 + g) * w_cs], b, out[hb]);
+    }
+}
+
+// ------------------------------------------------------------------ forward
+template <int H, int D, typename TO>
+__global__ __launch_bounds__(HW * 64) void headmix_fwd_kernel(HmArgs a, const bf16_t *__restrict__ Q,
+                                                              const bf16_t *__restrict__ K, const bf16_t *__restrict__ V,
+                                                              const float *__restrict__ W, TO *__restrict__ O,
+                                                              float *__restrict__ L, float *__restrict__ M) {
+    using Lds = HmLds<H, D>;
+    constexpr int DB = D / 16, HPW = H / HW, RPW = HT / HW;  // heads and rows per wave
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    float *S = reinterpret_cast<float *>(smem + Lds::s_off);
+    float *Wl = reinterpret_cast<float *>(smem + Lds::w_off);
+    float *al = reinterpret_cast<float *>(smem + Lds::stat_off);   // alpha[h][i], at the end 1 / l
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, g = lane >> 4, n = lane & 15;
+    unsigned char *xt = smem + Lds::x_off + wave * HT * Lds::XST;
+    const int b = blockIdx.y, i0 = (gridDim.x - 1 - blockIdx.x) * HT;   // longest (causal) tiles first
+    const size_t bo = (size_t)b * a.H * a.N * D;
+    const bf16_t *Qb = Q + bo, *Kb = K + bo, *Vb = V + bo;
+
+    load_w<H>(Wl, Lds::WST, W, tid);
+    f32x4 acc_o[HPW][DB];
+#pragma unroll
+    for (int t = 0; t < HPW; ++t)
+#pragma unroll
+        for (int db = 0; db < DB; ++db) acc_o[t][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    // softmax state of this wave's rows (phase 2): [row][head block][r], the same in the 16 lanes of a group
+    float m_run[RPW][H / 16][4], l_run[RPW][H / 16][4];
+#pragma unroll
+    for (int rl = 0; rl < RPW; ++rl)
+#pragma unroll
+        for (int hb = 0; hb < H / 16; ++hb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) { m_run[rl][hb][r] = kNegInf; l_run[rl][hb][r] = 0.f; }
+
+    const int j_end = a.causal ? min(a.N, i0 + HT) : a.N;
+    for (int j0 = 0; j0 < j_end; j0 += HT) {
+        __syncthreads();   // the last tile's P has been used (and, first, W is in place)
+        scores_phase<H, D>(S, a, Qb, Kb, i0, j0, wave, g, n);
+        __syncthreads();
+#pragma unroll
+        for (int rl = 0; rl < RPW; ++rl) {
+            const int i = wave * RPW + rl;
+            f32x4 z[H / 16];
+            mix_row<H>(z, Wl, Lds::WST, 1, S, i, g, n);
+            const bool visible = j0 + n < a.N && !(a.causal && j0 + n > i0 + i);
+#pragma unroll
+            for (int hb = 0; hb < H / 16; ++hb)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float zv = visible ? z[hb][r] : kNegInf;
+                    const float m_old = m_run[rl][hb][r];
+                    const float m_new = fmaxf(m_old, row16_max(zv));
+                    const float pv = m_new == kNegInf ? 0.f : __expf(zv - m_new);
+                    const float alpha = m_old == kNegInf ? 0.f : __expf(m_old - m_new);
+                    l_run[rl][hb][r] = l_run[rl][hb][r] * alpha + row16_sum(pv);
+                    m_run[rl][hb][r] = m_new;
+                    const int h = hb * 16 + 4 * g + r;
+                    S[h * HST + i * SST + n] = pv;   // P in place: this wave alone reads and writes row i
+                    if (n == 0) al[h * HT + i] = alpha;
+                }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int t = 0; t < HPW; ++t) {
+            const int h = wave + t * HW;
+            stage_rows<D>(xt, Lds::XST, Vb + (size_t)h * a.N * D, j0, a.N, lane);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float alpha = al[h * HT + 4 * g + r];
+#pragma unroll
+                for (int db = 0; db < DB; ++db) acc_o[t][db][r] *= alpha;
+            }
+            tile_times_staged<D>(acc_o[t], S + h * HST, SST, 1, xt, Lds::XST, g, n);
+            __builtin_amdgcn_wave_barrier();
+        }
+    }
+    // row sums and maxima from the row waves to the head waves
+    __syncthreads();
+    float *lf = al, *mf = al + H * HT;
+#pragma unroll
+    for (int rl = 0; rl < RPW; ++rl)
+#pragma unroll
+        for (int hb = 0; hb < H / 16; ++hb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (n == 0) {
+                    const int h = hb * 16 + 4 * g + r, i = wave * RPW + rl;
+                    lf[h * HT + i] = l_run[rl][hb][r];
+                    mf[h * HT + i] = m_run[rl][hb][r];
+                }
+    __syncthreads();
+#pragma unroll
+    for (int t = 0; t < HPW; ++t) {
+        const int h = wave + t * HW;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int i = i0 + 4 * g + r;
+            if (i < a.N) {
+                const float inv = 1.f / lf[h * HT + 4 * g + r];
+                TO *orow = O + bo + ((size_t)h * a.N + i) * D;
+#pragma unroll
+                for (int db = 0; db < DB; ++db) orow[db * 16 + n] = from_f32<TO>(acc_o[t][db][r] * inv);
+            }
+        }
+    }
+    for (int idx = tid; idx < H * HT; idx += HW * 64) {
+        const int h = idx / HT, i = i0 + idx % HT;
+        if (i < a.N) {
+            L[((size_t)b * a.H + h) * a.N + i] = lf[idx];
+            M[((size_t)b * a.H + h) * a.N + i] = mf[idx];
+        }
+    }
+}
+
+// ----------------------------------------------------------------- backward
+// WHAT = 0: dQ and the dW partial of a row tile (grid: row tiles x batch);
+// WHAT = 1: dK and dV of 16 heads (blockIdx.z) of a key tile (grid: key tiles x batch x H / 16).
+template <int H, int D, int WHAT>
+__global__ __launch_bounds__(HW * 64) void headmix_bwd_kernel(HmArgs a, const bf16_t *__restrict__ Q,
+                                                              const bf16_t *__restrict__ K, const bf16_t *__restrict__ V,
+                                                              const float *__restrict__ W, const bf16_t *__restrict__ dO,
+                                                              const float *__restrict__ LSE, const float *__restrict__ Dl,
+                                                              float *__restrict__ out0, float *__restrict__ out1) {
+    using Lds = HmLds<H, D>;
+    constexpr int DB = D / 16, HPW = H / HW, RPW = HT / HW, HB = H / 16;
+    constexpr int OPW = 2;   // WHAT = 1: heads of this workgroup's 16 that a wave accumulates for
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    float *S = reinterpret_cast<float *>(smem + Lds::s_off);
+    float *P = reinterpret_cast<float *>(smem + Lds::p_off);
+    float *Wl = reinterpret_cast<float *>(smem + Lds::w_off);
+    float *lse_s = reinterpret_cast<float *>(smem + Lds::stat_off), *d_s = lse_s + H * HT;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, g = lane >> 4, n = lane & 15;
+    unsigned char *xt = smem + Lds::x_off + wave * HT * Lds::XST;
+    const int b = blockIdx.y, hs = blockIdx.z;
+    const size_t bo = (size_t)b * a.H * a.N * D;
+    const bf16_t *Qb = Q + bo, *Kb = K + bo, *Vb = V + bo, *Gb = dO + bo;
+    const int fixed0 = (WHAT == 0 ? gridDim.x - 1 - blockIdx.x : blockIdx.x) * HT;   // own row tile (0) or key tile (1)
+
+    load_w<H>(Wl, Lds::WST, W, tid);
+    constexpr int NACC = WHAT == 0 ? HPW : 2 * OPW;
+    f32x4 acc[NACC][DB];   // WHAT 0: dQ of the wave's heads; WHAT 1: dK then dV of its output heads
+#pragma unroll
+    for (int t = 0; t < NACC; ++t)
+#pragma unroll
+        for (int db = 0; db < DB; ++db) acc[t][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    f32x4 acc_w[HB][HB];
+#pragma unroll
+    for (int x = 0; x < HB; ++x)
+#pragma unroll
+        for (int y = 0; y < HB; ++y) acc_w[x][y] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    auto load_stats = [&](int i0) {
+        for (int idx = tid; idx < H * HT; idx += HW * 64) {
+            const int h = idx / HT, i = i0 + idx % HT;
+            const size_t at = ((size_t)b * a.H + h) * a.N + i;
+            lse_s[idx] = i < a.N ? LSE[at] : 0.f;
+            d_s[idx] = i < a.N ? Dl[at] : 0.f;
+        }
+    };
+    if (WHAT == 0) load_stats(fixed0);
+
+    // the other axis: keys up to the diagonal (dQ) or rows from the diagonal on (dK / dV)
+    const int lo = WHAT == 0 ? 0 : (a.causal ? fixed0 : 0);
+    const int hi = WHAT == 0 ? (a.causal ? min(a.N, fixed0 + HT) : a.N) : a.N;
+    for (int o0 = lo; o0 < hi; o0 += HT) {
+        const int i0 = WHAT == 0 ? fixed0 : o0, j0 = WHAT == 0 ? o0 : fixed0;
+        __syncthreads();   // the last tile's dS has been used (and, first, W and the statistics are in place)
+        if (WHAT == 1) load_stats(i0);
+        scores_phase<H, D>(S, a, Qb, Kb, i0, j0, wave, g, n);
+        __syncthreads();
+        // ---- P = exp(Z - LSE), rows of this wave ----
+#pragma unroll
+        for (int rl = 0; rl < RPW; ++rl) {
+            const int i = wave * RPW + rl;
+            f32x4 z[HB];
+            mix_row<H>(z, Wl, Lds::WST, 1, S, i, g, n);
+            const bool visible = i0 + i < a.N && j0 + n < a.N && !(a.causal && j0 + n > i0 + i);
+#pragma unroll
+            for (int hb = 0; hb < HB; ++hb)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int h = hb * 16 + 4 * g + r;
+                    P[h * HST + i * SST + n] = visible ? __expf(z[hb][r] - lse_s[h * HT + i]) : 0.f;
+                }
+        }
+        __syncthreads();
+        // ---- heads of this wave: dP = dO V^T, (dV += P^T dO), dZ = P (dP - D) in place of P ----
+#pragma unroll
+        for (int t = 0; t < HPW; ++t) {
+            const int h = wave + t * HW;
+            const f32x4 dp = rows_times_rows<D>(Gb + (size_t)h * a.N * D, i0, Vb + (size_t)h * a.N * D, j0, a.N, g, n);
+            if constexpr (WHAT == 1) {
+                // heads wave + 8t of the half hs: t = 2 hs, 2 hs + 1 (H = 32) or t = 0, 1 (H = 16)
+                if (h / 16 == hs) {
+                    stage_rows<D>(xt, Lds::XST, Gb + (size_t)h * a.N * D, i0, a.N, lane);
+                    // dV[j][:] += sum_i P[i][j] dO[i][:]: A(m = j, k = i)
+                    tile_times_staged<D>(acc[OPW + (t % OPW)], P + h * HST, 1, SST, xt, Lds::XST, g, n);
+                    __builtin_amdgcn_wave_barrier();
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float *pp = P + h * HST + (4 * g + r) * SST + n;
+                *pp = *pp * (dp[r] - d_s[h * HT + 4 * g + r]);
+            }
+        }
+        __syncthreads();
+        // ---- rows of this wave: dW += dZ S^T over its elements, then dS = scale W^T dZ in place ----
+#pragma unroll
+        for (int rl = 0; rl < RPW; ++rl) {
+            const int i = wave * RPW + rl;
+            if constexpr (WHAT == 0) {
+#pragma unroll
+                for (int s = 0; s < 4; ++s)
+#pragma unroll
+                    for (int x = 0; x < HB; ++x) {
+                        const float av = P[(x * 16 + n) * HST + i * SST + 4 * s + g];
+#pragma unroll
+                        for (int y = 0; y < HB; ++y)
+                            acc_w[x][y] = mfma4(av, S[(y * 16 + n) * HST + i * SST + 4 * s + g], acc_w[x][y]);
+                    }
+            }
+            f32x4 ds[HB];
+            mix_row<H>(ds, Wl, 1, Lds::WST, P, i, g, n);   // W^T: element (m = h', k = h) is W[h][h']
+#pragma unroll
+            for (int hb = 0; hb < HB; ++hb)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) P[(hb * 16 + 4 * g + r) * HST + i * SST + n] = ds[hb][r] * a.scale;
+        }
+        __syncthreads();
+        // ---- heads of this wave: dQ += dS K, or dK += dS^T Q ----
+        if constexpr (WHAT == 0) {
+#pragma unroll
+            for (int t = 0; t < HPW; ++t) {
+                const int h = wave + t * HW;
+                stage_rows<D>(xt, Lds::XST, Kb + (size_t)h * a.N * D, j0, a.N, lane);
+                tile_times_staged<D>(acc[t], P + h * HST, SST, 1, xt, Lds::XST, g, n);
+                __builtin_amdgcn_wave_barrier();
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < HPW; ++t) {
+                const int h = wave + t * HW;
+                if (h / 16 == hs) {
+                    stage_rows<D>(xt, Lds::XST, Qb + (size_t)h * a.N * D, i0, a.N, lane);
+                    tile_times_staged<D>(acc[t % OPW], P + h * HST, 1, SST, xt, Lds::XST, g, n);
+                    __builtin_amdgcn_wave_barrier();
+                }
+            }
+        }
+    }
+
+    // ---- stores: lane (g, n) holds tile rows 4g .. 4g+3 at head-dim columns 16 db + n ----
+    if constexpr (WHAT == 0) {
+#pragma unroll
+        for (int t = 0; t < HPW; ++t) {
+            const int h = wave + t * HW;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int i = fixed0 + 4 * g + r;
+                if (i < a.N) {
+                    float *row = out0 + bo + ((size_t)h * a.N + i) * D;
+#pragma unroll
+                    for (int db = 0; db < DB; ++db) row[db * 16 + n] = acc[t][db][r];
+                }
+            }
+        }
+        // dW partial of the workgroup: the eight waves' accumulators added in wave order
+        __syncthreads();
+        float *red = S;   // [wave][h][h']
+#pragma unroll
+        for (int x = 0; x < HB; ++x)
+#pragma unroll
+            for (int y = 0; y < HB; ++y)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) red[(wave * H + x * 16 + 4 * g + r) * H + y * 16 + n] = acc_w[x][y][r];
+        __syncthreads();
+        float *part = out1 + ((size_t)b * gridDim.x + blockIdx.x) * H * H;
+        for (int idx = tid; idx < H * H; idx += HW * 64) {
+            float s = 0.f;
+#pragma unroll
+            for (int w8 = 0; w8 < HW; ++w8) s += red[w8 * H * H + idx];
+            part[idx] = s;
+        }
+    } else {
+#pragma unroll
+        for (int t = 0; t < HPW; ++t) {
+            const int h = wave + t * HW;
+            if (h / 16 != hs) continue;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int j = fixed0 + 4 * g + r;
+                if (j < a.N) {
+                    float *krow = out0 + bo + ((size_t)h * a.N + j) * D, *vrow = out1 + bo + ((size_t)h * a.N + j) * D;
+#pragma unroll
+                    for (int db = 0; db < DB; ++db) {
+                        krow[db * 16 + n] = acc[t % OPW][db][r];
+                        vrow[db * 16 + n] = acc[OPW + (t % OPW)][db][r];
+                    }
+                }
+            }
+        }
+    }
+}
+
+// dW[h][h'] = sum of the partials in index order
+__global__ void headmix_dw_reduce_kernel(int n_part, int hh, const float *__restrict__ part, float *__restrict__ dW) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= hh) return;
+    float s = 0.f;
+    for (int p = 0; p < n_part; ++p) s += part[(size_t)p * hh + idx];
+    dW[idx] = s;
+}
+
+template <auto Kern> hipError_t allow_lds(int bytes) {
+    static bool done[64] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 64 && done[dev]) return hipSuccess;
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(Kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess && dev < 64) done[dev] = true;
+    return e;
+}
+
+template <int H, int D>
+hipError_t launch_fwd(const HmArgs &a, int out_dt, const void *q, const void *k, const void *v, const float *w, void *o,
+                      float *l, float *m, hipStream_t s) {
+    constexpr int lds = HmLds<H, D>::total;
+    static_assert(lds <= 160 * 1024, "LDS budget");
+    dim3 grid((a.N + HT - 1) / HT, a.B);
+    if (out_dt == CONVATTN_BF16) {
+        hipError_t e = allow_lds<headmix_fwd_kernel<H, D, bf16_t>>(lds);
+        if (e != hipSuccess) return e;
+        headmix_fwd_kernel<H, D, bf16_t><<<grid, HW * 64, lds, s>>>(a, (const bf16_t *)q, (const bf16_t *)k,
+                                                                     (const bf16_t *)v, w, (bf16_t *)o, l, m);
+    } else {
+        hipError_t e = allow_lds<headmix_fwd_kernel<H, D, float>>(lds);
+        if (e != hipSuccess) return e;
+        headmix_fwd_kernel<H, D, float><<<grid, HW * 64, lds, s>>>(a, (const bf16_t *)q, (const bf16_t *)k,
+                                                                   (const bf16_t *)v, w, (float *)o, l, m);
+    }
+    return hipGetLastError();
+}
+
+template <int H, int D, int WHAT>
+hipError_t launch_bwd(const HmArgs &a, const void *q, const void *k, const void *v, const float *w, const void *d_o,
+                      const float *lse, const float *Dl, float *out0, float *out1, hipStream_t s) {
+    constexpr int lds = HmLds<H, D>::total;
+    static_assert(lds <= 160 * 1024, "LDS budget");
+    static_assert(HW * H * H * 4 <= HmLds<H, D>::arr_bytes, "room for the dW accumulators of the waves");
+    hipError_t e = allow_lds<headmix_bwd_kernel<H, D, WHAT>>(lds);
+    if (e != hipSuccess) return e;
+    dim3 grid((a.N + HT - 1) / HT, a.B, WHAT == 1 ? H / 16 : 1);
+    headmix_bwd_kernel<H, D, WHAT><<<grid, HW * 64, lds, s>>>(a, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v,
+                                                              w, (const bf16_t *)d_o, lse, Dl, out0, out1);
+    return hipGetLastError();
+}
+
+#define HM_DISPATCH(CALL)                                    \
+    do {                                                     \
+        if (a.H == 16 && d == 32) return CALL(16, 32);       \
+        if (a.H == 16 && d == 64) return CALL(16, 64);       \
+        if (a.H == 16 && d == 128) return CALL(16, 128);     \
+        if (a.H == 32 && d == 32) return CALL(32, 32);       \
+        if (a.H == 32 && d == 64) return CALL(32, 64);       \
+        if (a.H == 32 && d == 128) return CALL(32, 128);     \
+        return hipErrorInvalidValue;                         \
+    } while (0)
+
+}  // namespace
+
+hipError_t headmix_fwd(int B, int H, int N, int d, float scale, int causal, int out_dt, const void *q, const void *k,
+                       const void *v, const float *w, void *o, float *l, float *m, hipStream_t s) {
+    const HmArgs a{B, H, N, causal, scale};
+#define CALL(HH, DD) launch_fwd<HH, DD>(a, out_dt, q, k, v, w, o, l, m, s)
+    HM_DISPATCH(CALL);
+#undef CALL
+}
+
+hipError_t headmix_bwd_dq_dw(int B, int H, int N, int d, float scale, int causal, const void *q, const void *k,
+                             const void *v, const float *w, const void *d_o, const float *lse, const float *Dl, float *dq,
+                             float *dw_part, float *dw, hipStream_t s) {
+    const HmArgs a{B, H, N, causal, scale};
+    hipError_t e = [&]() -> hipError_t {
+#define CALL(HH, DD) launch_bwd<HH, DD, 0>(a, q, k, v, w, d_o, lse, Dl, dq, dw_part, s)
+        HM_DISPATCH(CALL);
+#undef CALL
+    }();
+    if (e != hipSuccess) return e;
+    const int n_part = B * ((N + HT - 1) / HT), hh = H * H;
+    headmix_dw_reduce_kernel<<<(hh + 255) / 256, 256, 0, s>>>(n_part, hh, dw_part, dw);
+    return hipGetLastError();
+}
+
+hipError_t headmix_bwd_dkdv(int B, int H, int N, int d, float scale, int causal, const void *q, const void *k,
+                            const void *v, const float *w, const void *d_o, const float *lse, const float *Dl, float *dk,
+                            float *dv, hipStream_t s) {
+    const HmArgs a{B, H, N, causal, scale};
+#define CALL(HH, DD) launch_bwd<HH, DD, 1>(a, q, k, v, w, d_o, lse, Dl, dk, dv, s)
+    HM_DISPATCH(CALL);
+#undef CALL
+}
+
+int headmix_row_tiles(int N) { return (N + HT - 1) / HT; }
+
+}  // namespace convattn

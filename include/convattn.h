@@ -63,6 +63,7 @@ typedef enum convattn_status {
     CONVATTN_ERR_LDS = -11,        /* the window needs more LDS than a CU has */
     CONVATTN_ERR_TOO_LARGE = -12,  /* a launch dimension would overflow */
     CONVATTN_ERR_SCRATCH = -13,    /* convattn_decode_noalloc: partials larger than the built-in scratch */
+    CONVATTN_ERR_HEADMIX = -15,    /* convattn_headmix_*: H not 16 or 32, d not 32 / 64 / 128, or inputs not bf16 */
     CONVATTN_ERR_KV_LAYOUT = -14   /* convattn_decode_kv: bad KV-head count, page size, stride or table, or a
                                       descriptor outside the streaming decode kernel (bf16, d 64 / 128, c_k <= 17) */
 } convattn_status;
@@ -279,6 +280,52 @@ size_t convattn_decode_noalloc_bytes(const convattn_desc *desc);
 int convattn_decode_noalloc(const convattn_desc *desc, const void *q, const void *k, const void *v,
                             const float *w, long long kv_batch_stride, long long kv_head_stride,
                             void *o, float *m, float *l, void *stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Head-mixing attention, the reference's second variant (head_conv_attn/): the scores of all
+ * heads of a (batch, row, key) triple are mixed by a dense [H][H] matrix before the softmax,
+ *   Z[b,h] = sum_h' w[h][h'] * scale * Q[b,h'] K[b,h']^T,  P = softmax(Z + causal mask),  O = P V
+ * (head_conv_attn/head_conv_fn_pytorch.py:7-54).  q, k, v, o, d_o: dense [B,H,N,d]; w: fp32
+ * [H][H] (out head, in head); l, m: fp32 [B,H,N] with m the row maximum of Z and
+ * l = sum_j exp(Z - m), as the reference returns them.  H is 16 or 32 (fwd_kernel.py:289),
+ * d 32, 64 or 128, inputs bf16, O bf16 or fp32, gradients fp32 (bwd_dq_dw.py:381-382).
+ * ------------------------------------------------------------------------------------------ */
+typedef struct convattn_headmix_desc {
+    int32_t B, H, N, d;
+    float scale;
+    int32_t causal;
+    int32_t in_dtype;   /* CONVATTN_BF16 */
+    int32_t out_dtype;  /* dtype of O */
+} convattn_headmix_desc;
+
+/* Host-only check of a descriptor: 0 or a negative convattn_status. */
+int convattn_headmix_validate(const convattn_headmix_desc *desc);
+
+/*
+ * Forward.  Replaces head_conv_attention_forward and head_conv_attn_fwd_kernel
+ * (head_conv_attn/fwd_kernel.py:7-365): O stays in registers for the whole key loop instead of
+ * being read and written back per key block (fwd_kernel.py:214-250).
+ */
+int convattn_headmix_fwd(const convattn_headmix_desc *desc, const void *q, const void *k, const void *v,
+                         const float *w, void *o, float *l, float *m, void *stream);
+
+/* Bytes of the scratch buffer the two backward entry points need (D and LSE of every row, the dW
+ * partials of every row tile); its contents need not be initialised.  0 on a bad descriptor. */
+size_t convattn_headmix_bwd_workspace_bytes(const convattn_headmix_desc *desc);
+
+/*
+ * dQ [B,H,N,d] fp32 and dW [H][H] fp32.  Replaces head_conv_attention_bwd_dq_dw
+ * (head_conv_attn/bwd_dq_dw.py:7-470).  dW is summed over per-tile partials in a fixed order
+ * (the reference adds it with tl.atomic_add, bwd_dq_dw.py:370).
+ */
+int convattn_headmix_bwd_dq_dw(const convattn_headmix_desc *desc, const void *q, const void *k, const void *v,
+                               const float *w, const void *o, const void *d_o, const float *l, const float *m,
+                               void *workspace, float *dq, float *dw, void *stream);
+
+/* dK, dV [B,H,N,d] fp32.  Replaces head_conv_attention_bwd_dkdv (head_conv_attn/bwd_dk_dv.py:7-500). */
+int convattn_headmix_bwd_dkdv(const convattn_headmix_desc *desc, const void *q, const void *k, const void *v,
+                              const float *w, const void *o, const void *d_o, const float *l, const float *m,
+                              void *workspace, float *dk, float *dv, void *stream);
 
 #ifdef __cplusplus
 }
