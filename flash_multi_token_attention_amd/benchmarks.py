@@ -10,12 +10,17 @@ tensors (the reference's "Flash Attention" comparison line) and prints a markdow
 
     python -m flash_multi_token_attention_amd.benchmarks train  [--quick] [--md FILE]
     python -m flash_multi_token_attention_amd.benchmarks decode [--quick] [--md FILE]
+    python -m flash_multi_token_attention_amd.benchmarks head_conv [--quick] [--md FILE]
     python -m flash_multi_token_attention_amd.benchmarks plot --train FILE [--decode FILE] [--out DIR]
 
 ``plot`` draws the figures of the reference's plot scripts from such tables
 (scripts/plot_benchmark_seq_len.py:233-310: speed relative to the comparison line, forward
 times and backward times against the sequence length, one line per window;
 scripts/plot_fwd_inference_speedup.py: decode time against the cache length) and needs no GPU.
+
+``head_conv`` times the three kernels of the head-mixing variant (the reference's
+head_conv_attn package; it ships no benchmark for it, its own check runs B=2, 16 heads, N=201, d=32,
+head_conv_attn/fwd_kernel.py:383-390).
 
 The reference's third line, its materialising PyTorch module, allocates [B,H,N,N] fp32
 temporaries and is not part of this package; it is timed on the CPU by ``bench.py``.
@@ -112,6 +117,28 @@ def decode_case(B: int, H: int, Nk: int, d: int, c_q: int, c_k: int, iters: int)
     return r
 
 
+HEAD_CONV_SWEEP = [(2, 16, 201, 32), (2, 16, 2048, 64), (2, 32, 2048, 64), (2, 32, 2048, 128), (4, 16, 4096, 128)]
+
+
+def head_conv_case(B: int, H: int, N: int, d: int, iters: int) -> dict:
+    from .head_conv_attn import ops
+    dev = "cuda:0"
+    g = torch.Generator().manual_seed(42)
+    Q, K, V, dO = (torch.randn(B, H, N, d, generator=g).to(torch.bfloat16).to(dev) for _ in range(4))
+    W = (torch.randn(H, H, generator=g) / math.sqrt(H)).to(dev)
+    scale = 1.0 / math.sqrt(d)
+    O, L, M = ops.forward(Q, K, V, W, scale=scale, causal=True)
+    r = {"B": B, "H": H, "N": N, "d": d,
+         "fwd": time_ms(lambda: ops.forward(Q, K, V, W, scale=scale, causal=True), iters),
+         "dq_dw": time_ms(lambda: ops.bwd_dq_dw(Q, K, V, W, O, dO, L, M, causal=True, scale=scale), iters),
+         "dkdv": time_ms(lambda: ops.bwd_dkdv(Q, K, V, W, O, dO, L, M, causal=True, scale=scale), iters),
+         "sdpa_fwd": time_ms(lambda: F.scaled_dot_product_attention(Q, K, V, is_causal=True, scale=scale), iters)}
+    pairs = B * H * N * (N + 1) / 2
+    # per (row, key, head): 4 d (Q K^T, P V) + 2 H (head mix) forward; 10 d + 6 H backward (S, dP, dV, dQ, dK; mix, mix back, dW)
+    r["tflops"] = (14 * d + 8 * H) * pairs / ((r["fwd"] + r["dq_dw"] + r["dkdv"]) * 1e-3) / 1e12
+    return r
+
+
 def parse_table(path: str) -> List[dict]:
     """Rows of the first markdown table of ``path`` as dicts keyed by the header cells."""
     head, rows = None, []
@@ -184,13 +211,13 @@ def plot(train_md: str, decode_md: str, out_dir: str) -> List[str]:
 
 def main(argv=None) -> None:
     ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
-    ap.add_argument("which", choices=["train", "decode", "plot"])
+    ap.add_argument("which", choices=["train", "decode", "head_conv", "plot"])
     ap.add_argument("--quick", action="store_true", help="the reference's 7-line suite / fewer decode lengths")
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--batch", type=int, default=None)
     ap.add_argument("--heads", type=int, default=None)
     ap.add_argument("--head-dim", type=int, default=None)
-    ap.add_argument("--md", default=None, help="train / decode: also write the table, with its command line, to this file")
+    ap.add_argument("--md", default=None, help="train / decode / head_conv: also write the table, with its command line, to this file")
     ap.add_argument("--train", default=None, help="plot: table written by `train`")
     ap.add_argument("--decode", default=None, help="plot: table written by `decode`")
     ap.add_argument("--out", default="plots", help="plot: directory for the figures")
@@ -223,6 +250,17 @@ def main(argv=None) -> None:
             r = train_case(B, H, N, d, k, a.iters)
             emit(f"| {N} | {k}x{k} | {r['conv_fwd']:.3f} | {r['conv_fwd_bwd']:.3f} | {r['sdpa_fwd']:.3f} | "
                  f"{r['sdpa_fwd_bwd']:.3f} | {r['conv_fwd_bwd'] / r['sdpa_fwd_bwd']:.2f}x | {r['conv_tflops']:.1f} |")
+    elif a.which == "head_conv":
+        emit(f"bf16 inputs, causal; ms per call (median of {a.iters}); TFLOP/s = (14 d + 8 H) N(N+1)/2 B H / "
+             "(fwd + dq_dw + dkdv time): the three products of the forward and the seven of the backward, the "
+             "recomputation of S and of the head mix in the second backward kernel not counted")
+        emit("")
+        emit("| B | H | N | d | fwd | bwd dq+dw | bwd dk+dv | sdpa fwd | fwd+bwd TFLOP/s |")
+        emit("|---|---|---|---|---|---|---|---|---|")
+        for B, H, N, d in (HEAD_CONV_SWEEP[:2] if a.quick else HEAD_CONV_SWEEP):
+            r = head_conv_case(B, H, N, d, a.iters)
+            emit(f"| {B} | {H} | {N} | {d} | {r['fwd']:.3f} | {r['dq_dw']:.3f} | {r['dkdv']:.3f} | {r['sdpa_fwd']:.3f} | "
+                 f"{r['tflops']:.1f} |")
     else:
         B, H, d = a.batch or 2, a.heads or 2, a.head_dim or 64
         emit(f"B={B} H={H} d={d} bf16, 11x11 window, 11 resident query rows; ms per call (median of {a.iters}); "

@@ -1,15 +1,17 @@
-// Head-mixing attention ("head_conv_attn" of the reference) on fp32 MFMA (gfx950).
+// Head-mixing attention ("head_conv_attn" of the reference) on the matrix cores of gfx950.
 //
 //   S_h' = scale Q_h' K_h'^T,   Z_h = sum_h' w[h][h'] S_h',   P_h = softmax_j(Z_h + causal mask),
 //   O_h = P_h V_h.
 // The heads of a (batch, row, key) triple are coupled before the softmax, so a workgroup handles
 // ALL heads of 16 query rows (forward, dQ + dW) or of 16 keys (dK / dV) of one batch entry and
-// walks the other axis in tiles of 16.  Every product runs on v_mfma_f32_16x16x4_f32 with fp32
-// accumulation; bf16 inputs are widened to fp32 operands, scores and probabilities stay fp32.
+// walks the other axis in tiles of 16.  Products of two inputs (Q K^T, dO V^T) run on the bf16 MFMA
+// (exact products, fp32 accumulation); scores, the head mix, the softmax and dW stay fp32
+// (v_mfma_f32_16x16x4_f32 for the mix and dW); products of a computed tile with an input (P V,
+// P^T dO, dS K, dS^T Q) round the tile to bf16 and run on v_mfma_f32_16x16x16_bf16.
 //
 // Per 16 x 16 tile (8 waves):
 //   1. waves take heads: S_h' from Q / K row fragments read straight from global memory
-//      (the contraction index is permuted so that one 16-byte load feeds 8 MFMA steps)  -> LDS;
+//      (16 bytes of a row are a lane's operand of the bf16 MFMA as they lie in memory)    -> LDS;
 //   2. waves take rows: Z = W S as a product over the head index (A = W, B = the scores of one
 //      row across the heads), mask, softmax (or P = exp(Z - LSE) in the backward)        -> LDS;
 //   3. waves take heads again: P V (forward), dP = dO V^T, dV += P^T dO, dZ = P (dP - D);
@@ -20,13 +22,12 @@
 // for the whole loop; nothing is accumulated through global memory and there are no atomics
 // (the reference's Triton kernels read-modify-write O per key block, fwd_kernel.py:214-250, and add
 // dW with tl.atomic_add, bwd_dq_dw.py:370): dW partials are summed in a fixed order.
-#include "common.hpp"
+#include "mfma_common.hpp"
 
 namespace convattn {
 namespace {
 
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef short short4_t __attribute__((ext_vector_type(4)));
 
 constexpr int HW = 8;            // waves per workgroup
 constexpr int HT = 16;           // rows / keys per tile
@@ -54,34 +55,63 @@ template <int H, int D> struct HmLds {
     static constexpr int total = stat_off + 3 * H * HT * 4;
 };
 
-// 8 consecutive bf16 of row `row` at column `col` as floats; zeros for rows outside [0, N)
+// 8 consecutive bf16 of row `row` at column `col`; zeros for rows outside [0, N)
 template <int D>
-__device__ __forceinline__ void row_frag(const bf16_t *__restrict__ base, int row, int N, int col, float (&f)[8]) {
+__device__ __forceinline__ bf16x8 row_frag(const bf16_t *__restrict__ base, int row, int N, int col) {
     u32x4 raw = {0u, 0u, 0u, 0u};
     if (row >= 0 && row < N) raw = *reinterpret_cast<const u32x4 *>(base + (size_t)row * D + col);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        f[2 * i] = __uint_as_float(raw[i] << 16);
-        f[2 * i + 1] = __uint_as_float(raw[i] & 0xffff0000u);
-    }
+    return __builtin_bit_cast(bf16x8, raw);
 }
 
 // C[16 x 16] (lane (g, n): rows 4g .. 4g+3, column n) = X Y^T for two row-major bf16 matrices in global
-// memory: rows x0 + n of X against rows y0 + n of Y.  Contraction index of lane group g at step s of
-// block blk: 32 blk + 8 g + s, the same for both operands.
+// memory: rows x0 + n of X against rows y0 + n of Y; the operands of the bf16 MFMA are the rows as
+// they lie in memory (lane (g, n): 8 consecutive columns at 32 blk + 8 g).
 template <int D>
 __device__ __forceinline__ f32x4 rows_times_rows(const bf16_t *__restrict__ X, int x0, const bf16_t *__restrict__ Y,
                                                  int y0, int N, int g, int n) {
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int blk = 0; blk < D / 32; ++blk) {
-        float a[8], b[8];
-        row_frag<D>(X, x0 + n, N, blk * 32 + 8 * g, a);
-        row_frag<D>(Y, y0 + n, N, blk * 32 + 8 * g, b);
-#pragma unroll
-        for (int s = 0; s < 8; ++s) acc = mfma4(a[s], b[s], acc);
-    }
+    for (int blk = 0; blk < D / 32; ++blk)
+        acc = mfma_bf16(row_frag<D>(X, x0 + n, N, blk * 32 + 8 * g), row_frag<D>(Y, y0 + n, N, blk * 32 + 8 * g), acc);
     return acc;
+}
+
+// The same in two steps, for loads issued a tile ahead of their use: the row fragments of a 16-row tile ...
+template <int D>
+__device__ __forceinline__ void load_frags(bf16x8 (&f)[D / 32], const bf16_t *__restrict__ X, int x0, int N, int g, int n) {
+#pragma unroll
+    for (int blk = 0; blk < D / 32; ++blk) f[blk] = row_frag<D>(X, x0 + n, N, blk * 32 + 8 * g);
+}
+template <int D>
+__device__ __forceinline__ f32x4 frags_dot(const bf16x8 (&x)[D / 32], const bf16x8 (&y)[D / 32]) {
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int blk = 0; blk < D / 32; ++blk) acc = mfma_bf16(x[blk], y[blk], acc);
+    return acc;
+}
+// ... and the 16-byte chunks of 16 rows that a lane stages (chunk c of the tile: row c / (D / 8))
+template <int D>
+__device__ __forceinline__ void load_chunks(u32x4 (&r)[(HT * D / 8 + 63) / 64], const bf16_t *__restrict__ base, int r0,
+                                            int N, int lane) {
+    constexpr int CPR = D / 8;
+#pragma unroll
+    for (int i = 0; i < (HT * CPR + 63) / 64; ++i) {
+        const int c = lane + i * 64, row = c / CPR, cc = c % CPR;
+        r[i] = (u32x4){0u, 0u, 0u, 0u};
+        if (c < HT * CPR && r0 + row >= 0 && r0 + row < N)
+            r[i] = *reinterpret_cast<const u32x4 *>(base + (size_t)(r0 + row) * D + cc * 8);
+    }
+}
+template <int D>
+__device__ __forceinline__ void stage_chunks(unsigned char *xt, int xst, const u32x4 (&r)[(HT * D / 8 + 63) / 64], int lane) {
+    constexpr int CPR = D / 8;
+#pragma unroll
+    for (int i = 0; i < (HT * CPR + 63) / 64; ++i) {
+        const int c = lane + i * 64, row = c / CPR, cc = c % CPR;
+        if (c < HT * CPR) *reinterpret_cast<u32x4 *>(xt + row * xst + cc * 16) = r[i];
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
 }
 
 // Rows r0 .. r0+15 of a [N][D] bf16 matrix into this wave's staging tile (zeros outside [0, N)).
@@ -99,21 +129,21 @@ __device__ __forceinline__ void stage_rows(unsigned char *xt, int xst, const bf1
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
 }
-__device__ __forceinline__ float staged(const unsigned char *xt, int xst, int row, int col) {
-    return __uint_as_float((unsigned int)*reinterpret_cast<const unsigned short *>(xt + row * xst + col * 2) << 16);
-}
 
 // acc[db] (lane (g, n): tile row 4g .. 4g+3, head-dim column 16 db + n) += A X, with A a 16 x 16 fp32 tile
-// in LDS (element (m, k) at a[m * a_rs + k * a_cs]) and X this wave's staged 16-row tile.
+// in LDS (element (m, k) at a[m * a_rs + k * a_cs]; rounded to bf16 here) and X this wave's staged
+// 16-row bf16 tile, read with transpose reads (lane (g, n): rows 4g .. 4g+3 of column 16 db + n).
 template <int D>
 __device__ __forceinline__ void tile_times_staged(f32x4 (&acc)[D / 16], const float *a, int a_rs, int a_cs,
                                                   const unsigned char *xt, int xst, int g, int n) {
+    bf16x4 av;
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-        const float av = a[n * a_rs + (4 * s + g) * a_cs];
+    for (int e = 0; e < 4; ++e) av[e] = (bf16_t)a[n * a_rs + (4 * g + e) * a_cs];
 #pragma unroll
-        for (int db = 0; db < D / 16; ++db) acc[db] = mfma4(av, staged(xt, xst, 4 * s + g, db * 16 + n), acc[db]);
-    }
+    for (int db = 0; db < D / 16; ++db)
+        acc[db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, av),
+                                                             __builtin_bit_cast(short4_t, lds_read_tr4x16(xt, xst, 4 * g, db * 16, n)),
+                                                             acc[db], 0, 0, 0);
 }
 
 // Max / sum over the 16 lanes of a lane group (all of them get the result).
@@ -193,10 +223,38 @@ __global__ __launch_bounds__(HW * 64) void headmix_fwd_kernel(HmArgs a, const bf
 #pragma unroll
             for (int r = 0; r < 4; ++r) { m_run[rl][hb][r] = kNegInf; l_run[rl][hb][r] = 0.f; }
 
+    // Where the registers allow it the Q fragments of the wave's heads stay resident, the K fragments
+    // of a tile are loaded while the tile before it is worked on, and the V rows of a tile are on their
+    // way during its score and softmax phases: a workgroup fills its CU alone, so nothing else hides
+    // the latency of these loads.
+    constexpr bool AHEAD = HPW * (D / 32) <= 8;
+    constexpr int NCH = (HT * D / 8 + 63) / 64;
+    bf16x8 qf[AHEAD ? HPW : 1][D / 32], kf[AHEAD ? HPW : 1][D / 32];
+    u32x4 vr[AHEAD ? HPW : 1][NCH];
+    if constexpr (AHEAD) {
+#pragma unroll
+        for (int t = 0; t < HPW; ++t) {
+            load_frags<D>(qf[t], Qb + (size_t)(wave + t * HW) * a.N * D, i0, a.N, g, n);
+            load_frags<D>(kf[t], Kb + (size_t)(wave + t * HW) * a.N * D, 0, a.N, g, n);
+        }
+    }
+
     const int j_end = a.causal ? min(a.N, i0 + HT) : a.N;
     for (int j0 = 0; j0 < j_end; j0 += HT) {
         __syncthreads();   // the last tile's P has been used (and, first, W is in place)
-        scores_phase<H, D>(S, a, Qb, Kb, i0, j0, wave, g, n);
+        if constexpr (AHEAD) {
+#pragma unroll
+            for (int t = 0; t < HPW; ++t) {
+                const int h = wave + t * HW;
+                load_chunks<D>(vr[t], Vb + (size_t)h * a.N * D, j0, a.N, lane);
+                const f32x4 sc = frags_dot<D>(qf[t], kf[t]);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) S[h * HST + (4 * g + r) * SST + n] = sc[r] * a.scale;
+                load_frags<D>(kf[t], Kb + (size_t)h * a.N * D, j0 + HT, a.N, g, n);
+            }
+        } else {
+            scores_phase<H, D>(S, a, Qb, Kb, i0, j0, wave, g, n);
+        }
         __syncthreads();
 #pragma unroll
         for (int rl = 0; rl < RPW; ++rl) {
@@ -224,7 +282,8 @@ __global__ __launch_bounds__(HW * 64) void headmix_fwd_kernel(HmArgs a, const bf
 #pragma unroll
         for (int t = 0; t < HPW; ++t) {
             const int h = wave + t * HW;
-            stage_rows<D>(xt, Lds::XST, Vb + (size_t)h * a.N * D, j0, a.N, lane);
+            if constexpr (AHEAD) stage_chunks<D>(xt, Lds::XST, vr[t], lane);
+            else stage_rows<D>(xt, Lds::XST, Vb + (size_t)h * a.N * D, j0, a.N, lane);
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const float alpha = al[h * HT + 4 * g + r];
