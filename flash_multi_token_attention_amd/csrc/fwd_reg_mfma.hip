@@ -73,29 +73,18 @@ __device__ long long g_fwd_ts[4][64][8];
 #define FTSX(a, b)
 #endif
 
-#ifndef FWD_DMA
-#define FWD_DMA 1
-#endif
 #ifndef FWD_NBUF
-#define FWD_NBUF 2
+#define FWD_NBUF 2   // LDS buffers: 2 = the rows of step u+1 arrive during step u (3: two steps ahead; measured: no faster)
 #endif
 template <int D> struct FwdLds {
-#if FWD_DMA
     // K / V rows go from global memory straight into LDS (buffer loads with the LDS modifier: the
     // 64 lanes of a load fill 1 KB of consecutive LDS, which rules out padded rows), so the rows are
     // dense and the 16-byte chunk c of row r sits at chunk position c ^ (r mod chunks per row):
     // a fragment read (16 rows, one column) then touches 16 different bank groups.
     static constexpr int KST = D * 2;
-#else
-    static constexpr int KST = D * 2 + 16;  // bytes per K / V row (== 16 mod 256 for D = 128)
-#endif
     static constexpr int k_bytes = BK * KST;
     static constexpr int buf_bytes = 2 * k_bytes;  // K rows, then V rows
-#if FWD_DMA
     static constexpr int n_buf = FWD_NBUF;         // steps u, u+1 (and u+2) resident or on their way
-#else
-    static constexpr int n_buf = 2;
-#endif
     static constexpr int total = n_buf * buf_bytes;
 };
 
@@ -190,18 +179,9 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
     // 2u-1, 2u (keys 32u-16 .. 32u+15, V rows of the step); an output block needs the score
     // block 8 keys before it and the one 8 keys after it, so the packed scores of block 2u-1
     // are carried from the previous step.
-    // Staging registers: every thread holds its 16-byte chunks of the K / V rows of step u+2
-    // while step u is computed.
-#if !FWD_DMA
-    u32x4 kr[N_LD], vr[N_LD];
-#endif
-    // Buffer loads: rows before the first or after the last key are outside the descriptor's
-    // range and read as zeros, which is what the window's zero padding asks for.
-    const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)Kb, 0, p.Nk * D * 2, 0x00020000);
-    const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)Vb, 0, p.Nk * D * 2, 0x00020000);
-    const int ld_off = ((tid / CPR) * D + (tid % CPR) * 8) * 2;  // byte offset of this thread's first chunk in a step
-    constexpr int kChunkStep = (NW * 64 / CPR) * D * 2;         // and from one of its chunks to the next
-#if FWD_DMA
+    // K / V rows: buffer loads with the LDS modifier.  Rows before the first or after the last key
+    // are outside the descriptor's range and arrive as zeros, which is what the window's zero
+    // padding asks for.
     // Load i of a wave fills rows RPL (i NW + wave) .. + RPL - 1 of a tile (RPL = rows per KB): lane l
     // writes chunk position l % CPR of row l / CPR and therefore reads chunk (l % CPR) ^ (row % CPR).
     constexpr int RPL = 1024 / (D * 2);
@@ -242,25 +222,6 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
         const int r = 4 * g + (n >> 2);
         va[db] = opaque_u32(r * KST + (((db * 2 + ((n >> 1) & 1)) ^ (r % CPR)) << 4) + (n & 1) * 8);
     }
-#else
-    auto load_step = [&](int u) {
-        const int k0 = (32 * u - 8) * D * 2 + ld_off, v0 = (32 * u - 16) * D * 2 + ld_off;
-#pragma unroll
-        for (int i = 0; i < N_LD; ++i) {
-            kr[i] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, k0 + i * kChunkStep, 0, 0);
-            vr[i] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, v0 + i * kChunkStep, 0, 0);
-        }
-    };
-    auto stage_step = [&](int u) {
-        unsigned char *Ks = smem + (u & 1) * Lds::buf_bytes, *Vs = Ks + Lds::k_bytes;
-#pragma unroll
-        for (int i = 0; i < N_LD; ++i) {
-            const int c = tid + i * NW * 64, row = c / CPR, cc = c % CPR;
-            *reinterpret_cast<u32x4 *>(Ks + row * KST + cc * 16) = kr[i];
-            *reinterpret_cast<u32x4 *>(Vs + row * KST + cc * 16) = vr[i];
-        }
-    };
-#endif
 
     // packed fp16 scores of the last score block of the previous step:
     // carry[f][dword] = row base + 2n + f, keys 4g .. 4g+3 of the block
@@ -270,13 +231,9 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
     // (wave-uniform), only then are the masks evaluated.
     auto step = [&](int u, auto edge_tag) {
         constexpr bool EDGE = decltype(edge_tag)::value;
-#if FWD_DMA
         // (the address registers ka / va point into the buffer of the step: they are moved to the
         // other buffer at the end of every step)
         const unsigned char *Ks = smem, *Vs = Ks + Lds::k_bytes;
-#else
-        const unsigned char *Ks = smem + (u & 1) * Lds::buf_bytes, *Vs = Ks + Lds::k_bytes;
-#endif
         const int jk = 32 * u - 8, jv = 32 * u - 16;
         f32x4 c[2][2];
         bf16x8 kf[KS];  // K fragments of one score block; the second block's are read during the first's convolution
@@ -284,11 +241,7 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
         auto load_kf = [&](int blk) {
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks)
-#if FWD_DMA
                 kf[ks] = *reinterpret_cast<const bf16x8 *>(Ks + ka[ks] + blk * 16 * KST);
-#else
-                kf[ks] = *reinterpret_cast<const bf16x8 *>(Ks + (blk * 16 + n) * KST + (ks * 32 + g * 8) * 2);
-#endif
         };
         load_kf(0);
         static_for<2>([&](auto BL) {
@@ -359,13 +312,8 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
         constexpr int PFV = FWD_PFV < DB ? FWD_PFV : DB;
         bf16x8 vf[PFV + 1];
         auto load_vf = [&](int buf, int db) {
-#if FWD_DMA
             bf16x4 lo = lds_tr64(Vs + va[db]);
             bf16x4 hi = lds_tr64(Vs + va[db] + 16 * KST);
-#else
-            bf16x4 lo = lds_read_tr4x16(Vs, KST, 4 * g, db * 16, n);
-            bf16x4 hi = lds_read_tr4x16(Vs, KST, 16 + 4 * g, db * 16, n);
-#endif
             vf[buf] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
         };
 #pragma unroll
@@ -464,14 +412,8 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
 
     const int k_end = causal ? min(p.Nk, i0 + BQ) : p.Nk;
     const int n_steps = (k_end + 16 + BK - 1) / BK;
-#if FWD_DMA
     fetch_step(0);
     if constexpr (Lds::n_buf == 3) fetch_step(1);
-#else
-    load_step(0);
-    stage_step(0);
-    load_step(1);
-#endif
     // Along the keys a wave's steps are: step 0 (keys before the first one to mask), steps whose
     // keys all lie at or before its first score row (no masks), steps on the diagonal or at the
     // end of the keys (masks), and steps entirely after its rows (it only takes part in the
@@ -481,14 +423,11 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
 #pragma unroll 1
         for (int u = ua; u < ub; ++u) {
             FTS(0);
-#if FWD_DMA
             // this wave's rows of step u have landed (with three buffers those of step u + 1 may be on their way)
             if constexpr (Lds::n_buf == 3) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * N_LD) : "memory");
             else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#endif
             __syncthreads();  // step u-1 is done everywhere: its buffer is free, and step u's is written
             FTS(1);
-#if FWD_DMA
             fetch_step(u + Lds::n_buf - 1);
             FTS(2);
             if constexpr (KIND != 2) step(u, std::integral_constant<bool, KIND == 1>{});
@@ -497,12 +436,6 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
             for (int ks = 0; ks < KS; ++ks) ka[ks] += to_other;
 #pragma unroll
             for (int db = 0; db < DB; ++db) va[db] += to_other;
-#else
-            stage_step(u + 1);
-            load_step(u + 2);
-            FTS(2);
-            if constexpr (KIND != 2) step(u, std::integral_constant<bool, KIND == 1>{});
-#endif
         }
     };
     const int u_diag = base < 23 ? 1 : (base - 23) / 32 + 1;    // first u >= 1 with 32u + 23 > base

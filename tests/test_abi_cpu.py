@@ -218,3 +218,35 @@ def test_kv_layout_rejected_before_launch(lib):
     dd32 = desc(Nq=6, causal=0, n_splits=2, H=8, Nk=4096, d=128, in_dtype=_lib.F32)
     assert lib.convattn_decode_kv(C.byref(dd32), ok, ok, ok, C.byref(_lib.KvLayout(**dense)), ok, ok, ok, ok, null) == -14
     assert b"KV layout" in lib.convattn_strerror(-14)
+
+
+def test_headmix_descriptor_checks_and_import_paths(lib):
+    # host-only checks of the head-mixing entry points (nothing below reaches a launch)
+    def hd(**kw):
+        base = dict(B=2, H=16, N=201, d=32, scale=0.17, causal=1, in_dtype=_lib.BF16, out_dtype=_lib.BF16)
+        base.update(kw)
+        return _lib.HeadmixDesc(**base)
+
+    assert lib.convattn_headmix_validate(C.byref(hd())) == 0
+    assert lib.convattn_headmix_validate(C.byref(hd(H=8))) == -15
+    assert lib.convattn_headmix_validate(C.byref(hd(d=48))) == -15
+    assert lib.convattn_headmix_validate(C.byref(hd(in_dtype=_lib.F32))) == -15
+    assert lib.convattn_headmix_validate(C.byref(hd(N=0))) == -2
+    assert lib.convattn_headmix_validate(C.byref(hd(scale=float("nan")))) == -9
+    assert b"16 or 32" in lib.convattn_strerror(-15)
+    # D and LSE of every row, one [H][H] partial per 16-row tile and batch entry
+    want = 2 * ((2 * 16 * 201 * 4 + 255) // 256 * 256) + (2 * 13 * 16 * 16 * 4 + 255) // 256 * 256
+    assert lib.convattn_headmix_bwd_workspace_bytes(C.byref(hd())) == want
+    assert lib.convattn_headmix_bwd_workspace_bytes(C.byref(hd(H=7))) == 0
+    null, ok = C.c_void_p(0), C.c_void_p(4096)
+    assert lib.convattn_headmix_fwd(C.byref(hd()), ok, ok, null, ok, ok, ok, ok, null) == -1
+    assert lib.convattn_headmix_fwd(C.byref(hd()), ok, ok, C.c_void_p(4100), ok, ok, ok, ok, null) == -6
+    # the import statements of the reference's head_conv_attn/head_conv_attn.py:6-8 and of its users
+    from flash_multi_token_attention.head_conv_attn.fwd_kernel import head_conv_attention_forward  # noqa: F401
+    from flash_multi_token_attention.head_conv_attn.bwd_dq_dw import head_conv_attention_bwd_dq_dw  # noqa: F401
+    from flash_multi_token_attention.head_conv_attn.bwd_dk_dv import head_conv_attention_bwd_dkdv  # noqa: F401
+    from flash_multi_token_attention.head_conv_attn.head_conv_attn import (  # noqa: F401
+        HeadConvAttention, HeadConvAttentionFunction, head_conv_attention)
+    mod = HeadConvAttention(16, dtype=torch.bfloat16)
+    assert tuple(mod.head_conv_weights.shape) == (16, 16) and mod.head_conv_weights.dtype == torch.bfloat16
+    assert list(mod.state_dict()) == ["head_conv_weights"]
