@@ -1,9 +1,11 @@
 // fp32-arithmetic conv-attention kernels for gfx950: every supported shape and
 // both input types.  These are the "exact" path (CONVATTN_FLAG_EXACT, fp32
-// inputs, shapes the MFMA kernels do not cover): all dot products, the
-// convolution and the softmax run in fp32 on the vector ALUs out of LDS tiles,
-// accumulators stay in registers for the whole key (or query) loop, and nothing
-// is accumulated through HBM or with atomics.
+// inputs, shapes the bf16 MFMA kernels do not cover): all operands, scores and
+// probabilities are fp32.  The dot products (Q K^T, P V, dO V^T, dS K, dS^T Q,
+// P^T dO) run on v_mfma_f32_16x16x4_f32 with both operands read from fp32 LDS
+// tiles; the convolution, its transpose, dW and the softmax run on the vector
+// ALUs.  Accumulators stay in registers for the whole key (or query) loop, and
+// nothing is accumulated through HBM or with atomics.
 //
 // Index conventions (per batch b, head h): query row i, key column j, tap
 // (a, b) of W[h] looks at S_m[i + a - pq][j + b - pk].  A workgroup owns
@@ -16,21 +18,45 @@ namespace {
 
 constexpr int TR = kGenTR;
 constexpr int NT = 256;  // threads per workgroup
+constexpr int NWV = NT / 64;
 
-// dst[r][c] (row stride `stride`) = src[(row0 + r) * d + c], zero outside [0, N).
+// dst[r][c] (row stride `stride`) = src[(row0 + r) * d + c], zero outside [0, N): eight elements (d is
+// a multiple of 8) per thread and turn.
+__device__ __forceinline__ void load8_f32(const float *src, float (&v)[8]) {
+    const float4 a = *reinterpret_cast<const float4 *>(src), b = *reinterpret_cast<const float4 *>(src + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+__device__ __forceinline__ void load8_f32(const bf16_t *src, float (&v)[8]) {
+    const uint4 raw = *reinterpret_cast<const uint4 *>(src);
+    const unsigned int w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        v[2 * i] = __uint_as_float(w[i] << 16);
+        v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+}
 template <typename T>
 __device__ __forceinline__ void load_rows(float *dst, int stride, const T *src, int row0, int nrows,
                                           int N, int d) {
-    for (int idx = threadIdx.x; idx < nrows * d; idx += NT) {
-        int r = idx / d, c = idx - r * d;
-        int g = row0 + r;
-        dst[r * stride + c] = (g >= 0 && g < N) ? to_f32(src[(size_t)g * d + c]) : 0.f;
+    const int cpr = d / 8;
+    for (int idx = threadIdx.x; idx < nrows * cpr; idx += NT) {
+        const int r = idx / cpr, c = (idx - r * cpr) * 8;
+        const int g = row0 + r;
+        float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        if (g >= 0 && g < N) load8_f32(src + (size_t)g * d + c, v);
+        float *out = dst + r * stride + c;
+        if ((stride & 3) == 0) {
+            *reinterpret_cast<float4 *>(out) = make_float4(v[0], v[1], v[2], v[3]);
+            *reinterpret_cast<float4 *>(out + 4) = make_float4(v[4], v[5], v[6], v[7]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) out[i] = v[i];
+        }
     }
 }
 
-// S[r][c] = scale * <A[r], Kt[c]> for r < nr, c < nc; rows/cols outside the
-// sequence are zero because their operands were zero-filled; the causal
-// pre-mask zeroes keys after the row's own position.
+// S[r][c] = scale * <A[r], Kt[c]> for r < nr, c < nc on the vector ALUs (the decode kernel's few rows);
+// the causal pre-mask zeroes keys after the row's own position.
 __device__ __forceinline__ void score_tile(float *S, int sstride, const float *A, int astride,
                                            const float *Kt, int kstride, int nr, int nc, int d,
                                            int row_pos0, int col_pos0, float scale, int causal) {
@@ -43,6 +69,119 @@ __device__ __forceinline__ void score_tile(float *S, int sstride, const float *A
         if (causal && (col_pos0 + c) > (row_pos0 + r)) acc = 0.f;
         S[r * sstride + c] = acc * scale;
     }
+}
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// Four adjacent outputs of the convolution, out[k] = sum_ab W[a][b] * X[(a) rows down][k + b columns on],
+// with `x` pointing at the window's first element for output 0: one new tile element and one weight
+// are read per four multiply-adds, and the four sums are independent.
+__device__ __forceinline__ void conv4(float (&out)[4], const float *Ws, int c_q, int c_k, const float *x, int xstride) {
+    out[0] = out[1] = out[2] = out[3] = 0.f;
+    for (int a = 0; a < c_q; ++a) {
+        const float *row = x + a * xstride, *w = Ws + a * c_k;
+        float s0 = row[0], s1 = row[1], s2 = row[2];
+#pragma unroll 4
+        for (int bb = 0; bb < c_k; ++bb) {
+            const float s3 = row[bb + 3], wv = w[bb];
+            out[0] = fmaf(wv, s0, out[0]);
+            out[1] = fmaf(wv, s1, out[1]);
+            out[2] = fmaf(wv, s2, out[2]);
+            out[3] = fmaf(wv, s3, out[3]);
+            s0 = s1; s1 = s2; s2 = s3;
+        }
+    }
+}
+// The transposed convolution: out[k] = sum_ab W[a][b] * X[a rows UP][k - b columns], `x` pointing at the
+// element under output 0 for tap (0, 0).
+__device__ __forceinline__ void conv4_t(float (&out)[4], const float *Ws, int c_q, int c_k, const float *x, int xstride) {
+    out[0] = out[1] = out[2] = out[3] = 0.f;
+    for (int a = 0; a < c_q; ++a) {
+        const float *row = x - a * xstride, *w = Ws + a * c_k;
+        float s1 = row[1], s2 = row[2], s3 = row[3];
+#pragma unroll 4
+        for (int bb = 0; bb < c_k; ++bb) {
+            const float s0 = row[-bb], wv = w[bb];
+            out[0] = fmaf(wv, s0, out[0]);
+            out[1] = fmaf(wv, s1, out[1]);
+            out[2] = fmaf(wv, s2, out[2]);
+            out[3] = fmaf(wv, s3, out[3]);
+            s3 = s2; s2 = s1; s1 = s0;
+        }
+    }
+}
+
+// NB 16 x 16 blocks at once that share the left operand: acc[u] (lane (g, n): rows 4g .. 4g+3, column n)
+// += A B_u over k < K (a multiple of 4), operands fp32 in LDS.  `ap` / `bp[u]` are this lane's operand
+// pointers at k = 0 (A: row n at k = g; B: column n at k = g), a_ks / b_ks the strides per unit of k.  Independent accumulators keep the
+// matrix pipe busy where one chain of dependent MFMAs would wait for itself.
+template <int NB>
+__device__ __forceinline__ void lds_mma_n(f32x4 (&acc)[NB], const float *ap, int a_ks, const float *const (&bp)[NB],
+                                          int b_ks, int K) {
+    for (int k = 0; k < K; k += 4) {
+        const float a = ap[k * a_ks];
+#pragma unroll
+        for (int u = 0; u < NB; ++u) acc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, bp[u][k * b_ks], acc[u], 0, 0, 0);
+    }
+}
+
+// S[r][c] = scale * <A[r], Kt[c]> for r < nr, c < nc on the matrix cores: a wave takes strips of one
+// 16-row block times three 16-column blocks; the causal pre-mask zeroes keys after the row's own position.
+__device__ __forceinline__ void score_tile_mma(float *S, int sstride, const float *A, int astride, const float *Kt,
+                                               int kstride, int nr, int nc, int d, int row_pos0, int col_pos0,
+                                               float scale, int causal) {
+    constexpr int CBW = 3;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 4, n = lane & 15;
+    const int nrb = (nr + 15) / 16, ncb = (nc + 15) / 16, ncs = (ncb + CBW - 1) / CBW;
+    for (int strip = wave; strip < nrb * ncs; strip += NWV) {
+        const int rb = strip / ncs, cb0 = (strip - rb * ncs) * CBW;
+        f32x4 acc[CBW];
+        const float *bp[CBW];
+#pragma unroll
+        for (int u = 0; u < CBW; ++u) {
+            acc[u] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            bp[u] = Kt + min((cb0 + u) * 16 + n, nc - 1) * kstride + g;   // (blocks past the last one repeat it)
+        }
+        lds_mma_n<CBW>(acc, A + min(rb * 16 + n, nr - 1) * astride + g, 1, bp, 1, d);
+#pragma unroll
+        for (int u = 0; u < CBW; ++u) {
+            const int c = (cb0 + u) * 16 + n;
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+                const int r = rb * 16 + 4 * g + rr;
+                if (r < nr && c < nc && cb0 + u < ncb)
+                    S[r * sstride + c] = (causal && (col_pos0 + c) > (row_pos0 + r)) ? 0.f : acc[u][rr] * scale;
+            }
+        }
+    }
+}
+
+// LDS carve-up of the forward.  Row strides: == 4 mod 32 floats where the 16 lanes of an MFMA operand
+// read 16 rows at one column (Q, K), == 16 mod 32 where they read one row at 16 columns and the lane
+// groups 4 rows (V as the right-hand side of P V).
+struct FwdLds {
+    float *Qs, *KVs, *Ss, *Ps, *Ws, *m_s, *l_s, *al_s;
+    int qst, kst, vst, sst, pst;
+};
+__host__ __device__ inline size_t fwd_lds_floats(int d, int pq, int pk, int ntap) {
+    const int QR = TR + pq, SC = kGenFwdTC + 2 * pk;
+    const size_t kv = (size_t)SC * (d + 4) > (size_t)kGenFwdTC * (d + 16) ? (size_t)SC * (d + 4) : (size_t)kGenFwdTC * (d + 16);
+    return (size_t)QR * (d + 4) + kv + (size_t)QR * (SC + 1) + (size_t)TR * (kGenFwdTC + 4) + ntap + 3 * TR;
+}
+__device__ __forceinline__ FwdLds carve_fwd(float *lds, const Problem &p) {
+    FwdLds t;
+    const int d = p.d, QR = TR + p.pq, SC = kGenFwdTC + 2 * p.pk;
+    t.qst = d + 4; t.kst = d + 4; t.vst = d + 16; t.sst = SC + 1; t.pst = kGenFwdTC + 4;
+    const int kv = max(SC * t.kst, kGenFwdTC * t.vst);
+    t.Qs = lds;
+    t.KVs = t.Qs + QR * t.qst;
+    t.Ss = t.KVs + kv;
+    t.Ps = t.Ss + QR * t.sst;
+    t.Ws = t.Ps + TR * t.pst;
+    t.m_s = t.Ws + p.c_q * p.c_k;
+    t.l_s = t.m_s + TR;
+    t.al_s = t.l_s + TR;
+    return t;
 }
 
 // ------------------------------------------------------------------ forward
@@ -59,117 +198,122 @@ __global__ __launch_bounds__(NT) void gen_fwd_kernel(Problem p, const TI *__rest
     const int r0 = blockIdx.x * TR;
     const int pq = p.pq, pk = p.pk, d = p.d;
     const int QR = TR + pq, SC = TC + 2 * pk;
-    const int kst = d + 1, sst = SC + 1, ntap = p.c_q * p.c_k;
-    float *Qs = lds;
-    float *KVs = Qs + QR * d;
-    float *Ss = KVs + SC * kst;
-    float *Ps = Ss + QR * sst;
-    float *Ws = Ps + TR * TC;
-    float *m_s = Ws + ntap;
-    float *l_s = m_s + TR;
-    float *al_s = l_s + TR;
+    const FwdLds t = carve_fwd(lds, p);
+    const int ntap = p.c_q * p.c_k;
+    float *Qs = t.Qs, *KVs = t.KVs, *Ss = t.Ss, *Ps = t.Ps, *Ws = t.Ws, *m_s = t.m_s, *l_s = t.l_s, *al_s = t.al_s;
+    const int qst = t.qst, kst = t.kst, vst = t.vst, sst = t.sst, pst = t.pst;
 
     const size_t bh = (size_t)b * p.H + h;
     const TI *Qb = Q + bh * p.Nq * d;
     const TI *Kb = K + bh * p.Nk * d;
     const TI *Vb = V + bh * p.Nk * d;
 
-    load_rows(Qs, d, Qb, r0 - pq, QR, p.Nq, d);
+    load_rows(Qs, qst, Qb, r0 - pq, QR, p.Nq, d);
     for (int i = tid; i < ntap; i += NT) Ws[i] = W[(size_t)h * ntap + i];
     if (tid < TR) { m_s[tid] = kNegInf; l_s[tid] = 0.f; }
 
-    const int orow = tid >> 4, ocol = tid & 15;  // this thread's output row and column phase
-    float acc[kMaxD / 16];
+    // O: a wave holds the 16 x 16 blocks wave, wave + 4 of the head dimension (lane (g, n): rows 4g .. 4g+3)
+    const int wave = tid >> 6, lane = tid & 63, g = lane >> 4, n = lane & 15;
+    f32x4 acc[kMaxD / 16 / NWV];
 #pragma unroll
-    for (int u = 0; u < kMaxD / 16; ++u) acc[u] = 0.f;
+    for (int u = 0; u < kMaxD / 16 / NWV; ++u) acc[u] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
     const int kend = p.causal ? min(p.Nk, r0 + TR) : p.Nk;
     for (int c0 = 0; c0 < kend; c0 += TC) {
         load_rows(KVs, kst, Kb, c0 - pk, SC, p.Nk, d);
         __syncthreads();
-        score_tile(Ss, sst, Qs, d, KVs, kst, QR, SC, d, r0 - pq, c0 - pk, p.scale, p.causal);
+        score_tile_mma(Ss, sst, Qs, qst, KVs, kst, QR, SC, d, r0 - pq, c0 - pk, p.scale, p.causal);
         __syncthreads();
-        load_rows(KVs, kst, Vb, c0, TC, p.Nk, d);  // V replaces K
-        for (int idx = tid; idx < TR * TC; idx += NT) {
-            int i = idx / TC, j = idx - i * TC;
-            int qi = r0 + i, kj = c0 + j;
-            float c = kNegInf;
-            if (kj < p.Nk && !(p.causal && kj > qi)) {
-                c = 0.f;
-                for (int a = 0; a < p.c_q; ++a)
-                    for (int bb = 0; bb < p.c_k; ++bb)
-                        c = fmaf(Ws[a * p.c_k + bb], Ss[(i + a) * sst + j + bb], c);
+        load_rows(KVs, vst, Vb, c0, TC, p.Nk, d);  // V replaces K
+        for (int idx = tid; idx < TR * TC / 4; idx += NT) {
+            const int i = idx / (TC / 4), j = (idx - i * (TC / 4)) * 4;
+            float c[4];
+            conv4(c, Ws, p.c_q, p.c_k, Ss + i * sst + j, sst);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int qi = r0 + i, kj = c0 + j + k;
+                Ps[i * pst + j + k] = (kj < p.Nk && !(p.causal && kj > qi)) ? c[k] : kNegInf;
             }
-            Ps[idx] = c;
         }
         __syncthreads();
         {   // online softmax: one wave per 4 rows, one lane per key of the tile
-            const int wv = tid >> 6, lane = tid & 63;
             for (int rr = 0; rr < 4; ++rr) {
-                int i = wv * 4 + rr;
-                float c = Ps[i * TC + lane];
+                int i = wave * 4 + rr;
+                float c = Ps[i * pst + lane];
                 float m_old = m_s[i];
                 float m_new = fmaxf(m_old, wave_max(c));
                 float e = (c == kNegInf) ? 0.f : __expf(c - m_new);
                 float sum = wave_sum(e);
                 float al = (m_old == kNegInf) ? 0.f : __expf(m_old - m_new);
-                Ps[i * TC + lane] = e;
+                Ps[i * pst + lane] = e;
                 if (lane == 0) { m_s[i] = m_new; l_s[i] = l_s[i] * al + sum; al_s[i] = al; }
             }
         }
         __syncthreads();
         {
-            const float al = al_s[orow];
-            const float *prow = Ps + orow * TC;
+            // P (16 x TC; keys past the end are 0) times V (rows zero-filled past the end); columns past d
+            // repeat the last one and are not stored
+            const float *bp[kMaxD / 16 / NWV];
 #pragma unroll
-            for (int u = 0; u < kMaxD / 16; ++u) {
-                int dc = ocol + 16 * u;
-                if (dc < d) {
-                    float s = acc[u] * al;
-                    for (int j = 0; j < TC; ++j) s = fmaf(prow[j], KVs[j * kst + dc], s);
-                    acc[u] = s;
-                }
+            for (int u = 0; u < kMaxD / 16 / NWV; ++u) {
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr) acc[u][rr] *= al_s[4 * g + rr];
+                bp[u] = KVs + g * vst + min((wave + NWV * u) * 16 + n, d - 1);
             }
+            lds_mma_n<kMaxD / 16 / NWV>(acc, Ps + n * pst + g, 1, bp, vst, TC);
         }
         __syncthreads();
     }
-    const int qi = r0 + orow;
-    if (qi < p.Nq) {
-        const float inv = 1.f / l_s[orow];
 #pragma unroll
-        for (int u = 0; u < kMaxD / 16; ++u) {
-            int dc = ocol + 16 * u;
-            if (dc < d) O[(bh * p.Nq + qi) * d + dc] = from_f32<TO>(acc[u] * inv);
+    for (int u = 0; u < kMaxD / 16 / NWV; ++u) {
+        const int dc = (wave + NWV * u) * 16 + n;
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+            const int qi = r0 + 4 * g + rr;
+            if (qi < p.Nq && dc < d) O[(bh * p.Nq + qi) * d + dc] = from_f32<TO>(acc[u][rr] / l_s[4 * g + rr]);
         }
-        if (ocol == 0) { M[bh * p.Nq + qi] = m_s[orow]; L[bh * p.Nq + qi] = l_s[orow]; }
     }
+    if (tid < TR && r0 + tid < p.Nq) { M[bh * p.Nq + r0 + tid] = m_s[tid]; L[bh * p.Nq + r0 + tid] = l_s[tid]; }
 }
 
 // ----------------------------------------------------------------- backward
-// LDS carve-up shared by the two backward kernels.
+// LDS carve-up shared by the two backward kernels (row strides as in the forward).
 struct BwdLds {
-    float *Qs, *dOs, *KVs, *Ss, *dCs, *Ps, *dSs, *Ws, *lse_s, *D_s;
-    int kst, sst, cst, pst;
+    float *Qs, *dOs, *KVs, *Ss, *dCs, *Ps, *dSs, *Ws, *lse_s, *D_s, *red;
+    int qst, gst, kst, kst2, sst, cst, pst;
 };
+constexpr int kDwRowGroups = 8;   // dW: a work item is one tap over TR / 8 rows of a tile
+constexpr int kDwItemsPerThread = (kMaxCq * kMaxCk * kDwRowGroups + NT - 1) / NT;
+
+__host__ __device__ inline size_t bwd_lds_floats(int d, int pq, int pk, int ntap) {
+    constexpr int TC = kGenBwdTC;
+    const size_t kv = (size_t)(TC + 4 * pk) * (d + 4) > (size_t)TC * (d + 16) ? (size_t)(TC + 4 * pk) * (d + 4)
+                                                                               : (size_t)TC * (d + 16);
+    return (size_t)(TR + 2 * pq) * (d + 4) + (size_t)(TR + pq) * (d + 4) + kv +
+           (size_t)(TR + 2 * pq) * (TC + 4 * pk + 1) + (size_t)(TR + pq) * (TC + 2 * pk + 1) + 2 * (size_t)TR * (TC + 4) +
+           ntap + 2 * (TR + pq) + (size_t)kDwRowGroups * ntap;
+}
 
 template <int TC>
 __device__ __forceinline__ BwdLds carve_bwd(float *lds, const Problem &p) {
     BwdLds t;
-    const int d = p.d, pq = p.pq, pk = p.pk;
-    t.kst = d + 1;
+    const int d = p.d, pq = p.pq, pk = p.pk, ntap = p.c_q * p.c_k;
+    t.qst = d + 4; t.gst = d + 4; t.kst = d + 4; t.kst2 = d + 16;
     t.sst = TC + 4 * pk + 1;
     t.cst = TC + 2 * pk + 1;
-    t.pst = TC + 1;
+    t.pst = TC + 4;
+    const int kv = max((TC + 4 * pk) * t.kst, TC * t.kst2);
     t.Qs = lds;
-    t.dOs = t.Qs + (TR + 2 * pq) * d;
-    t.KVs = t.dOs + (TR + pq) * d;
-    t.Ss = t.KVs + (TC + 4 * pk) * t.kst;
+    t.dOs = t.Qs + (TR + 2 * pq) * t.qst;
+    t.KVs = t.dOs + (TR + pq) * t.gst;
+    t.Ss = t.KVs + kv;
     t.dCs = t.Ss + (TR + 2 * pq) * t.sst;
     t.Ps = t.dCs + (TR + pq) * t.cst;
     t.dSs = t.Ps + TR * t.pst;
     t.Ws = t.dSs + TR * t.pst;
-    t.lse_s = t.Ws + p.c_q * p.c_k;
+    t.lse_s = t.Ws + ntap;
     t.D_s = t.lse_s + (TR + pq);
+    t.red = t.D_s + (TR + pq);   // dW partial sums of the row groups
     return t;
 }
 
@@ -178,8 +322,8 @@ __device__ __forceinline__ BwdLds carve_bwd(float *lds, const Problem &p) {
 template <typename TI>
 __device__ __forceinline__ void load_q_side(const BwdLds &t, const Problem &p, const TI *Qb,
                                             const TI *dOb, const float *lse, const float *D, int r0) {
-    load_rows(t.Qs, p.d, Qb, r0 - p.pq, TR + 2 * p.pq, p.Nq, p.d);
-    load_rows(t.dOs, p.d, dOb, r0, TR + p.pq, p.Nq, p.d);
+    load_rows(t.Qs, t.qst, Qb, r0 - p.pq, TR + 2 * p.pq, p.Nq, p.d);
+    load_rows(t.dOs, t.gst, dOb, r0, TR + p.pq, p.Nq, p.d);
     for (int i = threadIdx.x; i < TR + p.pq; i += NT) {
         int g = r0 + i;
         t.lse_s[i] = g < p.Nq ? lse[g] : 0.f;
@@ -198,30 +342,33 @@ __device__ __forceinline__ void bwd_tile(const BwdLds &t, const Problem &p, cons
     const int pq = p.pq, pk = p.pk, d = p.d;
     load_rows(t.KVs, t.kst, Kb, c0 - 2 * pk, TC + 4 * pk, p.Nk, d);
     __syncthreads();
-    score_tile(t.Ss, t.sst, t.Qs, d, t.KVs, t.kst, TR + 2 * pq, TC + 4 * pk, d, r0 - pq, c0 - 2 * pk,
-               p.scale, p.causal);
+    score_tile_mma(t.Ss, t.sst, t.Qs, t.qst, t.KVs, t.kst, TR + 2 * pq, TC + 4 * pk, d, r0 - pq, c0 - 2 * pk,
+                   p.scale, p.causal);
     __syncthreads();
     load_rows(t.KVs, t.kst, Vb, c0 - pk, TC + 2 * pk, p.Nk, d);
     __syncthreads();
     const int nr = TR + pq, nc = TC + 2 * pk;
-    for (int idx = threadIdx.x; idx < nr * nc; idx += NT) {
-        int i = idx / nc, j = idx - i * nc;
-        int qi = r0 + i, kj = c0 - pk + j;
-        float P = 0.f, dC = 0.f;
-        if (qi < p.Nq && kj >= 0 && kj < p.Nk && !(p.causal && kj > qi)) {
-            float c = 0.f;
-            for (int a = 0; a < p.c_q; ++a)
-                for (int bb = 0; bb < p.c_k; ++bb)
-                    c = fmaf(t.Ws[a * p.c_k + bb], t.Ss[(i + a) * t.sst + j + bb], c);
-            P = __expf(c - t.lse_s[i]);
-            const float *g = t.dOs + i * d;
-            const float *vv = t.KVs + j * t.kst;
-            float dP = 0.f;
-            for (int x = 0; x < d; ++x) dP = fmaf(g[x], vv[x], dP);
-            dC = P * (dP - t.D_s[i]);
+    // dP = dO V^T into dCs (scale 1, no mask), then dC = P (dP - D) in place
+    score_tile_mma(t.dCs, t.cst, t.dOs, t.gst, t.KVs, t.kst, nr, nc, d, 0, 0, 1.f, 0);
+    __syncthreads();
+    const int ng = (nc + 3) / 4;   // groups of four adjacent keys per row
+    for (int idx = threadIdx.x; idx < nr * ng; idx += NT) {
+        const int i = idx / ng, j0 = (idx - i * ng) * 4;
+        float c[4];
+        conv4(c, t.Ws, p.c_q, p.c_k, t.Ss + i * t.sst + j0, t.sst);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int j = j0 + k, qi = r0 + i, kj = c0 - pk + j;
+            if (j < nc) {
+                float P = 0.f, dC = 0.f;
+                if (qi < p.Nq && kj >= 0 && kj < p.Nk && !(p.causal && kj > qi)) {
+                    P = __expf(c[k] - t.lse_s[i]);
+                    dC = P * (t.dCs[i * t.cst + j] - t.D_s[i]);
+                }
+                t.dCs[i * t.cst + j] = dC;
+                if (i < TR && j >= pk && j < pk + TC) t.Ps[i * t.pst + j - pk] = P;
+            }
         }
-        t.dCs[i * t.cst + j] = dC;
-        if (i < TR && j >= pk && j < pk + TC) t.Ps[i * t.pst + j - pk] = P;
     }
     __syncthreads();
 }
@@ -230,16 +377,15 @@ __device__ __forceinline__ void bwd_tile(const BwdLds &t, const Problem &p, cons
 template <int TC>
 __device__ __forceinline__ void dscore_tile(const BwdLds &t, const Problem &p, int r0, int c0) {
     const int pq = p.pq, pk = p.pk;
-    for (int idx = threadIdx.x; idx < TR * TC; idx += NT) {
-        int r = idx / TC, c = idx - r * TC;
-        int qi = r0 + r, kj = c0 + c;
-        float s = 0.f;
-        if (qi < p.Nq && kj < p.Nk && !(p.causal && kj > qi)) {
-            for (int a = 0; a < p.c_q; ++a)
-                for (int bb = 0; bb < p.c_k; ++bb)
-                    s = fmaf(t.Ws[a * p.c_k + bb], t.dCs[(r - a + pq) * t.cst + c - bb + 2 * pk], s);
+    for (int idx = threadIdx.x; idx < TR * TC / 4; idx += NT) {
+        const int r = idx / (TC / 4), c = (idx - r * (TC / 4)) * 4;
+        float s[4];
+        conv4_t(s, t.Ws, p.c_q, p.c_k, t.dCs + (r + pq) * t.cst + c + 2 * pk, t.cst);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int qi = r0 + r, kj = c0 + c + k;
+            t.dSs[r * t.pst + c + k] = (qi < p.Nq && kj < p.Nk && !(p.causal && kj > qi)) ? s[k] : 0.f;
         }
-        t.dSs[r * t.pst + c] = s;
     }
 }
 
@@ -262,59 +408,74 @@ __global__ __launch_bounds__(NT) void gen_dq_dw_kernel(
     for (int i = tid; i < ntap; i += NT) t.Ws[i] = W[(size_t)h * ntap + i];
     load_q_side(t, p, Qb, dOb, LSE + bh * p.Nq, D + bh * p.Nq, r0);
 
-    const int orow = tid >> 4, ocol = tid & 15;
-    float acc[kMaxD / 16];
+    // dQ: a wave holds the 16 x 16 blocks wave, wave + 4 of the head dimension
+    const int wave = tid >> 6, lane = tid & 63, g = lane >> 4, n = lane & 15;
+    f32x4 acc[kMaxD / 16 / NWV];
 #pragma unroll
-    for (int u = 0; u < kMaxD / 16; ++u) acc[u] = 0.f;
-    constexpr int kTapsPerThread = (kMaxCq * kMaxCk + NT - 1) / NT;
-    float dw_acc[kTapsPerThread];
+    for (int u = 0; u < kMaxD / 16 / NWV; ++u) acc[u] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    // dW: thread t adds up the work items t, t + NT, ... (item = tap * 8 + row group) over all tiles
+    float dw_acc[kDwItemsPerThread];
 #pragma unroll
-    for (int u = 0; u < kTapsPerThread; ++u) dw_acc[u] = 0.f;
+    for (int u = 0; u < kDwItemsPerThread; ++u) dw_acc[u] = 0.f;
 
     const int kend = p.causal ? min(p.Nk, r0 + TR) : p.Nk;
     for (int c0 = 0; c0 < kend; c0 += TC) {
         bwd_tile<TI, TC>(t, p, Kb, Vb, r0, c0);
-        load_rows(t.KVs, t.kst, Kb, c0, TC, p.Nk, d);  // own keys, for dQ += dS K
+        load_rows(t.KVs, t.kst2, Kb, c0, TC, p.Nk, d);  // own keys, for dQ += dS K
         dscore_tile<TC>(t, p, r0, c0);
-        // dW[a][b] += dC[i][j] * S_m[i + a - pq][j + b - pk] over this tile's own
-        // (row, key) pairs; a thread owns whole taps, so the order is fixed.
+        // dW[a][b] += dC[i][j] * S_m[i + a - pq][j + b - pk] over this tile's own (row, key) pairs,
+        // always in the same order
 #pragma unroll
-        for (int u = 0; u < kTapsPerThread; ++u) {
-            int tap = tid + u * NT;
-            if (tap < ntap) {
-                int a = tap / p.c_k, bb = tap - a * p.c_k;
-                float s = dw_acc[u];
-                for (int i = 0; i < TR; ++i)
-                    for (int j = 0; j < TC; ++j)
-                        s = fmaf(t.dCs[i * t.cst + j + pk], t.Ss[(i + a) * t.sst + j + pk + bb], s);
-                dw_acc[u] = s;
+        for (int u = 0; u < kDwItemsPerThread; ++u) {
+            const int item = tid + u * NT;
+            if (item < ntap * kDwRowGroups) {
+                const int tap = item / kDwRowGroups, rg = item - tap * kDwRowGroups;
+                const int a = tap / p.c_k, bb = tap - a * p.c_k;
+                float s4[4] = {0.f, 0.f, 0.f, 0.f};   // four independent sums, added in a fixed order
+                for (int i = rg * (TR / kDwRowGroups); i < (rg + 1) * (TR / kDwRowGroups); ++i) {
+                    const float *dc = t.dCs + i * t.cst + pk, *sr = t.Ss + (i + a) * t.sst + pk + bb;
+#pragma unroll 2
+                    for (int j = 0; j < TC; j += 4) {
+                        s4[0] = fmaf(dc[j], sr[j], s4[0]);
+                        s4[1] = fmaf(dc[j + 1], sr[j + 1], s4[1]);
+                        s4[2] = fmaf(dc[j + 2], sr[j + 2], s4[2]);
+                        s4[3] = fmaf(dc[j + 3], sr[j + 3], s4[3]);
+                    }
+                }
+                dw_acc[u] += (s4[0] + s4[1]) + (s4[2] + s4[3]);
             }
         }
         __syncthreads();
+        {
+            const float *bp[kMaxD / 16 / NWV];
 #pragma unroll
-        for (int u = 0; u < kMaxD / 16; ++u) {
-            int dc = ocol + 16 * u;
-            if (dc < d) {
-                float s = acc[u];
-                for (int c = 0; c < TC; ++c) s = fmaf(t.dSs[orow * t.pst + c], t.KVs[c * t.kst + dc], s);
-                acc[u] = s;
-            }
+            for (int u = 0; u < kMaxD / 16 / NWV; ++u) bp[u] = t.KVs + g * t.kst2 + min((wave + NWV * u) * 16 + n, d - 1);
+            lds_mma_n<kMaxD / 16 / NWV>(acc, t.dSs + n * t.pst + g, 1, bp, t.kst2, TC);
         }
         __syncthreads();
     }
-    const int qi = r0 + orow;
-    if (qi < p.Nq) {
 #pragma unroll
-        for (int u = 0; u < kMaxD / 16; ++u) {
-            int dc = ocol + 16 * u;
-            if (dc < d) dQ[(bh * p.Nq + qi) * d + dc] = from_f32<TO>(acc[u] * p.scale);
+    for (int u = 0; u < kMaxD / 16 / NWV; ++u) {
+        const int dc = (wave + NWV * u) * 16 + n;
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+            const int qi = r0 + 4 * g + rr;
+            if (qi < p.Nq && dc < d) dQ[(bh * p.Nq + qi) * d + dc] = from_f32<TO>(acc[u][rr] * p.scale);
         }
     }
+    // the row groups' sums, added in group order
+#pragma unroll
+    for (int u = 0; u < kDwItemsPerThread; ++u) {
+        const int item = tid + u * NT;
+        if (item < ntap * kDwRowGroups) t.red[item] = dw_acc[u];   // [tap][row group]
+    }
+    __syncthreads();
     float *part = dW_part + (bh * gridDim.x + qt) * ntap;
+    for (int tap = tid; tap < ntap; tap += NT) {
+        float sum = 0.f;
 #pragma unroll
-    for (int u = 0; u < kTapsPerThread; ++u) {
-        int tap = tid + u * NT;
-        if (tap < ntap) part[tap] = dw_acc[u];
+        for (int rg = 0; rg < kDwRowGroups; ++rg) sum += t.red[tap * kDwRowGroups + rg];
+        part[tap] = sum;
     }
 }
 
@@ -336,10 +497,13 @@ __global__ __launch_bounds__(NT) void gen_dkdv_kernel(
 
     for (int i = tid; i < ntap; i += NT) t.Ws[i] = W[(size_t)h * ntap + i];
 
-    const int ocol = tid >> 3, oph = tid & 7;  // this thread's key and column phase
-    float acc_k[kMaxD / 8], acc_v[kMaxD / 8];
+    // dK, dV: TC keys x d = (TC / 16) x (d / 16) blocks each; a wave holds the blocks wave, wave + 4, ...
+    // (block x: keys 16 (x % (TC / 16)) .., head-dim columns 16 (x / (TC / 16)) ..; lane (g, n): keys 4g .. 4g+3)
+    constexpr int KB = TC / 16, NBLK = KB * (kMaxD / 16) / NWV;
+    const int wave = tid >> 6, lane = tid & 63, g = lane >> 4, n = lane & 15;
+    f32x4 acc_k[NBLK], acc_v[NBLK];
 #pragma unroll
-    for (int u = 0; u < kMaxD / 8; ++u) { acc_k[u] = 0.f; acc_v[u] = 0.f; }
+    for (int u = 0; u < NBLK; ++u) acc_k[u] = acc_v[u] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
     // Causal: rows before the tile's first key see none of its keys.
     const int rstart = p.causal ? (c0 / TR) * TR : 0;
@@ -349,28 +513,28 @@ __global__ __launch_bounds__(NT) void gen_dkdv_kernel(
         bwd_tile<TI, TC>(t, p, Kb, Vb, r0, c0);
         dscore_tile<TC>(t, p, r0, c0);
         __syncthreads();
+        // dV[key][:] += sum_r P[r][key] dO[r][:], dK[key][:] += sum_r dS[r][key] Q[r][:]  (A(m = key, k = r));
+        // eight independent accumulators per wave
+        for (int k = 0; k < TR; k += 4) {
 #pragma unroll
-        for (int u = 0; u < kMaxD / 8; ++u) {
-            int dc = oph + 8 * u;
-            if (dc < d) {
-                float sk = acc_k[u], sv = acc_v[u];
-                for (int r = 0; r < TR; ++r) {
-                    sv = fmaf(t.Ps[r * t.pst + ocol], t.dOs[r * d + dc], sv);
-                    sk = fmaf(t.dSs[r * t.pst + ocol], t.Qs[(r + pq) * d + dc], sk);
-                }
-                acc_k[u] = sk;
-                acc_v[u] = sv;
+            for (int u = 0; u < NBLK; ++u) {
+                const int x = wave + NWV * u, kb = x % KB, dc = min((x / KB) * 16 + n, d - 1);
+                acc_v[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(t.Ps[(k + g) * t.pst + kb * 16 + n],
+                                                                t.dOs[(k + g) * t.gst + dc], acc_v[u], 0, 0, 0);
+                acc_k[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(t.dSs[(k + g) * t.pst + kb * 16 + n],
+                                                                t.Qs[(k + g + pq) * t.qst + dc], acc_k[u], 0, 0, 0);
             }
         }
     }
-    const int kj = c0 + ocol;
-    if (kj < p.Nk) {
 #pragma unroll
-        for (int u = 0; u < kMaxD / 8; ++u) {
-            int dc = oph + 8 * u;
-            if (dc < d) {
-                dK[(bh * p.Nk + kj) * d + dc] = from_f32<TO>(acc_k[u] * p.scale);
-                dV[(bh * p.Nk + kj) * d + dc] = from_f32<TO>(acc_v[u]);
+    for (int u = 0; u < NBLK; ++u) {
+        const int x = wave + NWV * u, kb = x % KB, dc = (x / KB) * 16 + n;
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+            const int kj = c0 + kb * 16 + 4 * g + rr;
+            if (kj < p.Nk && dc < d) {
+                dK[(bh * p.Nk + kj) * d + dc] = from_f32<TO>(acc_k[u][rr] * p.scale);
+                dV[(bh * p.Nk + kj) * d + dc] = from_f32<TO>(acc_v[u][rr]);
             }
         }
     }
@@ -458,21 +622,9 @@ hipError_t allow_lds(F kernel, size_t bytes) {
 
 }  // namespace
 
-size_t generic_fwd_lds(const Problem &p) {
-    const int QR = TR + p.pq, SC = kGenFwdTC + 2 * p.pk;
-    size_t f = (size_t)QR * p.d + (size_t)SC * (p.d + 1) + (size_t)QR * (SC + 1) + TR * kGenFwdTC +
-               p.c_q * p.c_k + 3 * TR;
-    return f * sizeof(float);
-}
+size_t generic_fwd_lds(const Problem &p) { return fwd_lds_floats(p.d, p.pq, p.pk, p.c_q * p.c_k) * sizeof(float); }
 
-size_t generic_bwd_lds(const Problem &p) {
-    constexpr int TC = kGenBwdTC;
-    size_t f = (size_t)(TR + 2 * p.pq) * p.d + (size_t)(TR + p.pq) * p.d +
-               (size_t)(TC + 4 * p.pk) * (p.d + 1) + (size_t)(TR + 2 * p.pq) * (TC + 4 * p.pk + 1) +
-               (size_t)(TR + p.pq) * (TC + 2 * p.pk + 1) + 2 * TR * (TC + 1) + p.c_q * p.c_k +
-               2 * (TR + p.pq);
-    return f * sizeof(float);
-}
+size_t generic_bwd_lds(const Problem &p) { return bwd_lds_floats(p.d, p.pq, p.pk, p.c_q * p.c_k) * sizeof(float); }
 
 size_t generic_decode_lds(const Problem &p) {
     const int SC = kGenDecTC + 2 * p.pk;
