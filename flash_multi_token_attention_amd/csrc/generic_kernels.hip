@@ -55,6 +55,55 @@ __device__ __forceinline__ void load_rows(float *dst, int stride, const T *src, 
     }
 }
 
+// The same in two steps, for tiles that are loaded while the tile before them is worked on: issue()
+// starts the loads of this thread's pieces (8 elements each, MAXP pieces at most), commit() converts
+// them and writes them to LDS.
+template <typename T, int MAXP>
+struct RowPieces {
+    static constexpr int Q = sizeof(T) == 2 ? 1 : 2;   // 16-byte quantities per piece
+    uint4 raw[MAXP * Q];
+    __device__ __forceinline__ void issue(const T *src, int row0, int nrows, int N, int d) {
+        const int cpr = d / 8;
+#pragma unroll
+        for (int i = 0; i < MAXP; ++i) {
+            const int idx = threadIdx.x + i * NT, r = idx / cpr, c = (idx - r * cpr) * 8, g = row0 + r;
+#pragma unroll
+            for (int q = 0; q < Q; ++q) raw[i * Q + q] = make_uint4(0u, 0u, 0u, 0u);
+            if (idx < nrows * cpr && g >= 0 && g < N) {
+                const uint4 *ptr = reinterpret_cast<const uint4 *>(src + (size_t)g * d + c);
+#pragma unroll
+                for (int q = 0; q < Q; ++q) raw[i * Q + q] = ptr[q];
+            }
+        }
+    }
+    __device__ __forceinline__ void commit(float *dst, int stride, int nrows, int d) const {
+        const int cpr = d / 8;
+#pragma unroll
+        for (int i = 0; i < MAXP; ++i) {
+            const int idx = threadIdx.x + i * NT, r = idx / cpr, c = (idx - r * cpr) * 8;
+            if (idx < nrows * cpr) {
+                float4 lo, hi;
+                if constexpr (Q == 1) {
+                    const unsigned int w[4] = {raw[i].x, raw[i].y, raw[i].z, raw[i].w};
+                    lo = make_float4(__uint_as_float(w[0] << 16), __uint_as_float(w[0] & 0xffff0000u),
+                                     __uint_as_float(w[1] << 16), __uint_as_float(w[1] & 0xffff0000u));
+                    hi = make_float4(__uint_as_float(w[2] << 16), __uint_as_float(w[2] & 0xffff0000u),
+                                     __uint_as_float(w[3] << 16), __uint_as_float(w[3] & 0xffff0000u));
+                } else {
+                    lo = make_float4(__uint_as_float(raw[2 * i].x), __uint_as_float(raw[2 * i].y),
+                                     __uint_as_float(raw[2 * i].z), __uint_as_float(raw[2 * i].w));
+                    hi = make_float4(__uint_as_float(raw[2 * i + 1].x), __uint_as_float(raw[2 * i + 1].y),
+                                     __uint_as_float(raw[2 * i + 1].z), __uint_as_float(raw[2 * i + 1].w));
+                }
+                float *out = dst + r * stride + c;   // (strides of the tiles loaded this way are multiples of 4 floats)
+                *reinterpret_cast<float4 *>(out) = lo;
+                *reinterpret_cast<float4 *>(out + 4) = hi;
+            }
+        }
+    }
+};
+constexpr int pieces_per_thread(int rows) { return (rows * (kMaxD / 8) + NT - 1) / NT; }
+
 // S[r][c] = scale * <A[r], Kt[c]> for r < nr, c < nc on the vector ALUs (the decode kernel's few rows);
 // the causal pre-mask zeroes keys after the row's own position.
 __device__ __forceinline__ void score_tile(float *S, int sstride, const float *A, int astride,
@@ -73,42 +122,72 @@ __device__ __forceinline__ void score_tile(float *S, int sstride, const float *A
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-// Four adjacent outputs of the convolution, out[k] = sum_ab W[a][b] * X[(a) rows down][k + b columns on],
+// Four adjacent outputs of the convolution, out[k] = sum_ab W[a][b] * X[a rows down][k + b columns on],
 // with `x` pointing at the window's first element for output 0: one new tile element and one weight
-// are read per four multiply-adds, and the four sums are independent.
-__device__ __forceinline__ void conv4(float (&out)[4], const float *Ws, int c_q, int c_k, const float *x, int xstride) {
+// are read per four multiply-adds, and the four sums are independent.  CK > 0: the number of key taps
+// as a constant, so that the reads of a tap row are all issued before its multiply-adds (with a
+// run-time bound every few taps wait for their LDS reads).  FLIP: the transposed convolution,
+// out[k] = sum_ab W[a][b] * X[a rows UP][k - b columns], `x` at the element under output 0 for tap (0, 0).
+template <int CK, bool FLIP>
+__device__ __forceinline__ void conv4_impl(float (&out)[4], const float *Ws, int c_q, int c_k, const float *x, int xstride) {
     out[0] = out[1] = out[2] = out[3] = 0.f;
+    const int ck = CK > 0 ? CK : c_k;
     for (int a = 0; a < c_q; ++a) {
-        const float *row = x + a * xstride, *w = Ws + a * c_k;
-        float s0 = row[0], s1 = row[1], s2 = row[2];
+        const float *row = FLIP ? x - a * xstride : x + a * xstride, *w = Ws + a * ck;
+        if constexpr (CK > 0) {
+            float seg[CK + 3], wv[CK];
+#pragma unroll
+            for (int i = 0; i < CK + 3; ++i) seg[i] = FLIP ? row[3 - i] : row[i];   // FLIP: seg[i] = X[.. 3 - i]
+#pragma unroll
+            for (int bb = 0; bb < CK; ++bb) wv[bb] = w[bb];
+#pragma unroll
+            for (int bb = 0; bb < CK; ++bb) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) out[k] = fmaf(wv[bb], FLIP ? seg[3 - k + bb] : seg[k + bb], out[k]);
+            }
+        } else if constexpr (!FLIP) {
+            float s0 = row[0], s1 = row[1], s2 = row[2];
 #pragma unroll 4
-        for (int bb = 0; bb < c_k; ++bb) {
-            const float s3 = row[bb + 3], wv = w[bb];
-            out[0] = fmaf(wv, s0, out[0]);
-            out[1] = fmaf(wv, s1, out[1]);
-            out[2] = fmaf(wv, s2, out[2]);
-            out[3] = fmaf(wv, s3, out[3]);
-            s0 = s1; s1 = s2; s2 = s3;
+            for (int bb = 0; bb < ck; ++bb) {
+                const float s3 = row[bb + 3], wv = w[bb];
+                out[0] = fmaf(wv, s0, out[0]);
+                out[1] = fmaf(wv, s1, out[1]);
+                out[2] = fmaf(wv, s2, out[2]);
+                out[3] = fmaf(wv, s3, out[3]);
+                s0 = s1; s1 = s2; s2 = s3;
+            }
+        } else {
+            float s1 = row[1], s2 = row[2], s3 = row[3];
+#pragma unroll 4
+            for (int bb = 0; bb < ck; ++bb) {
+                const float s0 = row[-bb], wv = w[bb];
+                out[0] = fmaf(wv, s0, out[0]);
+                out[1] = fmaf(wv, s1, out[1]);
+                out[2] = fmaf(wv, s2, out[2]);
+                out[3] = fmaf(wv, s3, out[3]);
+                s3 = s2; s2 = s1; s1 = s0;
+            }
         }
     }
 }
-// The transposed convolution: out[k] = sum_ab W[a][b] * X[a rows UP][k - b columns], `x` pointing at the
-// element under output 0 for tap (0, 0).
-__device__ __forceinline__ void conv4_t(float (&out)[4], const float *Ws, int c_q, int c_k, const float *x, int xstride) {
-    out[0] = out[1] = out[2] = out[3] = 0.f;
-    for (int a = 0; a < c_q; ++a) {
-        const float *row = x - a * xstride, *w = Ws + a * c_k;
-        float s1 = row[1], s2 = row[2], s3 = row[3];
-#pragma unroll 4
-        for (int bb = 0; bb < c_k; ++bb) {
-            const float s0 = row[-bb], wv = w[bb];
-            out[0] = fmaf(wv, s0, out[0]);
-            out[1] = fmaf(wv, s1, out[1]);
-            out[2] = fmaf(wv, s2, out[2]);
-            out[3] = fmaf(wv, s3, out[3]);
-            s3 = s2; s2 = s1; s1 = s0;
-        }
+template <bool FLIP>
+__device__ __forceinline__ void conv4_any(float (&out)[4], const float *Ws, int c_q, int c_k, const float *x, int xstride) {
+    switch (c_k) {   // (workgroup-uniform)
+        case 3: conv4_impl<3, FLIP>(out, Ws, c_q, c_k, x, xstride); break;
+        case 5: conv4_impl<5, FLIP>(out, Ws, c_q, c_k, x, xstride); break;
+        case 7: conv4_impl<7, FLIP>(out, Ws, c_q, c_k, x, xstride); break;
+        case 9: conv4_impl<9, FLIP>(out, Ws, c_q, c_k, x, xstride); break;
+        case 11: conv4_impl<11, FLIP>(out, Ws, c_q, c_k, x, xstride); break;
+        case 13: conv4_impl<13, FLIP>(out, Ws, c_q, c_k, x, xstride); break;
+        case 15: conv4_impl<15, FLIP>(out, Ws, c_q, c_k, x, xstride); break;
+        default: conv4_impl<0, FLIP>(out, Ws, c_q, c_k, x, xstride); break;
     }
+}
+__device__ __forceinline__ void conv4(float (&out)[4], const float *Ws, int c_q, int c_k, const float *x, int xstride) {
+    conv4_any<false>(out, Ws, c_q, c_k, x, xstride);
+}
+__device__ __forceinline__ void conv4_t(float (&out)[4], const float *Ws, int c_q, int c_k, const float *x, int xstride) {
+    conv4_any<true>(out, Ws, c_q, c_k, x, xstride);
 }
 
 // NB 16 x 16 blocks at once that share the left operand: acc[u] (lane (g, n): rows 4g .. 4g+3, column n)
@@ -218,13 +297,19 @@ __global__ __launch_bounds__(NT) void gen_fwd_kernel(Problem p, const TI *__rest
 #pragma unroll
     for (int u = 0; u < kMaxD / 16 / NWV; ++u) acc[u] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
+    // The K rows of a tile are loaded during the tile before it, its V rows during its score phase.
+    RowPieces<TI, pieces_per_thread(kGenFwdTC + 2 * ((kMaxCk - 1) / 2))> kp;
+    RowPieces<TI, pieces_per_thread(kGenFwdTC)> vp;
     const int kend = p.causal ? min(p.Nk, r0 + TR) : p.Nk;
+    kp.issue(Kb, -pk, SC, p.Nk, d);
     for (int c0 = 0; c0 < kend; c0 += TC) {
-        load_rows(KVs, kst, Kb, c0 - pk, SC, p.Nk, d);
+        kp.commit(KVs, kst, SC, d);
+        vp.issue(Vb, c0, TC, p.Nk, d);
         __syncthreads();
         score_tile_mma(Ss, sst, Qs, qst, KVs, kst, QR, SC, d, r0 - pq, c0 - pk, p.scale, p.causal);
         __syncthreads();
-        load_rows(KVs, vst, Vb, c0, TC, p.Nk, d);  // V replaces K
+        vp.commit(KVs, vst, TC, d);  // V replaces K
+        if (c0 + TC < kend) kp.issue(Kb, c0 + TC - pk, SC, p.Nk, d);
         for (int idx = tid; idx < TR * TC / 4; idx += NT) {
             const int i = idx / (TC / 4), j = (idx - i * (TC / 4)) * 4;
             float c[4];
@@ -317,35 +402,47 @@ __device__ __forceinline__ BwdLds carve_bwd(float *lds, const Problem &p) {
     return t;
 }
 
-// Loads what depends on the query tile: Q rows r0-pq .. r0+TR+pq-1, dO / LSE / D
-// rows r0 .. r0+TR+pq-1.
+// What depends on the query tile: Q rows r0-pq .. r0+TR+pq-1, dO / LSE / D rows r0 .. r0+TR+pq-1
+// (TR + pq <= 31 rows: one LSE / D entry per thread), loaded in two steps like the tiles.
 template <typename TI>
-__device__ __forceinline__ void load_q_side(const BwdLds &t, const Problem &p, const TI *Qb,
-                                            const TI *dOb, const float *lse, const float *D, int r0) {
-    load_rows(t.Qs, t.qst, Qb, r0 - p.pq, TR + 2 * p.pq, p.Nq, p.d);
-    load_rows(t.dOs, t.gst, dOb, r0, TR + p.pq, p.Nq, p.d);
-    for (int i = threadIdx.x; i < TR + p.pq; i += NT) {
-        int g = r0 + i;
-        t.lse_s[i] = g < p.Nq ? lse[g] : 0.f;
-        t.D_s[i] = g < p.Nq ? D[g] : 0.f;
+struct QSide {
+    RowPieces<TI, pieces_per_thread(TR + 2 * (kMaxCq - 1))> qp;
+    RowPieces<TI, pieces_per_thread(TR + kMaxCq - 1)> gp;
+    float ls, dd;
+    __device__ __forceinline__ void issue(const Problem &p, const TI *Qb, const TI *dOb, const float *lse, const float *D,
+                                          int r0) {
+        qp.issue(Qb, r0 - p.pq, TR + 2 * p.pq, p.Nq, p.d);
+        gp.issue(dOb, r0, TR + p.pq, p.Nq, p.d);
+        const int g = r0 + (int)threadIdx.x;
+        ls = 0.f; dd = 0.f;
+        if ((int)threadIdx.x < TR + p.pq && g < p.Nq) { ls = lse[g]; dd = D[g]; }
     }
-}
+    __device__ __forceinline__ void commit(const BwdLds &t, const Problem &p) const {
+        qp.commit(t.Qs, t.qst, TR + 2 * p.pq, p.d);
+        gp.commit(t.dOs, t.gst, TR + p.pq, p.d);
+        if ((int)threadIdx.x < TR + p.pq) { t.lse_s[threadIdx.x] = ls; t.D_s[threadIdx.x] = dd; }
+    }
+};
 
 // For query tile r0 and key tile c0 (query side already in LDS) leaves in LDS:
 //   Ss  = S_m  rows r0-pq .. r0+TR+pq-1, keys c0-2pk .. c0+TC+2pk-1
 //   dCs = dC   rows r0    .. r0+TR+pq-1, keys c0-pk  .. c0+TC+pk-1
 //   Ps  = P    rows r0    .. r0+TR-1,    keys c0     .. c0+TC-1
-// Ends with a barrier; KVs is free afterwards.
-template <typename TI, int TC>
-__device__ __forceinline__ void bwd_tile(const BwdLds &t, const Problem &p, const TI *Kb,
-                                         const TI *Vb, int r0, int c0) {
+// Ends with a barrier; KVs is free afterwards.  The K rows (c0-2pk .. c0+TC+2pk-1) are on their way in `kp`
+// when this is called; the V rows are loaded during the score phase; `after_v` is where the caller starts
+// the loads it needs next.
+template <typename TI, int TC, typename KP, typename VP, typename Hook>
+__device__ __forceinline__ void bwd_tile(const BwdLds &t, const Problem &p, KP &kp, VP &vp, const TI *Vb, int r0, int c0,
+                                         Hook &&after_v) {
     const int pq = p.pq, pk = p.pk, d = p.d;
-    load_rows(t.KVs, t.kst, Kb, c0 - 2 * pk, TC + 4 * pk, p.Nk, d);
+    kp.commit(t.KVs, t.kst, TC + 4 * pk, d);
+    vp.issue(Vb, c0 - pk, TC + 2 * pk, p.Nk, d);
     __syncthreads();
     score_tile_mma(t.Ss, t.sst, t.Qs, t.qst, t.KVs, t.kst, TR + 2 * pq, TC + 4 * pk, d, r0 - pq, c0 - 2 * pk,
                    p.scale, p.causal);
     __syncthreads();
-    load_rows(t.KVs, t.kst, Vb, c0 - pk, TC + 2 * pk, p.Nk, d);
+    vp.commit(t.KVs, t.kst, TC + 2 * pk, d);
+    after_v();
     __syncthreads();
     const int nr = TR + pq, nc = TC + 2 * pk;
     // dP = dO V^T into dCs (scale 1, no mask), then dC = P (dP - D) in place
@@ -406,7 +503,15 @@ __global__ __launch_bounds__(NT) void gen_dq_dw_kernel(
     const TI *Kb = K + bh * p.Nk * d, *Vb = V + bh * p.Nk * d;
 
     for (int i = tid; i < ntap; i += NT) t.Ws[i] = W[(size_t)h * ntap + i];
-    load_q_side(t, p, Qb, dOb, LSE + bh * p.Nq, D + bh * p.Nq, r0);
+    {
+        QSide<TI> qs;
+        qs.issue(p, Qb, dOb, LSE + bh * p.Nq, D + bh * p.Nq, r0);
+        qs.commit(t, p);
+    }
+    constexpr int PKM = (kMaxCk - 1) / 2;
+    RowPieces<TI, pieces_per_thread(TC + 4 * PKM)> kp;   // K rows of the next tile
+    RowPieces<TI, pieces_per_thread(TC + 2 * PKM)> vp;   // V rows of this tile
+    RowPieces<TI, pieces_per_thread(TC)> op;             // this tile's own keys again, for dQ += dS K
 
     // dQ: a wave holds the 16 x 16 blocks wave, wave + 4 of the head dimension
     const int wave = tid >> 6, lane = tid & 63, g = lane >> 4, n = lane & 15;
@@ -419,9 +524,11 @@ __global__ __launch_bounds__(NT) void gen_dq_dw_kernel(
     for (int u = 0; u < kDwItemsPerThread; ++u) dw_acc[u] = 0.f;
 
     const int kend = p.causal ? min(p.Nk, r0 + TR) : p.Nk;
+    kp.issue(Kb, -2 * pk, TC + 4 * pk, p.Nk, d);
     for (int c0 = 0; c0 < kend; c0 += TC) {
-        bwd_tile<TI, TC>(t, p, Kb, Vb, r0, c0);
-        load_rows(t.KVs, t.kst2, Kb, c0, TC, p.Nk, d);  // own keys, for dQ += dS K
+        bwd_tile<TI, TC>(t, p, kp, vp, Vb, r0, c0, [&] { op.issue(Kb, c0, TC, p.Nk, d); });
+        op.commit(t.KVs, t.kst2, TC, d);
+        if (c0 + TC < kend) kp.issue(Kb, c0 + TC - 2 * pk, TC + 4 * pk, p.Nk, d);
         dscore_tile<TC>(t, p, r0, c0);
         // dW[a][b] += dC[i][j] * S_m[i + a - pq][j + b - pk] over this tile's own (row, key) pairs,
         // always in the same order
@@ -505,12 +612,24 @@ __global__ __launch_bounds__(NT) void gen_dkdv_kernel(
 #pragma unroll
     for (int u = 0; u < NBLK; ++u) acc_k[u] = acc_v[u] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
+    constexpr int PKM = (kMaxCk - 1) / 2;
+    RowPieces<TI, pieces_per_thread(TC + 4 * PKM)> kp;   // the K rows (the same for every row tile: KVs also holds V)
+    RowPieces<TI, pieces_per_thread(TC + 2 * PKM)> vp;
+    QSide<TI> qs;                                        // the next row tile's Q, dO, LSE, D
+    const int pk = p.pk;
     // Causal: rows before the tile's first key see none of its keys.
     const int rstart = p.causal ? (c0 / TR) * TR : 0;
+    kp.issue(Kb, c0 - 2 * pk, TC + 4 * pk, p.Nk, d);
+    qs.issue(p, Qb, dOb, LSE + bh * p.Nq, D + bh * p.Nq, rstart);
     for (int r0 = rstart; r0 < p.Nq; r0 += TR) {
         __syncthreads();
-        load_q_side(t, p, Qb, dOb, LSE + bh * p.Nq, D + bh * p.Nq, r0);
-        bwd_tile<TI, TC>(t, p, Kb, Vb, r0, c0);
+        qs.commit(t, p);
+        bwd_tile<TI, TC>(t, p, kp, vp, Vb, r0, c0, [&] {
+            if (r0 + TR < p.Nq) {
+                kp.issue(Kb, c0 - 2 * pk, TC + 4 * pk, p.Nk, d);
+                qs.issue(p, Qb, dOb, LSE + bh * p.Nq, D + bh * p.Nq, r0 + TR);
+            }
+        });
         dscore_tile<TC>(t, p, r0, c0);
         __syncthreads();
         // dV[key][:] += sum_r P[r][key] dO[r][:], dK[key][:] += sum_r dS[r][key] Q[r][:]  (A(m = key, k = r));
