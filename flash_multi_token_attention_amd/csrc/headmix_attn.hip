@@ -523,13 +523,24 @@ __global__ __launch_bounds__(HW * 64) void headmix_bwd_kernel(HmArgs a, const bf
     }
 }
 
-// dW[h][h'] = sum of the partials in index order
-__global__ void headmix_dw_reduce_kernel(int n_part, int hh, const float *__restrict__ part, float *__restrict__ dW) {
-    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= hh) return;
-    float s = 0.f;
-    for (int p = 0; p < n_part; ++p) s += part[(size_t)p * hh + idx];
-    dW[idx] = s;
+// dW[h][h'] = sum of the partials in a fixed order: a workgroup takes 64 entries (lane = entry), wave w
+// adds the partials w, w + 4, ... in four independent chains, the waves' sums are added in wave order.
+__global__ __launch_bounds__(256) void headmix_dw_reduce_kernel(int n_part, int hh, const float *__restrict__ part,
+                                                                float *__restrict__ dW) {
+    __shared__ float red[4][64];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, idx = blockIdx.x * 64 + lane;
+    float s[4] = {0.f, 0.f, 0.f, 0.f};
+    if (idx < hh) {
+        int q = wave;
+        for (; q + 12 < n_part; q += 16) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) s[c] += part[(size_t)(q + 4 * c) * hh + idx];
+        }
+        for (int c = 0; q < n_part; q += 4, ++c) s[c] += part[(size_t)q * hh + idx];
+    }
+    red[wave][lane] = (s[0] + s[1]) + (s[2] + s[3]);
+    __syncthreads();
+    if (wave == 0 && idx < hh) dW[idx] = (red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]);
 }
 
 template <auto Kern> hipError_t allow_lds(int bytes) {
@@ -609,7 +620,7 @@ hipError_t headmix_bwd_dq_dw(int B, int H, int N, int d, float scale, int causal
     }();
     if (e != hipSuccess) return e;
     const int n_part = B * ((N + HT - 1) / HT), hh = H * H;
-    headmix_dw_reduce_kernel<<<(hh + 255) / 256, 256, 0, s>>>(n_part, hh, dw_part, dw);
+    headmix_dw_reduce_kernel<<<(hh + 63) / 64, 256, 0, s>>>(n_part, hh, dw_part, dw);
     return hipGetLastError();
 }
 
