@@ -43,7 +43,8 @@ struct HmArgs {
     float scale;
 };
 
-template <int H, int D> struct HmLds {
+// XT: staging tiles per wave (1, or one per head of the wave where K tiles are staged a phase early)
+template <int H, int D, int XT = 1> struct HmLds {
     static constexpr int WST = H + 4;                       // floats per row of W
     static constexpr int XST = D * 2 + 32;                  // bytes per row of a staged bf16 tile
     static constexpr int arr_bytes = H * HST * 4;           // one score array
@@ -51,7 +52,7 @@ template <int H, int D> struct HmLds {
     static constexpr int p_off = s_off + arr_bytes;         // backward: P, then dZ, then dS
     static constexpr int w_off = p_off + arr_bytes;
     static constexpr int x_off = w_off + H * WST * 4;       // per-wave staging tiles
-    static constexpr int stat_off = x_off + HW * HT * XST;  // three [H][16] float arrays
+    static constexpr int stat_off = x_off + HW * XT * HT * XST;  // three [H][16] float arrays
     static constexpr int total = stat_off + 3 * H * HT * 4;
 };
 
@@ -332,6 +333,10 @@ __global__ __launch_bounds__(HW * 64) void headmix_fwd_kernel(HmArgs a, const bf
     }
 }
 
+template <int H, int D, int WHAT> constexpr bool bwd_ahead() {
+    return WHAT == 0 && (H / HW) * (D / 32) <= 8 && HmLds<H, D, H / HW>::total <= 160 * 1024;
+}
+
 // ----------------------------------------------------------------- backward
 // WHAT = 0: dQ and the dW partial of a row tile (grid: row tiles x batch);
 // WHAT = 1: dK and dV of 16 heads (blockIdx.z) of a key tile (grid: key tiles x batch x H / 16).
@@ -341,16 +346,20 @@ __global__ __launch_bounds__(HW * 64) void headmix_bwd_kernel(HmArgs a, const bf
                                                               const float *__restrict__ W, const bf16_t *__restrict__ dO,
                                                               const float *__restrict__ LSE, const float *__restrict__ Dl,
                                                               float *__restrict__ out0, float *__restrict__ out1) {
-    using Lds = HmLds<H, D>;
     constexpr int DB = D / 16, HPW = H / HW, RPW = HT / HW, HB = H / 16;
     constexpr int OPW = 2;   // WHAT = 1: heads of this workgroup's 16 that a wave accumulates for
+    // dQ + dW, where registers and LDS allow: the Q / dO fragments of the wave's heads stay resident, the
+    // K / V fragments of a key tile are loaded while the tile before it is worked on, dP is taken in the
+    // score phase and the K tile is staged for the last phase from the fragments (no second load).
+    constexpr bool AHEAD = bwd_ahead<H, D, WHAT>();
+    using Lds = HmLds<H, D, AHEAD ? HPW : 1>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     float *S = reinterpret_cast<float *>(smem + Lds::s_off);
     float *P = reinterpret_cast<float *>(smem + Lds::p_off);
     float *Wl = reinterpret_cast<float *>(smem + Lds::w_off);
     float *lse_s = reinterpret_cast<float *>(smem + Lds::stat_off), *d_s = lse_s + H * HT;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, g = lane >> 4, n = lane & 15;
-    unsigned char *xt = smem + Lds::x_off + wave * HT * Lds::XST;
+    unsigned char *xt = smem + Lds::x_off + wave * (AHEAD ? HPW : 1) * HT * Lds::XST;
     const int b = blockIdx.y, hs = blockIdx.z;
     const size_t bo = (size_t)b * a.H * a.N * D;
     const bf16_t *Qb = Q + bo, *Kb = K + bo, *Vb = V + bo, *Gb = dO + bo;
@@ -378,6 +387,18 @@ __global__ __launch_bounds__(HW * 64) void headmix_bwd_kernel(HmArgs a, const bf
         }
     };
     if (WHAT == 0) load_stats(fixed0);
+    constexpr int NF = AHEAD ? HPW : 1;
+    bf16x8 qf[NF][D / 32], gf[NF][D / 32], kf[NF][D / 32], vf[NF][D / 32];
+    if constexpr (AHEAD) {
+#pragma unroll
+        for (int t = 0; t < HPW; ++t) {
+            const size_t ho = (size_t)(wave + t * HW) * a.N * D;
+            load_frags<D>(qf[t], Qb + ho, fixed0, a.N, g, n);
+            load_frags<D>(gf[t], Gb + ho, fixed0, a.N, g, n);
+            load_frags<D>(kf[t], Kb + ho, 0, a.N, g, n);
+            load_frags<D>(vf[t], Vb + ho, 0, a.N, g, n);
+        }
+    }
 
     // the other axis: keys up to the diagonal (dQ) or rows from the diagonal on (dK / dV)
     const int lo = WHAT == 0 ? 0 : (a.causal ? fixed0 : 0);
@@ -386,7 +407,28 @@ __global__ __launch_bounds__(HW * 64) void headmix_bwd_kernel(HmArgs a, const bf
         const int i0 = WHAT == 0 ? fixed0 : o0, j0 = WHAT == 0 ? o0 : fixed0;
         __syncthreads();   // the last tile's dS has been used (and, first, W and the statistics are in place)
         if (WHAT == 1) load_stats(i0);
-        scores_phase<H, D>(S, a, Qb, Kb, i0, j0, wave, g, n);
+        f32x4 dp_early[NF];
+        if constexpr (AHEAD) {
+#pragma unroll
+            for (int t = 0; t < HPW; ++t) {
+                const int h = wave + t * HW;
+                const f32x4 sc = frags_dot<D>(qf[t], kf[t]);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) S[h * HST + (4 * g + r) * SST + n] = sc[r] * a.scale;
+                dp_early[t] = frags_dot<D>(gf[t], vf[t]);
+                // the K rows of the tile, as the fragments hold them, for dQ += dS K
+#pragma unroll
+                for (int blk = 0; blk < D / 32; ++blk)
+                    *reinterpret_cast<u32x4 *>(xt + t * HT * Lds::XST + n * Lds::XST + (blk * 32 + 8 * g) * 2) =
+                        __builtin_bit_cast(u32x4, kf[t][blk]);
+                if (o0 + HT < hi) {
+                    load_frags<D>(kf[t], Kb + (size_t)h * a.N * D, j0 + HT, a.N, g, n);
+                    load_frags<D>(vf[t], Vb + (size_t)h * a.N * D, j0 + HT, a.N, g, n);
+                }
+            }
+        } else {
+            scores_phase<H, D>(S, a, Qb, Kb, i0, j0, wave, g, n);
+        }
         __syncthreads();
         // ---- P = exp(Z - LSE), rows of this wave ----
 #pragma unroll
@@ -408,7 +450,9 @@ __global__ __launch_bounds__(HW * 64) void headmix_bwd_kernel(HmArgs a, const bf
 #pragma unroll
         for (int t = 0; t < HPW; ++t) {
             const int h = wave + t * HW;
-            const f32x4 dp = rows_times_rows<D>(Gb + (size_t)h * a.N * D, i0, Vb + (size_t)h * a.N * D, j0, a.N, g, n);
+            f32x4 dp;
+            if constexpr (AHEAD) dp = dp_early[t];
+            else dp = rows_times_rows<D>(Gb + (size_t)h * a.N * D, i0, Vb + (size_t)h * a.N * D, j0, a.N, g, n);
             if constexpr (WHAT == 1) {
                 // heads wave + 8t of the half hs: t = 2 hs, 2 hs + 1 (H = 32) or t = 0, 1 (H = 16)
                 if (h / 16 == hs) {
@@ -453,9 +497,13 @@ __global__ __launch_bounds__(HW * 64) void headmix_bwd_kernel(HmArgs a, const bf
 #pragma unroll
             for (int t = 0; t < HPW; ++t) {
                 const int h = wave + t * HW;
-                stage_rows<D>(xt, Lds::XST, Kb + (size_t)h * a.N * D, j0, a.N, lane);
-                tile_times_staged<D>(acc[t], P + h * HST, SST, 1, xt, Lds::XST, g, n);
-                __builtin_amdgcn_wave_barrier();
+                if constexpr (AHEAD) {
+                    tile_times_staged<D>(acc[t], P + h * HST, SST, 1, xt + t * HT * Lds::XST, Lds::XST, g, n);
+                } else {
+                    stage_rows<D>(xt, Lds::XST, Kb + (size_t)h * a.N * D, j0, a.N, lane);
+                    tile_times_staged<D>(acc[t], P + h * HST, SST, 1, xt, Lds::XST, g, n);
+                    __builtin_amdgcn_wave_barrier();
+                }
             }
         } else {
 #pragma unroll
@@ -577,7 +625,7 @@ hipError_t launch_fwd(const HmArgs &a, int out_dt, const void *q, const void *k,
 template <int H, int D, int WHAT>
 hipError_t launch_bwd(const HmArgs &a, const void *q, const void *k, const void *v, const float *w, const void *d_o,
                       const float *lse, const float *Dl, float *out0, float *out1, hipStream_t s) {
-    constexpr int lds = HmLds<H, D>::total;
+    constexpr int lds = HmLds<H, D, bwd_ahead<H, D, WHAT>() ? H / HW : 1>::total;
     static_assert(lds <= 160 * 1024, "LDS budget");
     static_assert(HW * H * H * 4 <= HmLds<H, D>::arr_bytes, "room for the dW accumulators of the waves");
     hipError_t e = allow_lds<headmix_bwd_kernel<H, D, WHAT>>(lds);
