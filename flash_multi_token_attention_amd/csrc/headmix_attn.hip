@@ -336,6 +336,20 @@ __global__ __launch_bounds__(HW * 64) void headmix_fwd_kernel(HmArgs a, const bf
 template <int H, int D, int WHAT> constexpr bool bwd_ahead() {
     return WHAT == 0 && (H / HW) * (D / 32) <= 8 && HmLds<H, D, H / HW>::total <= 160 * 1024;
 }
+// dK + dV, where LDS allows three staging tiles per wave: the Q and dO tiles of the products with dS^T
+// and P^T are staged from the row fragments that the score and dP products load anyway, and the
+// fragments of two heads are loaded before the first of them is used.
+template <int H, int D, int WHAT> constexpr bool bwd_frag_staging() {
+    return WHAT == 1 && HmLds<H, D, 3>::total <= 160 * 1024;
+}
+template <int D>
+__device__ __forceinline__ void stage_frags(unsigned char *xt, int xst, const bf16x8 (&f)[D / 32], int g, int n) {
+#pragma unroll
+    for (int blk = 0; blk < D / 32; ++blk)
+        *reinterpret_cast<u32x4 *>(xt + n * xst + (blk * 32 + 8 * g) * 2) = __builtin_bit_cast(u32x4, f[blk]);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
 
 // ----------------------------------------------------------------- backward
 // WHAT = 0: dQ and the dW partial of a row tile (grid: row tiles x batch);
@@ -352,14 +366,16 @@ __global__ __launch_bounds__(HW * 64) void headmix_bwd_kernel(HmArgs a, const bf
     // K / V fragments of a key tile are loaded while the tile before it is worked on, dP is taken in the
     // score phase and the K tile is staged for the last phase from the fragments (no second load).
     constexpr bool AHEAD = bwd_ahead<H, D, WHAT>();
-    using Lds = HmLds<H, D, AHEAD ? HPW : 1>;
+    constexpr bool FSTAGE = bwd_frag_staging<H, D, WHAT>();
+    constexpr int XTILES = AHEAD ? HPW : (FSTAGE ? 3 : 1);   // FSTAGE: tile 0 = dO of the head at hand, 1 + x = Q of output head x
+    using Lds = HmLds<H, D, XTILES>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     float *S = reinterpret_cast<float *>(smem + Lds::s_off);
     float *P = reinterpret_cast<float *>(smem + Lds::p_off);
     float *Wl = reinterpret_cast<float *>(smem + Lds::w_off);
     float *lse_s = reinterpret_cast<float *>(smem + Lds::stat_off), *d_s = lse_s + H * HT;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, g = lane >> 4, n = lane & 15;
-    unsigned char *xt = smem + Lds::x_off + wave * (AHEAD ? HPW : 1) * HT * Lds::XST;
+    unsigned char *xt = smem + Lds::x_off + wave * XTILES * HT * Lds::XST;
     const int b = blockIdx.y, hs = blockIdx.z;
     const size_t bo = (size_t)b * a.H * a.N * D;
     const bf16_t *Qb = Q + bo, *Kb = K + bo, *Vb = V + bo, *Gb = dO + bo;
@@ -417,13 +433,29 @@ __global__ __launch_bounds__(HW * 64) void headmix_bwd_kernel(HmArgs a, const bf
                 for (int r = 0; r < 4; ++r) S[h * HST + (4 * g + r) * SST + n] = sc[r] * a.scale;
                 dp_early[t] = frags_dot<D>(gf[t], vf[t]);
                 // the K rows of the tile, as the fragments hold them, for dQ += dS K
-#pragma unroll
-                for (int blk = 0; blk < D / 32; ++blk)
-                    *reinterpret_cast<u32x4 *>(xt + t * HT * Lds::XST + n * Lds::XST + (blk * 32 + 8 * g) * 2) =
-                        __builtin_bit_cast(u32x4, kf[t][blk]);
+                stage_frags<D>(xt + t * HT * Lds::XST, Lds::XST, kf[t], g, n);
                 if (o0 + HT < hi) {
                     load_frags<D>(kf[t], Kb + (size_t)h * a.N * D, j0 + HT, a.N, g, n);
                     load_frags<D>(vf[t], Vb + (size_t)h * a.N * D, j0 + HT, a.N, g, n);
+                }
+            }
+        } else if constexpr (FSTAGE) {
+#pragma unroll
+            for (int t0 = 0; t0 < HPW; t0 += 2) {
+                bf16x8 xq[2][D / 32], xk[2][D / 32];
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const size_t ho = (size_t)(wave + (t0 + u) * HW) * a.N * D;
+                    load_frags<D>(xq[u], Qb + ho, i0, a.N, g, n);
+                    load_frags<D>(xk[u], Kb + ho, j0, a.N, g, n);
+                }
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const int t = t0 + u, h = wave + t * HW;
+                    const f32x4 sc = frags_dot<D>(xq[u], xk[u]);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) S[h * HST + (4 * g + r) * SST + n] = sc[r] * a.scale;
+                    if (h / 16 == hs) stage_frags<D>(xt + (1 + t % OPW) * HT * Lds::XST, Lds::XST, xq[u], g, n);
                 }
             }
         } else {
@@ -447,6 +479,33 @@ __global__ __launch_bounds__(HW * 64) void headmix_bwd_kernel(HmArgs a, const bf
         }
         __syncthreads();
         // ---- heads of this wave: dP = dO V^T, (dV += P^T dO), dZ = P (dP - D) in place of P ----
+        if constexpr (FSTAGE) {
+#pragma unroll
+            for (int t0 = 0; t0 < HPW; t0 += 2) {
+                bf16x8 xg[2][D / 32], xv[2][D / 32];
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const size_t ho = (size_t)(wave + (t0 + u) * HW) * a.N * D;
+                    load_frags<D>(xg[u], Gb + ho, i0, a.N, g, n);
+                    load_frags<D>(xv[u], Vb + ho, j0, a.N, g, n);
+                }
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const int t = t0 + u, h = wave + t * HW;
+                    const f32x4 dp = frags_dot<D>(xg[u], xv[u]);
+                    if (h / 16 == hs) {
+                        stage_frags<D>(xt, Lds::XST, xg[u], g, n);
+                        tile_times_staged<D>(acc[OPW + (t % OPW)], P + h * HST, 1, SST, xt, Lds::XST, g, n);
+                        __builtin_amdgcn_wave_barrier();
+                    }
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        float *pp = P + h * HST + (4 * g + r) * SST + n;
+                        *pp = *pp * (dp[r] - d_s[h * HT + 4 * g + r]);
+                    }
+                }
+            }
+        } else {
 #pragma unroll
         for (int t = 0; t < HPW; ++t) {
             const int h = wave + t * HW;
@@ -467,6 +526,7 @@ __global__ __launch_bounds__(HW * 64) void headmix_bwd_kernel(HmArgs a, const bf
                 float *pp = P + h * HST + (4 * g + r) * SST + n;
                 *pp = *pp * (dp[r] - d_s[h * HT + 4 * g + r]);
             }
+        }
         }
         __syncthreads();
         // ---- rows of this wave: dW += dZ S^T over its elements, then dS = scale W^T dZ in place ----
@@ -510,9 +570,13 @@ __global__ __launch_bounds__(HW * 64) void headmix_bwd_kernel(HmArgs a, const bf
             for (int t = 0; t < HPW; ++t) {
                 const int h = wave + t * HW;
                 if (h / 16 == hs) {
-                    stage_rows<D>(xt, Lds::XST, Qb + (size_t)h * a.N * D, i0, a.N, lane);
-                    tile_times_staged<D>(acc[t % OPW], P + h * HST, 1, SST, xt, Lds::XST, g, n);
-                    __builtin_amdgcn_wave_barrier();
+                    if constexpr (FSTAGE) {
+                        tile_times_staged<D>(acc[t % OPW], P + h * HST, 1, SST, xt + (1 + t % OPW) * HT * Lds::XST, Lds::XST, g, n);
+                    } else {
+                        stage_rows<D>(xt, Lds::XST, Qb + (size_t)h * a.N * D, i0, a.N, lane);
+                        tile_times_staged<D>(acc[t % OPW], P + h * HST, 1, SST, xt, Lds::XST, g, n);
+                        __builtin_amdgcn_wave_barrier();
+                    }
                 }
             }
         }
@@ -625,7 +689,7 @@ hipError_t launch_fwd(const HmArgs &a, int out_dt, const void *q, const void *k,
 template <int H, int D, int WHAT>
 hipError_t launch_bwd(const HmArgs &a, const void *q, const void *k, const void *v, const float *w, const void *d_o,
                       const float *lse, const float *Dl, float *out0, float *out1, hipStream_t s) {
-    constexpr int lds = HmLds<H, D, bwd_ahead<H, D, WHAT>() ? H / HW : 1>::total;
+    constexpr int lds = HmLds<H, D, bwd_ahead<H, D, WHAT>() ? H / HW : (bwd_frag_staging<H, D, WHAT>() ? 3 : 1)>::total;
     static_assert(lds <= 160 * 1024, "LDS budget");
     static_assert(HW * H * H * 4 <= HmLds<H, D>::arr_bytes, "room for the dW accumulators of the waves");
     hipError_t e = allow_lds<headmix_bwd_kernel<H, D, WHAT>>(lds);
