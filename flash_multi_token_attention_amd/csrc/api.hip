@@ -158,7 +158,7 @@ int convattn_bwd_preprocess(const convattn_desc *desc, const void *o, const void
 }
 
 // Workspace of the one-pass backward on the MFMA path: dS blocks, dW partials and (windows of up
-// to 6 query taps) the dC scale of every (batch, head), each part 256-byte aligned.
+// to 8 query taps) the dC scale of every (batch, head), each part 256-byte aligned.
 struct FusedWs {
     size_t ds_bytes, part_off, scale_off, total;
     bool chain;
@@ -173,7 +173,7 @@ static FusedWs fused_ws(const Problem &p) {
     return w;
 }
 
-// The dQ + dW pass on the chain path (windows of up to 6 query taps) is the key-stationary kernel
+// The dQ + dW pass on the chain path (windows of up to 8 query taps) is the key-stationary kernel
 // without its dK / dV half plus the dQ = dS K product: its "dW partial buffer" is the one-pass
 // backward's workspace (dS blocks, dW partials, dC scales).
 static bool dq_dw_uses_chain(const convattn_desc *desc, const Problem &p) {

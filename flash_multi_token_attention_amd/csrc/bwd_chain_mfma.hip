@@ -1046,7 +1046,8 @@ hipError_t pick_cq(const Problem &p, const void *q, const void *k, const void *v
                    const float *Dl, const float *lse, const float *w, const float *dc_scale, void *dk, void *dv,
                    void *ds_ws, float *dw_part, hipStream_t s) {
     if (p.c_q <= 3) return launch_chain<D, 3, TO, WANT>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
-    return launch_chain<D, 6, TO, WANT>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
+    if (p.c_q <= 6) return launch_chain<D, 6, TO, WANT>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
+    return launch_chain<D, 8, TO, WANT>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
 }
 
 template <int WANT>

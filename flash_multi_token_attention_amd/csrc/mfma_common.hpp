@@ -258,11 +258,11 @@ hipError_t mfma_dq_from_ds(const Problem &p, int out_dt, const void *k, const vo
                            void *dq, hipStream_t s);
 
 // ---- whole backward with the score chain in registers (bwd_chain_mfma.hip, bwd_dq_rows.hip) ----
-// Windows of up to 6 query taps.  The key-stationary kernel's workgroups cover 128 keys each (+ 8:
+// Windows of up to 8 query taps.  The key-stationary kernel's workgroups cover 128 keys each (+ 8:
 // the dV ranges start 8 keys early); it leaves one dW partial per workgroup and dS as bf16 blocks
 // [key tile of 32][row tile of 32][32 rows][32 keys], which mfma_dq_from_rows multiplies with K.
 // dc_scale holds {s, log2 s} per (batch, head): the power of two dC is carried at (mfma_dc_scale).
-constexpr int kChainKeys = 32, kChainRows = 32, kChainMaxCq = 6;
+constexpr int kChainKeys = 32, kChainRows = 32, kChainMaxCq = 8;
 inline bool chain_ok(const Problem &p) { return p.c_q <= kChainMaxCq && (long long)p.B * p.H <= 65535; }
 inline int chain_key_tiles(const Problem &p) { return mfma_kv_tiles(p) * (kKvKeysPerWg / kChainKeys); }
 __host__ __device__ inline int chain_row_tiles(const Problem &p) { return (p.Nq + kChainRows - 1) / kChainRows; }
