@@ -6,8 +6,9 @@
 // Lane n of score fragment f holds row base + 2n + f.  Per 32-key step:
 //   1. all waves issue the loads of the next step's K / V rows, which go from global memory
 //      straight into the LDS buffer the step before this one has just left (buffer loads with the
-//      LDS modifier: no staging registers, no LDS writes by the waves; rows are dense and their
-//      16-byte chunks XOR-swizzled with the row index; one barrier per step);
+//      LDS modifier: no staging registers, no LDS writes by the waves; a tile is kept as
+//      [k-step][row][64 bytes] with the four 16-byte chunks XOR-swizzled with the row index, so that
+//      one lane address per matrix serves every fragment; one barrier per step);
 //   2. S^T = K Q^T for two 16-key blocks; the accumulator layout (lane = query row, 4 keys per
 //      lane group) is, packed to fp16 after the causal pre-mask, already the B operand layout of
 //      the convolution MFMA: k slots 0..3 of a lane group come from one block, 4..7 from the next
@@ -40,7 +41,7 @@ __device__ __forceinline__ unsigned int opaque_u32(unsigned int x) {
     asm volatile("" : "+v"(x));
     return x;
 }
-__device__ __forceinline__ bf16x4 lds_tr64(const unsigned char *ptr) {
+__device__ __forceinline__ bf16x4 lds_tr64(__attribute__((address_space(3))) const unsigned char *ptr) {
     typedef short s16x4 __attribute__((ext_vector_type(4)));
     s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(ptr));
     return __builtin_bit_cast(bf16x4, v);
@@ -78,10 +79,12 @@ __device__ long long g_fwd_ts[4][64][8];
 #endif
 template <int D> struct FwdLds {
     // K / V rows go from global memory straight into LDS (buffer loads with the LDS modifier: the
-    // 64 lanes of a load fill 1 KB of consecutive LDS, which rules out padded rows), so the rows are
-    // dense and the 16-byte chunk c of row r sits at chunk position c ^ (r mod chunks per row):
-    // a fragment read (16 rows, one column) then touches 16 different bank groups.
-    static constexpr int KST = D * 2;
+    // 64 lanes of a load fill 1 KB of consecutive LDS, which rules out padded rows).  A tile of 32
+    // rows is kept as [k-step ks][row][64 bytes]: the 4 chunks of 16 bytes that a row holds of
+    // head-dim columns 32 ks .. 32 ks + 31, chunk c at position c ^ (row / 4 mod 4).  Row fragments
+    // (lane n reads row n) and transposed fragments then touch every bank equally often, and k-step,
+    // row block and head-dim block are constant offsets from one lane address.
+    static constexpr int KST = D * 2;              // bytes of a row in global memory
     static constexpr int k_bytes = BK * KST;
     static constexpr int buf_bytes = 2 * k_bytes;  // K rows, then V rows
     static constexpr int n_buf = FWD_NBUF;         // steps u, u+1 (and u+2) resident or on their way
@@ -97,10 +100,7 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
     constexpr int KST = Lds::KST;
     constexpr int KS = D / 32;   // MFMA k-steps over the head dimension
     constexpr int DB = D / 16;   // 16-wide blocks of the head dimension
-    constexpr int CPR = D / 8;   // 16-byte chunks per row
     constexpr int WR = wave_rows(CQT), BQ = NW * WR;
-    constexpr int N_LD = BK * CPR / (NW * 64);  // 16-byte chunks per thread and matrix
-    static_assert(BK * CPR % (NW * 64) == 0 && (NW * 64) % CPR == 0, "whole chunks per thread, whole rows per pass");
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
     const int tid = threadIdx.x;
@@ -182,11 +182,11 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
     // K / V rows: buffer loads with the LDS modifier.  Rows before the first or after the last key
     // are outside the descriptor's range and arrive as zeros, which is what the window's zero
     // padding asks for.
-    // Load i of a wave fills rows RPL (i NW + wave) .. + RPL - 1 of a tile (RPL = rows per KB): lane l
-    // writes chunk position l % CPR of row l / CPR and therefore reads chunk (l % CPR) ^ (row % CPR).
-    constexpr int RPL = 1024 / (D * 2);
-    static_assert(N_LD * NW * RPL == BK, "whole tiles");
-    const int dma_off = ((lane / CPR) * D + ((lane % CPR) ^ ((lane / CPR + RPL * wave) % CPR)) * 8) * 2 + wave * 1024;
+    // A tile is 2 KS units of 1 KB (unit 2 ks + blk = rows 16 blk .. 16 blk + 15 of k-step ks); wave w
+    // issues the units w, w + NW, ...  Lane l of a load fills chunk position l % 4 of row l / 4.
+    constexpr int UNITS = Lds::k_bytes / 1024, N_LD = UNITS / NW;
+    static_assert(UNITS == 2 * KS && UNITS % NW == 0 && NW == 4, "whole units per wave");
+    const int dma_off = (16 * (wave & 1) + (lane >> 2)) * KST + (((wave >> 1) * 4 + ((lane & 3) ^ ((lane >> 4) & 3))) << 4);
     // rows of step u: issued right after the barrier that ends step u - 1 (their buffer is free then),
     // landed by the barrier that starts step u (the barrier waits for the wave's loads)
     // (issued as inline assembly: for the builtin the compiler makes every later LDS read wait for the
@@ -197,31 +197,44 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
         return (i32x4){(int)(unsigned int)a, (int)(unsigned int)(a >> 32), p.Nk * D * 2, 0x00020000};
     };
     const i32x4 k_dma = dma_rsrc(Kb), v_dma = dma_rsrc(Vb);
-    const unsigned int lds_base =
-        (unsigned int)(unsigned long long)(__attribute__((address_space(3))) unsigned char *)smem + wave * 1024;
-    auto dma16 = [&](const i32x4 &rsrc, unsigned int lds_addr, int voffset) {
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
-                     :: "s"(lds_addr), "v"(voffset), "s"(rsrc) : "memory");
+    const unsigned int lds_u = (unsigned int)(unsigned long long)(__attribute__((address_space(3))) unsigned char *)smem;
+    const unsigned int lds_base = lds_u + wave * 1024;
+    // unit i of the wave: k-step + 2 i = 128 bytes further along the row (the instruction's offset
+    // field, which the hardware adds to the LDS address as well as to the global one), 4 KB further in
+    // LDS; the step's first row is the scalar offset of the load
+    auto dma16 = [&](const i32x4 &rsrc, unsigned int lds_addr, int voffset, int soffset, auto I) {
+        constexpr int i = decltype(I)::value;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen offset:%4 lds"
+                     :: "s"(__builtin_amdgcn_readfirstlane((int)lds_addr + i * (4096 - 128))), "v"(voffset), "s"(rsrc),
+                        "s"(__builtin_amdgcn_readfirstlane(soffset)), "n"(i * 128) : "memory");
     };
+    // step 0 starts before the first key: those rows have negative offsets, which only the vector
+    // offset (a wrapping 32-bit sum made here) may carry; later steps pass theirs as the scalar offset
     auto fetch_step = [&](int u) {
         const unsigned int Ks = lds_base + (u % Lds::n_buf) * Lds::buf_bytes, Vs = Ks + Lds::k_bytes;
-        const int k0 = (32 * u - 8) * D * 2 + dma_off, v0 = (32 * u - 16) * D * 2 + dma_off;
-#pragma unroll
-        for (int i = 0; i < N_LD; ++i) {
-            dma16(k_dma, Ks + i * NW * 1024, k0 + i * NW * 1024);
-            dma16(v_dma, Vs + i * NW * 1024, v0 + i * NW * 1024);
-        }
+        const int k0 = (32 * u - 8) * KST, v0 = (32 * u - 16) * KST;
+        static_for<N_LD>([&](auto I) {
+            if (u == 0) {
+                dma16(k_dma, Ks, dma_off + k0, 0, I);
+                dma16(v_dma, Vs, dma_off + v0, 0, I);
+            } else {
+                // (a scalar offset past the end is held at the end: everything is out of range then,
+                // whichever way the range check treats a scalar offset beyond the number of records)
+                dma16(k_dma, Ks, dma_off, min(k0, p.Nk * KST), I);
+                dma16(v_dma, Vs, dma_off, min(v0, p.Nk * KST), I);
+            }
+        });
     };
-    // lane addresses of the fragment reads inside a tile: chunk c of row r at r KST + ((c ^ (r % CPR)) << 4);
-    // row blocks of 16 and the buffers are constant offsets on top
-    unsigned int ka[KS], va[DB];
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) ka[ks] = opaque_u32(n * KST + (((ks * 4 + g) ^ (n % CPR)) << 4));
-#pragma unroll
-    for (int db = 0; db < DB; ++db) {
-        const int r = 4 * g + (n >> 2);
-        va[db] = opaque_u32(r * KST + (((db * 2 + ((n >> 1) & 1)) ^ (r % CPR)) << 4) + (n & 1) * 8);
-    }
+    // lane addresses (absolute LDS addresses) of the fragment reads inside the buffer of the step; they
+    // are moved to the other buffer at the end of every step.  K row fragment: row n, chunk 4 ks + g;
+    // row block and k-step are constant offsets.  V^T fragment: rows 4g + n/4 (+ 16), 8 bytes at byte
+    // column 32 db + 8 (n % 4): head-dim blocks 2 x and 2 x + 1 differ in bit 5 of the lane part.
+    unsigned int ka = opaque_u32(lds_u + n * 64 + ((g ^ ((n >> 2) & 3)) << 4));
+    unsigned int va[2];
+    va[0] = opaque_u32(lds_u + Lds::k_bytes + (4 * g + (n >> 2)) * 64 + ((((n >> 1) & 1) ^ g) << 4) + (n & 1) * 8);
+    va[1] = opaque_u32(va[0] ^ 32u);
+    typedef __attribute__((address_space(3))) const bf16x8 *lds_bf16x8_ptr;
+    typedef __attribute__((address_space(3))) const unsigned char *lds_byte_ptr;
 
     // packed fp16 scores of the last score block of the previous step:
     // carry[f][dword] = row base + 2n + f, keys 4g .. 4g+3 of the block
@@ -231,9 +244,6 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
     // (wave-uniform), only then are the masks evaluated.
     auto step = [&](int u, auto edge_tag) {
         constexpr bool EDGE = decltype(edge_tag)::value;
-        // (the address registers ka / va point into the buffer of the step: they are moved to the
-        // other buffer at the end of every step)
-        const unsigned char *Ks = smem, *Vs = Ks + Lds::k_bytes;
         const int jk = 32 * u - 8, jv = 32 * u - 16;
         f32x4 c[2][2];
         bf16x8 kf[KS];  // K fragments of one score block; the second block's are read during the first's convolution
@@ -241,7 +251,7 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
         auto load_kf = [&](int blk) {
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks)
-                kf[ks] = *reinterpret_cast<const bf16x8 *>(Ks + ka[ks] + blk * 16 * KST);
+                kf[ks] = *(lds_bf16x8_ptr)(size_t)(ka + blk * 1024 + ks * 2048);
         };
         load_kf(0);
         static_for<2>([&](auto BL) {
@@ -312,8 +322,8 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
         constexpr int PFV = FWD_PFV < DB ? FWD_PFV : DB;
         bf16x8 vf[PFV + 1];
         auto load_vf = [&](int buf, int db) {
-            bf16x4 lo = lds_tr64(Vs + va[db]);
-            bf16x4 hi = lds_tr64(Vs + va[db] + 16 * KST);
+            bf16x4 lo = lds_tr64((lds_byte_ptr)(size_t)(va[db & 1] + (db >> 1) * 2048));
+            bf16x4 hi = lds_tr64((lds_byte_ptr)(size_t)(va[db & 1] + (db >> 1) * 2048 + 1024));
             vf[buf] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
         };
 #pragma unroll
@@ -432,10 +442,9 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
             FTS(2);
             if constexpr (KIND != 2) step(u, std::integral_constant<bool, KIND == 1>{});
             const int to_other = (u % Lds::n_buf == Lds::n_buf - 1) ? -(Lds::n_buf - 1) * Lds::buf_bytes : Lds::buf_bytes;
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) ka[ks] += to_other;
-#pragma unroll
-            for (int db = 0; db < DB; ++db) va[db] += to_other;
+            ka += to_other;
+            va[0] += to_other;
+            va[1] += to_other;
         }
     };
     const int u_diag = base < 23 ? 1 : (base - 23) / 32 + 1;    // first u >= 1 with 32u + 23 > base
