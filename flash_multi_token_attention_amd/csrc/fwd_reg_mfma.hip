@@ -81,9 +81,10 @@ template <int D> struct FwdLds {
     // K / V rows go from global memory straight into LDS (buffer loads with the LDS modifier: the
     // 64 lanes of a load fill 1 KB of consecutive LDS, which rules out padded rows).  A tile of 32
     // rows is kept as [k-step ks][row][64 bytes]: the 4 chunks of 16 bytes that a row holds of
-    // head-dim columns 32 ks .. 32 ks + 31, chunk c at position c ^ (row / 4 mod 4).  Row fragments
-    // (lane n reads row n) and transposed fragments then touch every bank equally often, and k-step,
-    // row block and head-dim block are constant offsets from one lane address.
+    // head-dim columns 32 ks .. 32 ks + 31, chunk c at position c ^ s(row) with s = row / 4 mod 4 for
+    // K and the same two bits swapped for V.  The row fragments of K (lane n reads row n) and the
+    // transposed fragments of V then touch every bank equally often, and k-step, row block and head-dim
+    // block are constant offsets from one lane address.
     static constexpr int KST = D * 2;              // bytes of a row in global memory
     static constexpr int k_bytes = BK * KST;
     static constexpr int buf_bytes = 2 * k_bytes;  // K rows, then V rows
@@ -186,7 +187,12 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
     // issues the units w, w + NW, ...  Lane l of a load fills chunk position l % 4 of row l / 4.
     constexpr int UNITS = Lds::k_bytes / 1024, N_LD = UNITS / NW;
     static_assert(UNITS == 2 * KS && UNITS % NW == 0 && NW == 4, "whole units per wave");
-    const int dma_off = (16 * (wave & 1) + (lane >> 2)) * KST + (((wave >> 1) * 4 + ((lane & 3) ^ ((lane >> 4) & 3))) << 4);
+    // (K rows are read as row fragments, 16 rows of one chunk column at a time: swizzle value row / 4 mod 4;
+    // V rows through transpose reads, 8 rows x 32 bytes per half wave: the same value with its two bits
+    // swapped, so that rows r and r + 4 use different halves of their 64 bytes)
+    const int dma_row = (16 * (wave & 1) + (lane >> 2)) * KST;
+    const int dma_off = dma_row + (((wave >> 1) * 4 + ((lane & 3) ^ ((lane >> 4) & 3))) << 4);
+    const int dma_off_v = dma_row + (((wave >> 1) * 4 + ((lane & 3) ^ ((((lane >> 4) & 1) << 1) | ((lane >> 5) & 1)))) << 4);
     // rows of step u: issued right after the barrier that ends step u - 1 (their buffer is free then),
     // landed by the barrier that starts step u (the barrier waits for the wave's loads)
     // (issued as inline assembly: for the builtin the compiler makes every later LDS read wait for the
@@ -216,12 +222,12 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
         static_for<N_LD>([&](auto I) {
             if (u == 0) {
                 dma16(k_dma, Ks, dma_off + k0, 0, I);
-                dma16(v_dma, Vs, dma_off + v0, 0, I);
+                dma16(v_dma, Vs, dma_off_v + v0, 0, I);
             } else {
                 // (a scalar offset past the end is held at the end: everything is out of range then,
                 // whichever way the range check treats a scalar offset beyond the number of records)
                 dma16(k_dma, Ks, dma_off, min(k0, p.Nk * KST), I);
-                dma16(v_dma, Vs, dma_off, min(v0, p.Nk * KST), I);
+                dma16(v_dma, Vs, dma_off_v, min(v0, p.Nk * KST), I);
             }
         });
     };
@@ -231,7 +237,7 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
     // column 32 db + 8 (n % 4): head-dim blocks 2 x and 2 x + 1 differ in bit 5 of the lane part.
     unsigned int ka = opaque_u32(lds_u + n * 64 + ((g ^ ((n >> 2) & 3)) << 4));
     unsigned int va[2];
-    va[0] = opaque_u32(lds_u + Lds::k_bytes + (4 * g + (n >> 2)) * 64 + ((((n >> 1) & 1) ^ g) << 4) + (n & 1) * 8);
+    va[0] = opaque_u32(lds_u + Lds::k_bytes + (4 * g + (n >> 2)) * 64 + ((((n >> 1) & 1) ^ (((g & 1) << 1) | (g >> 1))) << 4) + (n & 1) * 8);
     va[1] = opaque_u32(va[0] ^ 32u);
     typedef __attribute__((address_space(3))) const bf16x8 *lds_bf16x8_ptr;
     typedef __attribute__((address_space(3))) const unsigned char *lds_byte_ptr;
