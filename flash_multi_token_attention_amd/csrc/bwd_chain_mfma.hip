@@ -260,6 +260,12 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
     const int g = lane >> 4, n = lane & 15;
     constexpr bool producer = ROLE == 0;
     constexpr bool WANT_KV = (WANT & 1) != 0, WANT_QW = (WANT & 2) != 0;
+    // LIGHT: only the last pair's producer computes the C / dP / dC block after its own keys (the others'
+    // consumers read it from the next pair's stage); its consumer in turn takes no part in dW, which the
+    // other three share (2 CQT (pair group, tap slot) units, a multiple of 6).  The instance with 8 tap
+    // slots has no registers for a third of the units per wave: there every pair computes its own block.
+    constexpr bool LIGHT = CQT <= 6;
+    static_assert(!LIGHT || (2 * CQT) % 6 == 0, "whole dW units per wave and half");
     const int pr = wave & (NP - 1);
     TSX(0, 10);
 
@@ -340,21 +346,25 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
         else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     };
     static_assert((2 * KBT) % (2 * NP) == 0, "whole units per wave");
-    // LSE and D of a tile: loaded by the first 32 threads one iteration before they are written to LDS
+    // LSE and D of a tile: loaded by 32 threads one iteration before they are written to LDS.  STAT_ROLE: the
+    // role whose wave does it (its first 32 lanes): the last consumer wave where it has the lightest
+    // iteration (LIGHT), else the first producer wave.
+    constexpr bool STAT_ROLE = (ROLE == 1) == LIGHT;
+    const int stat_tt = tid - (LIGHT ? NT - 64 : 0);
     float ls = 0.f, dd = 0.f;
     auto load_stats = [&](int r0) {
-        if constexpr (producer) {
+        if constexpr (STAT_ROLE) {
             // raw values: arithmetic on them here would wait for the loads in this iteration
-            const int tt = (int)opaque((unsigned int)tid);
+            const int tt = (int)opaque((unsigned int)stat_tt);
             ls = 1e30f; dd = 0.f;  // rows past the end: exp2(C - LSE) = 0
-            if (tt < BR && r0 + tt < p.Nq) { ls = lse_b[r0 + tt]; dd = dl_b[r0 + tt]; }
+            if (tt >= 0 && tt < BR && r0 + tt < p.Nq) { ls = lse_b[r0 + tt]; dd = dl_b[r0 + tt]; }
         }
     };
     auto stage_stats = [&](int t) {
-        if constexpr (producer) {
-            const int tt = (int)opaque((unsigned int)tid);
+        if constexpr (STAT_ROLE) {
+            const int tt = (int)opaque((unsigned int)stat_tt);
             float *st = stat_slot(t);
-            if (tt < BR) { st[tt] = ls * kLog2e - dcs_log2; st[BR + tt] = dd; }
+            if (tt >= 0 && tt < BR) { st[tt] = ls * kLog2e - dcs_log2; st[BR + tt] = dd; }
         }
     };
     // Lane parts of the fragment addresses inside a tile.  Row fragment (producers): row 2n + f,
@@ -412,6 +422,13 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
         stage_stats(0);
         load_stats(r_begin + BR);
 
+        // The C / dP / dC block after a pair's own keys (keys c0+24 .. c0+39) is the first block of the next
+        // pair, whose producer computes it anyway: only the last pair of the workgroup (HEAVY) computes it
+        // itself, and with it the fourth S^T block; the consumers of the other pairs read that block from
+        // the next pair's stage.
+        auto producer_loop = [&](auto heavy_tag) {
+        constexpr bool HEAVY = decltype(heavy_tag)::value;
+        constexpr int PNSB = HEAVY ? NSB : NSB - 1, PNCB = HEAVY ? NCB : NCB - 1;
         // packed fp16 scores of the previous tile: [block][fragment][dword]
         unsigned int prev_pd[NSB][2][2];
 
@@ -420,7 +437,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
             constexpr bool EDGE = decltype(edge_tag)::value;
             f32x4 acc[NSB][2];
 #pragma unroll
-            for (int kb = 0; kb < NSB; ++kb)
+            for (int kb = 0; kb < PNSB; ++kb)
 #pragma unroll
                 for (int f = 0; f < 2; ++f) acc[kb][f] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -429,13 +446,13 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
 #pragma unroll
                 for (int f = 0; f < 2; ++f) qf[f] = load_qf(f, ks);
 #pragma unroll
-                for (int kb = 0; kb < NSB; ++kb)
+                for (int kb = 0; kb < PNSB; ++kb)
 #pragma unroll
                     for (int f = 0; f < 2; ++f) acc[kb][f] = mfma_bf16(kf[kb][ks], qf[f], acc[kb][f]);
             }
             const int rbase = (tp * BR) % S_RING;
 #pragma unroll
-            for (int kb = 0; kb < NSB; ++kb)
+            for (int kb = 0; kb < PNSB; ++kb)
 #pragma unroll
                 for (int f = 0; f < 2; ++f) {
                     if constexpr (EDGE) {
@@ -487,7 +504,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                 const unsigned int ln = opaque((unsigned int)lane);
                 unsigned char *Cs = c_stage(it) + 2 * (ln & 15) * CST + (ln >> 4) * 8;
 #pragma unroll
-                for (int cb = 0; cb < NCB; ++cb)
+                for (int cb = 0; cb < PNCB; ++cb)
 #pragma unroll
                     for (int ob = 0; ob < 2; ++ob)
                         *reinterpret_cast<u32x2 *>(Cs + ob * CST + cb * 32) = (u32x2){0u, 0u};
@@ -504,7 +521,9 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                 // row fragments: lane n of fragment f reads row 2n + f, 16 bytes at column 32 ks + 8 g
                 const unsigned char *Qs = smem + opaque((unsigned int)(q_slot(it) - smem) + row_frag_off());
                 const unsigned char *Gs = smem + opaque((unsigned int)(g_slot(it) - smem) + row_frag_off());
-                __builtin_amdgcn_s_setprio(CHAIN_PRIO_P);
+                // (with the light producers the consumers are the longer role: they get the issue slot first)
+                if constexpr (LIGHT) __builtin_amdgcn_s_setprio(0);
+                else __builtin_amdgcn_s_setprio(CHAIN_PRIO_P);
                 f32x4 dp[NCB][2];
                 float2 l2 = {0.f, 0.f};
                 if constexpr (FULL) l2 = *reinterpret_cast<const float2 *>(stat_slot(it) + 2 * n);
@@ -524,7 +543,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                     // 0 with tap slot DL and parity 1 with tap slot DL - 1. ----
                     f32x4 c[NCB][2];
 #pragma unroll
-                    for (int cb = 0; cb < NCB; ++cb) {
+                    for (int cb = 0; cb < PNCB; ++cb) {
                         c[cb][0] = (f32x4){-l2.x, -l2.x, -l2.x, -l2.x};
                         c[cb][1] = (f32x4){-l2.y, -l2.y, -l2.y, -l2.y};
                     }
@@ -537,11 +556,11 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                         if constexpr (t0 < CQT) tf_cur = *reinterpret_cast<const f16x8 *>(bands + t0 * 1024);
                         unsigned int sh[NSB][2];
 #pragma unroll
-                        for (int kb = 0; kb < NSB; ++kb)
+                        for (int kb = 0; kb < PNSB; ++kb)
 #pragma unroll
                             for (int dw = 0; dw < 2; ++dw) sh[kb][dw] = win_up<s>(prev_pd[kb][f][dw], pd[kb][f][dw]);
 #pragma unroll
-                        for (int cb = 0; cb < NCB; ++cb) {
+                        for (int cb = 0; cb < PNCB; ++cb) {
                             const u32x4 bv = {sh[cb][0], sh[cb][1], sh[cb + 1][0], sh[cb + 1][1]};
                             if constexpr (t0 < CQT) c[cb][0] = mfma_f16(tf_cur, __builtin_bit_cast(f16x8, bv), c[cb][0]);
                             if constexpr (t0 >= 1) c[cb][1] = mfma_f16(tf_prev, __builtin_bit_cast(f16x8, bv), c[cb][1]);
@@ -549,7 +568,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                         tf_prev = tf_cur;
                     });
 #pragma unroll
-                    for (int kb = 0; kb < NSB; ++kb)
+                    for (int kb = 0; kb < PNSB; ++kb)
 #pragma unroll
                         for (int f = 0; f < 2; ++f) { prev_pd[kb][f][0] = pd[kb][f][0]; prev_pd[kb][f][1] = pd[kb][f][1]; }
                     // ---- dP^T = V dO^T - D, after the convolution: the shifted score windows are no
@@ -557,7 +576,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                     if constexpr (!(CHAIN_ABLATE & 32)) {
                         const float2 d2 = *reinterpret_cast<const float2 *>(stat_slot(it) + BR + 2 * n);
 #pragma unroll
-                        for (int cb = 0; cb < NCB; ++cb) {
+                        for (int cb = 0; cb < PNCB; ++cb) {
                             dp[cb][0] = (f32x4){-d2.x, -d2.x, -d2.x, -d2.x};
                             dp[cb][1] = (f32x4){-d2.y, -d2.y, -d2.y, -d2.y};
                         }
@@ -568,7 +587,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                             for (int f = 0; f < 2; ++f)
                                 gf[f] = *reinterpret_cast<const bf16x8 *>(Gs + f * 1024 + ks * 2048);
 #pragma unroll
-                            for (int cb = 0; cb < NCB; ++cb)
+                            for (int cb = 0; cb < PNCB; ++cb)
 #pragma unroll
                                 for (int f = 0; f < 2; ++f) dp[cb][f] = mfma_bf16(vf[cb][ks], gf[f], dp[cb][f]);
                         }
@@ -576,7 +595,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                     CHAIN_SCHED_BARRIER;
                     TS(5);
                     // ---- P = exp2(C - LSE) (times the dC scale), dC = P dP ----
-                    static_for<(CHAIN_ABLATE & 128) ? 0 : NCB>([&](auto CB) {
+                    static_for<(CHAIN_ABLATE & 128) ? 0 : PNCB>([&](auto CB) {
                         constexpr int cb = decltype(CB)::value;
                         __builtin_amdgcn_s_setprio(0);
 #pragma unroll
@@ -607,7 +626,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                     });
                 } else {
 #pragma unroll
-                    for (int kb = 0; kb < NSB; ++kb)
+                    for (int kb = 0; kb < PNSB; ++kb)
 #pragma unroll
                         for (int f = 0; f < 2; ++f) { prev_pd[kb][f][0] = pd[kb][f][0]; prev_pd[kb][f][1] = pd[kb][f][1]; }
                     zero_dc();
@@ -618,6 +637,9 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
             else ptile(std::false_type{}, std::true_type{});
             TS(6);
         }
+        };
+        if (!LIGHT || pr == NP - 1) producer_loop(std::true_type{});
+        else producer_loop(std::false_type{});
         TSX(1, 10);
         __syncthreads();  // the consumers' barrier before they hand over their dW accumulators
         __syncthreads();  // ... and the one after it
@@ -650,9 +672,21 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
         unsigned char *bands = smem + opaque((unsigned int)Lds::band_off + CQT * 1024 + lane * 16);
         for (int t = pr; t < CQT; t += NP)
             *reinterpret_cast<f16x8 *>(bands + t * 1024) = band_frag<CQT>(t, w_head, cq, ck, pk, g, n, true, p.scale);
-        // dW: this wave takes the key blocks of two pairs (pg) and half of the tap slots (t_lo ..)
-        constexpr int TH = (CQT + 1) / 2;
-        const int pg = pr >> 1, t_lo = (pr & 1) * TH;
+        stage_stats(0);
+        load_stats(r_begin + BR);
+        // dW: a unit is the key blocks of two pairs (pair group) times one tap slot.  LIGHT: the waves 0 .. 2 take
+        // 2 CQT / 3 consecutive units each, in two passes of NU units of one pair group; otherwise every wave
+        // takes one pair group and half of the tap slots in one pass.
+        constexpr int NU = LIGHT ? CQT / 3 : (CQT + 1) / 2;   // units per pass
+        constexpr int NPASS = LIGHT ? 2 : 1, TH = NU * NPASS;
+        int dw_pg[NPASS], dw_t[NPASS];                         // pair group and first tap slot of each pass
+#pragma unroll
+        for (int ps = 0; ps < NPASS; ++ps) {
+            const int q = LIGHT ? pr * TH + ps * NU : 0;
+            dw_pg[ps] = LIGHT ? q / CQT : pr >> 1;
+            dw_t[ps] = LIGHT ? q - dw_pg[ps] * CQT : (pr & 1) * NU;
+        }
+        const bool dw_wave = !LIGHT || pr < NP - 1;
         f32x4 acc_k[NDB][DB], acc_v[2][DB];
 #pragma unroll
         for (int m = 0; m < 2; ++m)
@@ -680,6 +714,9 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
             ds_stored = false;
             __syncthreads();
             TS(1);
+            // (the LSE / D loads before the tile loads: the counted wait above relies on that order)
+            if (it + 1 < n_tiles) stage_stats(it + 1);
+            load_stats(r_begin + (it + 2) * BR);
             if (it + 1 < n_tiles) fetch_tile(it + 1);
             TS(2);
             const int u = it - 1, v = it - 2;
@@ -726,11 +763,14 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                 // read unconditionally: the producer writes zeros for a tile without dC; what the first
                 // iteration reads (nothing written yet) is dropped before any use
                 const unsigned char *Cl = smem + opaque((unsigned int)(c_stage(max(u, 0)) - smem) + 2 * n * CST + 4 * g * 2);
+                // the block after the pair's own keys: the first block of the next pair's stage (the last
+                // pair's producer writes it to its own stage)
+                const unsigned char *Cn = Cl + ((!LIGHT || pr == NP - 1) ? 2 * 32 : Lds::pair_bytes);
 #pragma unroll
                 for (int cb = 0; cb < NCB; ++cb)
 #pragma unroll
                     for (int f = 0; f < 2; ++f) {
-                        const u32x2 t2 = *reinterpret_cast<const u32x2 *>(Cl + f * CST + cb * 32);
+                        const u32x2 t2 = *reinterpret_cast<const u32x2 *>(cb < 2 ? Cl + f * CST + cb * 32 : Cn + f * CST);
                         cur_dc[cb][f][0] = t2[0];
                         cur_dc[cb][f][1] = t2[1];
                     }
@@ -802,15 +842,17 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
             // pair 2 pg + jb / 2, keys k0 + 64 pg - 8 + 16 jb ..), tap slots t_lo .. t_lo + TH - 1:
             // G_t[j][j'] += sum_rows dC[row][j] S[row + t - (CQT-1)][j'] with j' in the score block
             // 8 keys before the dC block (x = 0) and the one 8 keys after it (x = 1) ----
-            if (WANT_QW && u_in && !(CHAIN_ABLATE & 1)) {
+            if (WANT_QW && u_in && dw_wave && !(CHAIN_ABLATE & 1)) static_for<NPASS>([&](auto PS) {
+                constexpr int ps = decltype(PS)::value;
+                const int pg = dw_pg[ps], t_lo = dw_t[ps];
                 // Ring rows of this lane's two transpose reads at the wave's first tap slot: tile row 0
                 // at tap slot 0 is ring row wbase; the TH tap slots are consecutive rows (mod S_RING).
                 const int wbase = ((u + 1) * BR - (CQT - 1) + S_RING) % S_RING;
                 const unsigned int c_lane = opaque(tr_lane_off(CST, g, n));
                 const unsigned int ring0 = Lds::pair_off + 2 * pg * Lds::pair_bytes + 4 * (n & 3) * 2;
-                unsigned int a_lo[TH], a_hi[TH];
+                unsigned int a_lo[NU], a_hi[NU];
 #pragma unroll
-                for (int tt = 0; tt < TH; ++tt) {
+                for (int tt = 0; tt < NU; ++tt) {
                     const unsigned int ra = wbase + 4 * g + (n >> 2) + min(t_lo + tt, CQT - 1), rb = ra + 16;
                     a_lo[tt] = opaque(ring0 + min(ra, ra - S_RING) * SST);
                     a_hi[tt] = opaque(ring0 + min(rb, rb - S_RING) * SST);
@@ -819,9 +861,9 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                 // (blocks 0..3: a constant offset from the lane's address; block 4 is block 0 of the pair
                 // after the group or, for the last group, block 2 of its second pair: a[][] of it apart)
                 const unsigned int off4 = pg == NP / 2 - 1 ? Lds::pair_bytes + 64 : 2 * Lds::pair_bytes;
-                unsigned int a4_lo[TH], a4_hi[TH];
+                unsigned int a4_lo[NU], a4_hi[NU];
 #pragma unroll
-                for (int tt = 0; tt < TH; ++tt) { a4_lo[tt] = a_lo[tt] + off4; a4_hi[tt] = a_hi[tt] + off4; }
+                for (int tt = 0; tt < NU; ++tt) { a4_lo[tt] = a_lo[tt] + off4; a4_hi[tt] = a_hi[tt] + off4; }
                 auto s_frag = [&](auto JBP, int tt) {
                     constexpr int jbp = decltype(JBP)::value;
                     constexpr int off = (jbp >> 1) * Lds::pair_bytes + (jbp & 1) * 32;
@@ -845,34 +887,34 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                 // Software pipeline over the four key blocks: the operands of block jb + 1 are read
                 // while block jb is multiplied.  Every tap slot of the wave is multiplied, also the
                 // zero taps in front of a narrow window (their sums are not used).
-                f16x8 af = c_frag(0), b0[TH], b1[TH];
+                f16x8 af = c_frag(0), b0[NU], b1[NU];
 #pragma unroll
-                for (int tt = 0; tt < TH; ++tt) {
+                for (int tt = 0; tt < NU; ++tt) {
                     b0[tt] = s_frag(std::integral_constant<int, 0>{}, tt);
                     b1[tt] = s_frag(std::integral_constant<int, 1>{}, tt);
                 }
                 static_for<4>([&](auto JB) {
                     constexpr int jb = decltype(JB)::value;
-                    f16x8 af_n = af, b2[TH];
+                    f16x8 af_n = af, b2[NU];
 #pragma unroll
-                    for (int tt = 0; tt < TH; ++tt) b2[tt] = b1[tt];
+                    for (int tt = 0; tt < NU; ++tt) b2[tt] = b1[tt];
                     if constexpr (jb < 3) {
                         af_n = c_frag(jb + 1);
 #pragma unroll
-                        for (int tt = 0; tt < TH; ++tt) b2[tt] = s_frag(std::integral_constant<int, jb + 2>{}, tt);
-                        SCHED_DS_READ_ID(2 + 2 * TH, 40 + jb);
+                        for (int tt = 0; tt < NU; ++tt) b2[tt] = s_frag(std::integral_constant<int, jb + 2>{}, tt);
+                        SCHED_DS_READ_ID(2 + 2 * NU, 40 + 4 * ps + jb);
                     }
 #pragma unroll
-                    for (int tt = 0; tt < TH; ++tt) {
-                        acc_w[tt][0] = mfma_f16(af, b0[tt], acc_w[tt][0]);
-                        acc_w[tt][1] = mfma_f16(af, b1[tt], acc_w[tt][1]);
+                    for (int tt = 0; tt < NU; ++tt) {
+                        acc_w[ps * NU + tt][0] = mfma_f16(af, b0[tt], acc_w[ps * NU + tt][0]);
+                        acc_w[ps * NU + tt][1] = mfma_f16(af, b1[tt], acc_w[ps * NU + tt][1]);
                     }
-                    SCHED_MFMA_ID(2 * TH, 40 + jb);
+                    SCHED_MFMA_ID(2 * NU, 40 + 4 * ps + jb);
                     af = af_n;
 #pragma unroll
-                    for (int tt = 0; tt < TH; ++tt) { b0[tt] = b1[tt]; b1[tt] = b2[tt]; }
+                    for (int tt = 0; tt < NU; ++tt) { b0[tt] = b1[tt]; b1[tt] = b2[tt]; }
                 });
-            }
+            });
             CHAIN_SCHED_BARRIER;
             TS(5);
             if (WANT_KV && v_ok && !(CHAIN_ABLATE & 8)) {
@@ -914,13 +956,15 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
         __syncthreads();
         float *red = reinterpret_cast<float *>(smem + Lds::pair_off);
 #pragma unroll
-        for (int tt = 0; tt < TH; ++tt)
+        for (int ps = 0; ps < NPASS; ++ps)
 #pragma unroll
-            for (int x = 0; x < 2; ++x)
+            for (int tt = 0; tt < NU; ++tt)
 #pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    if (WANT_QW && t_lo + tt < CQT)
-                        red[(((pg * CQT + t_lo + tt) * 2 + x) * 16 + 4 * g + r) * 16 + n] = acc_w[tt][x][r];
+                for (int x = 0; x < 2; ++x)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (WANT_QW && dw_wave && dw_t[ps] + tt < CQT)
+                            red[(((dw_pg[ps] * CQT + dw_t[ps] + tt) * 2 + x) * 16 + 4 * g + r) * 16 + n] = acc_w[ps * NU + tt][x][r];
         __syncthreads();  // the producers add the dW partial up while the consumers store dK and dV
 
         // ---- stores: lane = key, 4 consecutive head-dim columns per block ----
