@@ -102,8 +102,9 @@ def executed_mfma_flops(wl: Workload, two_pass: bool = False) -> Dict[str, objec
       the keys in 32-key steps up to its last row + 16: per step S^T 2 (row fragments) x 2 (key
       blocks) x d/32, convolution 4 T, P V 2 x d/16 MFMAs.
     key-stationary backward: a wave pair owns 32 keys and walks 32-row tiles from the first row that
-      sees its keys: per tile S^T 8 d/32 (64 keys for 32 owned), convolution 6 T (48 keys), dP 6 d/32,
-      transposed convolution 4 T, dV and dK 2 d/16 each, dW 4 T MFMAs.
+      sees its keys: per tile S^T 6 d/32 (48 keys for 32 owned), convolution 4 T (32 keys), dP 4 d/32,
+      transposed convolution 4 T, dV and dK 2 d/16 each, dW 4 T MFMAs; the last of a workgroup's four
+      pairs also computes the 16 keys after its own (S^T 8 d/32, convolution 6 T, dP 6 d/32).
     dQ = dS K: 2 x d/16 per 32 rows x 32 keys below the diagonal (nothing wasted but the diagonal
       blocks' upper halves).
     """
@@ -116,25 +117,28 @@ def executed_mfma_flops(wl: Workload, two_pass: bool = False) -> Dict[str, objec
         wg_end = min(N, (w0 // (4 * rows) + 1) * 4 * rows)          # its workgroup's last row + 1
         steps = min((w0 + rows + 15) // 32 + 1, (wg_end + 16 + 31) // 32)
         fwd += steps * (4 * d // 32 + 4 * T + 2 * d // 16)
-    per_tile = 8 * d // 32 + 6 * T + 6 * d // 32 + 4 * T + 4 * d // 16 + 4 * T
-    per_tile_kv = per_tile - 4 * T                     # dK / dV pass: no dW
-    per_tile_qw = per_tile - 4 * d // 16               # dQ + dW pass: no dV, dK
-    tiles = s_only = 0
+    consumer = 4 * T + 4 * d // 16 + 4 * T             # transposed convolution, dV and dK, dW
+    light, heavy = 6 * d // 32 + 4 * T + 4 * d // 32, 8 * d // 32 + 6 * T + 6 * d // 32
+    full = kv = qw = s_only = 0
     for c0 in range(0, (N + 8 + 127) // 128 * 128, 32):   # one wave pair per 32 keys
         k0 = c0 // 128 * 128
+        last = c0 - k0 == 96                            # the last pair of its workgroup
         r_begin = max(0, k0 - 8) // 32 * 32
         n_t = max(0, (N - r_begin + 31) // 32)
         skipped = sum(1 for t in range(n_t) if r_begin + 32 * t + 31 < c0 - 8)   # scores only
-        tiles += n_t - skipped
-        s_only += skipped + 1                           # + the 32 rows above the first tile
+        producer = heavy if last else light
+        full += (n_t - skipped) * (producer + consumer)
+        kv += (n_t - skipped) * (producer + consumer - 4 * T)          # dK / dV pass: no dW
+        qw += (n_t - skipped) * (producer + consumer - 4 * d // 16)    # dQ + dW pass: no dV, dK
+        s_only += (skipped + 1) * (8 if last else 6) * d // 32         # + the 32 rows above the first tile
     dq = sum((min(N, (r // 128 + 1) * 128) + 63) // 64 * 2 for r in range(0, N, 32)) * 2 * d // 16
     out = {"fwd": fwd * mf * bh}
     if wl.backward:
         if two_pass:
-            out["bwd_dkdv"] = (tiles * per_tile_kv + s_only * 8 * d // 32) * mf * bh
-            out["bwd_dq_dw"] = (tiles * per_tile_qw + s_only * 8 * d // 32 + dq) * mf * bh
+            out["bwd_dkdv"] = (kv + s_only) * mf * bh
+            out["bwd_dq_dw"] = (qw + s_only + dq) * mf * bh
         else:
-            out["bwd_fused_dkdv"] = (tiles * per_tile + s_only * 8 * d // 32) * mf * bh
+            out["bwd_fused_dkdv"] = (full + s_only) * mf * bh
             out["bwd_fused_dq"] = dq * mf * bh
     total = sum(out.values())
     fl = useful_flops(wl)
