@@ -17,6 +17,11 @@
 // One workgroup barrier per tile; Q and dO tiles go from global memory straight into LDS (buffer
 // loads with the LDS modifier, one tile ahead), in a layout that serves both the 128-bit row
 // fragment reads of the producers and the 64-bit transpose reads of dV / dK (see ChainLds).
+// The transposed convolution of a pair's 32 keys needs dC on the 16 keys after them as well: that
+// block is the first block of the next pair, so (windows of up to 6 query taps) only the last pair
+// of a workgroup computes it itself and the other consumers read it from the next pair's stage;
+// the last pair's consumer, which shares its SIMD with that heavier producer, leaves dW to the
+// other three consumers and stages the LSE / D values of the tiles instead.
 //
 // dW[a][b] = sum_i sum_j dC[i][j] S_m[i+a-pq][j+b-pk] is computed as G_a = dC^T S(rows shifted by
 // a), a [key j] x [key j'] product contracted over the rows on the matrix cores; only its
