@@ -40,6 +40,9 @@ UNITS = [
     ("bwd_chain_mfma.hip", "bwd_chain_mfma_all", ["-DCONVATTN_CHAIN_UNIT=3"]),
     ("bwd_chain_mfma.hip", "bwd_chain_mfma_kv", ["-DCONVATTN_CHAIN_UNIT=1"]),
     ("bwd_chain_mfma.hip", "bwd_chain_mfma_qw", ["-DCONVATTN_CHAIN_UNIT=2"]),
+    ("bwd_chain3_mfma.hip", "bwd_chain3_mfma_all", ["-DCONVATTN_CHAIN_UNIT=3"]),
+    ("bwd_chain3_mfma.hip", "bwd_chain3_mfma_kv", ["-DCONVATTN_CHAIN_UNIT=1"]),
+    ("bwd_chain3_mfma.hip", "bwd_chain3_mfma_qw", ["-DCONVATTN_CHAIN_UNIT=2"]),
     ("bwd_dq_rows.hip", "bwd_dq_rows", []),
     ("decode_stream.hip", "decode_stream", []),
     ("headmix_attn.hip", "headmix_attn", []),

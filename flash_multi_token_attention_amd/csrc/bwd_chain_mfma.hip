@@ -34,138 +34,15 @@
 // and (in the dQ product) dQ are multiplied by its inverse when they are stored.
 #include <type_traits>
 
-#include "mfma_common.hpp"
+#include "chain_common.hpp"
 
 namespace convattn {
 namespace {
 
-typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+using namespace chain;
 
-constexpr int NP = 4;            // wave pairs = 32-key ranges per workgroup
+
 constexpr int NT = 2 * NP * 64;  // 512 threads
-constexpr int WK = 32;           // own keys per pair
-constexpr int BKW = NP * WK;     // 128 keys per workgroup
-constexpr int BR = 32;           // query rows per tile
-constexpr int NSB = 4;           // S^T blocks of a pair: keys c0-16+16kb
-constexpr int NCB = 3;           // C / dP / dC blocks: keys c0-8+16cb
-constexpr int NDB = 2;           // dS blocks: keys c0+16sb
-constexpr int SST = 112;         // bytes per row of the S tile in LDS (48 keys fp16 + 16)
-constexpr int S_RING = 72;       // rows of the S ring: a tile being written, the tile before it and 8 rows more (>= c_q - 1)
-constexpr int CST = 112;         // bytes per row of the dC tile (48 keys fp16 + 16)
-constexpr int PST = 72;          // bytes per row of the P and dS tiles (32 keys bf16 + 8)
-static_assert(BKW == kKvKeysPerWg && WK == kChainKeys && BR == kChainRows, "dS workspace layout");
-
-template <int D, int CQT> struct ChainLds {
-    // Q / dO tiles are filled by buffer loads with the LDS modifier (64 lanes = 1 KB of consecutive
-    // LDS), which rules out padded rows.  A tile of 32 rows is kept as [k-step ks][row parity f]
-    // [row pair n][64 bytes]: the 4 chunks of 16 bytes that row 2n + f holds of head-dim columns
-    // 32 ks .. 32 ks + 31, chunk c at position c ^ (n / 4 mod 4).  Row fragments (lane n reads row
-    // 2n + f) and transposed fragments then touch every bank equally often, and k-step, parity and
-    // head-dim block are constant offsets from one lane address.
-    static constexpr int RST = D * 2;                               // bytes per Q / dO row
-    static constexpr int tile_bytes = BR * RST;
-    static constexpr int q_off = 0, q_slots = 4;                    // tiles it-2 .. it+1
-    static constexpr int g_off = q_off + q_slots * tile_bytes, g_slots = 3;  // tiles it-1 .. it+1
-    static constexpr int stat_off = g_off + g_slots * tile_bytes;   // LSE and D of a tile: two slots
-    static constexpr int stat_bytes = 2 * (2 * BR * 4);
-    static constexpr int band_off = stat_off + stat_bytes;          // bands, then flipped bands: one KB per tap slot
-    static constexpr int band_bytes = 2 * CQT * 1024;
-    static constexpr int pair_off = band_off + band_bytes;
-    static constexpr int s_bytes = S_RING * SST;
-    static constexpr int c_bytes = 2 * BR * CST;
-    static constexpr int p_bytes = 2 * BR * PST;
-    static constexpr int ds_bytes = BR * PST;
-    static constexpr int pair_bytes = s_bytes + c_bytes + p_bytes + ds_bytes;
-    static constexpr int total = pair_off + NP * pair_bytes;
-    static_assert(CQT * 2 * 1024 <= pair_bytes, "room for the dW accumulators");
-};
-
-// A lane-dependent LDS offset the compiler may not fold or hoist: what is added to it afterwards
-// stays a constant and ends up in the instructions' offset fields instead of one address register
-// per fragment.
-__device__ __forceinline__ unsigned int opaque(unsigned int x) {
-    asm volatile("" : "+v"(x));
-    return x;
-}
-
-__device__ __forceinline__ bf16x4 lds_tr64(const unsigned char *ptr) {
-    typedef short s16x4 __attribute__((ext_vector_type(4)));
-    s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(ptr));
-    return __builtin_bit_cast(bf16x4, v);
-}
-// Transposed fragment of a row-major tile of 16-bit elements with `stride` bytes per row:
-// k = rows 4g .. 4g+3 then 16+4g .. 16+4g+3, column col0 + n.  `lane_ptr` is the tile's address plus
-// tr_lane_off(stride, g, n).
-__device__ __forceinline__ unsigned int tr_lane_off(int stride, int g, int n) {
-    return (4 * g + (n >> 2)) * stride + 4 * (n & 3) * 2;
-}
-__device__ __forceinline__ bf16x8 read_tr(const unsigned char *lane_ptr, int stride, int col0) {
-    bf16x4 lo = lds_tr64(lane_ptr + col0 * 2);
-    bf16x4 hi = lds_tr64(lane_ptr + 16 * stride + col0 * 2);
-    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-}
-
-template <int CTRL>
-__device__ __forceinline__ unsigned int dpp_keep(unsigned int old, unsigned int src) {
-    return (unsigned int)__builtin_amdgcn_update_dpp((int)old, (int)src, CTRL, 0xf, 0xf, false);
-}
-// A DPP move that writes every lane (rotations): no previous value to keep.
-template <int CTRL>
-__device__ __forceinline__ unsigned int dpp_mov(unsigned int src) {
-    return (unsigned int)__builtin_amdgcn_mov_dpp((int)src, CTRL, 0xf, 0xf, true);
-}
-// Lane n of a row of 16 gets cur[n - S] for n >= S and prev[16 + n - S] below: a window that
-// starts S lanes before `cur` in the sequence prev | cur.
-template <int S>
-__device__ __forceinline__ unsigned int win_up(unsigned int prev, unsigned int cur) {
-    if constexpr (S == 0) {
-        return cur;
-    } else {
-        const unsigned int x = dpp_mov<0x120 + S>(prev);  // row_ror:S
-        return dpp_keep<0x110 + S>(x, cur);               // row_shr:S, lanes below S keep x
-    }
-}
-// Lane n gets a[n + S] for n + S < 16 and b[n + S - 16] above: a window that starts S lanes into
-// `a` in the sequence a | b.
-template <int S>
-__device__ __forceinline__ unsigned int win_down(unsigned int a, unsigned int b) {
-    if constexpr (S == 0) {
-        return a;
-    } else {
-        const unsigned int x = dpp_mov<0x120 + 16 - S>(b);  // row_ror:(16-S)
-        return dpp_keep<0x100 + S>(x, a);                   // row_shl:S, the last S lanes keep x
-    }
-}
-
-__device__ __forceinline__ unsigned int pack_f16_rtz(float a, float b) {
-    return __builtin_bit_cast(unsigned int, __builtin_amdgcn_cvt_pkrtz(a, b));
-}
-
-// Toeplitz bands for the packed operand order: k slot 8g+e of a 32-key window is key 4g+e of its
-// first 16-key block for e < 4 and key 4g+e-4 of its second for e >= 4; the output block starts 8
-// keys into the window.  Tap slot t stands for query tap a = t - (CQT - c_q) (zero taps in front).
-// `flip` builds the bands of the transposed convolution.
-template <int CQT>
-__device__ __forceinline__ f16x8 band_frag(int t, const float *__restrict__ w_head, int c_q, int c_k, int pk,
-                                           int g, int n, bool flip, float mul) {
-    const int a = t - (CQT - c_q);
-    // (unconditional loads from clamped indices: the eight of a fragment are in flight together)
-    const float *row = w_head + max(a, 0) * c_k;
-    float v[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        const int kappa = e < 4 ? 4 * g + e : 16 + 4 * g + e - 4;
-        const int off = kappa - kKeyHalo - n;
-        const int bb = flip ? pk - off : pk + off;
-        v[e] = row[min(max(bb, 0), c_k - 1)];
-        if (a < 0 || bb < 0 || bb >= c_k) v[e] = 0.f;
-    }
-    f16x8 f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) f[e] = (_Float16)(v[e] * mul);
-    return f;
-}
-
 #ifndef CHAIN_PF
 #define CHAIN_PF 3
 #endif
@@ -211,26 +88,6 @@ __device__ long long g_chain_ts[8][64][12];
 #else
 #define TS(i)
 #define TSX(a, b)
-#endif
-
-// Kernel arguments as one block: each role reads them from the kernel argument segment with
-// scalar loads (arguments of a device function would arrive in vector registers).
-struct ChainArgs {
-    Problem p;
-    const bf16_t *Q, *K, *V, *dO;
-    const float *Dl, *LSE, *W, *dc_scale;
-    void *dK, *dV;
-    bf16_t *dS_ws;
-    float *dW_part;
-    int n_rt;
-};
-
-// The kernel argument segment lives in the constant address space; host passes of the compiler
-// do not know that attribute.
-#if defined(__HIP_DEVICE_COMPILE__)
-#define CHAIN_CONST_AS __attribute__((address_space(4)))
-#else
-#define CHAIN_CONST_AS
 #endif
 
 // One role of the workgroup (ROLE 0 = producer waves, 1 = consumer waves).  The two roles have
@@ -355,21 +212,28 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
     // role whose wave does it (its first 32 lanes): the last consumer wave where it has the lightest
     // iteration (LIGHT), else the first producer wave.
     constexpr bool STAT_ROLE = (ROLE == 1) == LIGHT;
-    const int stat_tt = tid - (LIGHT ? NT - 64 : 0);
+    // (a wave-uniform test, i.e. a branch: the other waves of the role must not even touch `ls` / `dd`, whose
+    // reuse as load destinations makes the compiler wait for every outstanding vector memory operation of the
+    // wave, the dS stores of the last iteration among them)
+    const bool stat_wave = STAT_ROLE && wave == (LIGHT ? 2 * NP - 1 : 0);
     float ls = 0.f, dd = 0.f;
     auto load_stats = [&](int r0) {
         if constexpr (STAT_ROLE) {
-            // raw values: arithmetic on them here would wait for the loads in this iteration
-            const int tt = (int)opaque((unsigned int)stat_tt);
-            ls = 1e30f; dd = 0.f;  // rows past the end: exp2(C - LSE) = 0
-            if (tt >= 0 && tt < BR && r0 + tt < p.Nq) { ls = lse_b[r0 + tt]; dd = dl_b[r0 + tt]; }
+            if (stat_wave) {
+                // raw values: arithmetic on them here would wait for the loads in this iteration
+                const int tt = (int)opaque((unsigned int)lane);
+                ls = 1e30f; dd = 0.f;  // rows past the end: exp2(C - LSE) = 0
+                if (tt < BR && r0 + tt < p.Nq) { ls = lse_b[r0 + tt]; dd = dl_b[r0 + tt]; }
+            }
         }
     };
     auto stage_stats = [&](int t) {
         if constexpr (STAT_ROLE) {
-            const int tt = (int)opaque((unsigned int)stat_tt);
-            float *st = stat_slot(t);
-            if (tt >= 0 && tt < BR) { st[tt] = ls * kLog2e - dcs_log2; st[BR + tt] = dd; }
+            if (stat_wave) {
+                const int tt = (int)opaque((unsigned int)lane);
+                float *st = stat_slot(t);
+                if (tt < BR) { st[tt] = ls * kLog2e - dcs_log2; st[BR + tt] = dd; }
+            }
         }
     };
     // Lane parts of the fragment addresses inside a tile.  Row fragment (producers): row 2n + f,
@@ -468,13 +332,9 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                                 if (key0 + r > qpos) acc[kb][f][r] = 0.f;
                         }
                     }
-                    // rounded and clamped exactly as the forward rounds its scores: P = exp2(C - LSE)
+                    // rounded exactly as the forward rounds its scores: P = exp2(C - LSE)
                     // only sums to one over a row if C is the C the forward's LSE was taken from
-                    f16x4 hv;
-#pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        hv[r] = (_Float16)__builtin_amdgcn_fmed3f(acc[kb][f][r], -kF16Max, kF16Max);
-                    const u32x2 two = __builtin_bit_cast(u32x2, hv);
+                    const u32x2 two = pack_scores_f16(acc[kb][f]);
                     pd[kb][f][0] = two[0];
                     pd[kb][f][1] = two[1];
                     if (WANT_QW && kb < 3) {
@@ -830,7 +690,9 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                         // block layout [row parity][key half][16 row pairs][16 keys]: the 64 lanes of a store
                         // write 512 contiguous bytes
                         if constexpr (WANT_QW) {
-                            *reinterpret_cast<bf16x4 *>(ds_blk + ((ob * 2 + sb) * 16 + n) * 16 + 4 * g) = sv;
+                            // (non-temporal: read once, by another kernel; kept out of the L2)
+                            __builtin_nontemporal_store(__builtin_bit_cast(u32x2, sv),
+                                                        reinterpret_cast<u32x2 *>(ds_blk + ((ob * 2 + sb) * 16 + n) * 16 + 4 * g));
                             ds_stored = true;
                         }
                         if constexpr (WANT_KV) *reinterpret_cast<bf16x4 *>(ds_tile + (2 * n + ob) * PST + (sb * 16 + 4 * g) * 2) = sv;

@@ -224,11 +224,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_mfma_kernel(
                         for (int r = 0; r < 4; ++r)
                             if (key0 + r > qpos) acc[kb][r] = 0.f;
                     }
-                    f16x4 hv;
-#pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        hv[r] = (_Float16)__builtin_amdgcn_fmed3f(acc[kb][r], -kF16Max, kF16Max);
-                    *reinterpret_cast<f16x4 *>(Ss + (rb * 16 + n) * SST + (kb * 16 + 4 * g) * 2) = hv;
+                    *reinterpret_cast<u32x2 *>(Ss + (rb * 16 + n) * SST + (kb * 16 + 4 * g) * 2) = pack_scores_f16(acc[kb]);
                 }
             });
         }

@@ -28,7 +28,6 @@
 namespace convattn {
 namespace {
 
-typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 // DPP move (CTRL 0x110+s: row_shr:s, lane n of a row of 16 gets lane n-s); lanes without a
 // source lane get 0.
@@ -262,7 +261,7 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
         load_kf(0);
         static_for<2>([&](auto BL) {
             constexpr int blk = decltype(BL)::value;
-            // ---- S^T = K Q^T (raw), pre-mask, clamp, pack two keys per dword ----
+            // ---- S^T = K Q^T (raw), pre-mask, pack two keys per dword ----
             f32x4 acc[2];
 #pragma unroll
             for (int f = 0; f < 2; ++f) acc[f] = (f32x4){0.f, 0.f, 0.f, 0.f};
@@ -286,11 +285,7 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
                             if (key0 + r > qpos) acc[f][r] = 0.f;
                     }
                 }
-                f16x4 hv;
-#pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    hv[r] = (_Float16)__builtin_amdgcn_fmed3f(acc[f][r], -kF16Max, kF16Max);
-                const auto two = __builtin_bit_cast(u32x2, hv);
+                const u32x2 two = pack_scores_f16(acc[f]);
                 pd[blk][f][0] = two[0];
                 pd[blk][f][1] = two[1];
             }

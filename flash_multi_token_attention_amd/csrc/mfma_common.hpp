@@ -26,6 +26,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 // Five consecutive dwords at a 4-byte boundary of LDS, as 32-bit reads (the compiler pairs them
 // into ds_read2_b32).  A 128-bit LDS read that is not 16-byte aligned is legal on gfx950 but slow:
 // measured with four waves reading, one costs about 66 clocks of the LDS pipe against about 12 for
@@ -39,7 +40,7 @@ __device__ __forceinline__ void lds_read_dwords5(const unsigned char *p, u32x4 &
 constexpr int kKeyHalo = 8;          // LDS columns before a block's first output key
 constexpr int kMfmaMaxPk = 8;        // so c_k <= 17 on the MFMA path
 constexpr float kLog2e = 1.4426950408889634f;
-constexpr float kF16Max = 65504.f;
+constexpr float kF16Max = 65504.f;   // what a score beyond fp16's range is rounded to
 
 __device__ __forceinline__ f32x4 mfma_bf16(bf16x8 a, bf16x8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
@@ -77,6 +78,15 @@ __device__ __forceinline__ unsigned int lane_from_next(unsigned int v) {
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Four raw scores to fp16, two per dword (one v_cvt_pkrtz_f16_f32 per pair).  Rounded toward zero:
+// a finite score beyond fp16's range becomes +-65504 instead of infinity, so no clamp is needed.
+// Every kernel of the forward and the backward rounds its scores with this function: P = exp2(C - LSE)
+// only sums to one over a row if C is the C the forward's LSE was taken from.
+__device__ __forceinline__ u32x2 pack_scores_f16(f32x4 s) {
+    return (u32x2){__builtin_bit_cast(unsigned int, __builtin_amdgcn_cvt_pkrtz(s[0], s[1])),
+                   __builtin_bit_cast(unsigned int, __builtin_amdgcn_cvt_pkrtz(s[2], s[3]))};
+}
 
 // Toeplitz fragment of query tap `a` for this lane: element e is
 // W[a][b], b = (8g + e) - 8 - n + pk, zero outside the window.  `flip` builds the
@@ -281,11 +291,21 @@ hipError_t mfma_dc_scale(const Problem &p, const void *d_o, const void *v, float
 CHAIN_DECL(mfma_bwd_chain_kv);
 CHAIN_DECL(mfma_bwd_chain_qw);
 CHAIN_DECL(mfma_bwd_chain_all);
+// the same with three waves per SIMD (bwd_chain3_mfma.hip): windows of up to 6 query taps
+CHAIN_DECL(mfma_bwd_chain3_kv);
+CHAIN_DECL(mfma_bwd_chain3_qw);
+CHAIN_DECL(mfma_bwd_chain3_all);
 #undef CHAIN_DECL
+bool chain3_enabled();
 inline hipError_t mfma_bwd_chain(const Problem &p, int out_dt, int want, const void *q, const void *k, const void *v,
                                  const void *d_o, const float *Dl, const float *lse, const float *w,
                                  const float *dc_scale, void *dk, void *dv, void *ds_ws, float *dw_part,
                                  hipStream_t s) {
+    if (p.c_q <= 6 && chain3_enabled()) {
+        if (want == 1) return mfma_bwd_chain3_kv(p, out_dt, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
+        if (want == 2) return mfma_bwd_chain3_qw(p, out_dt, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
+        return mfma_bwd_chain3_all(p, out_dt, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
+    }
     if (want == 1) return mfma_bwd_chain_kv(p, out_dt, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
     if (want == 2) return mfma_bwd_chain_qw(p, out_dt, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
     return mfma_bwd_chain_all(p, out_dt, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
