@@ -27,6 +27,19 @@ namespace {
 using namespace chain;
 
 constexpr int NT3 = 3 * NP * 64;  // 768 threads
+// Wave priorities (s_setprio): the wave of a SIMD that has the least slack before the barrier issues first.
+#ifndef C3_PRIO_SCORE
+#define C3_PRIO_SCORE 1   // score waves, MFMA phases (0 in the P / dC arithmetic)
+#endif
+#ifndef C3_PRIO_EXTRA
+#define C3_PRIO_EXTRA 3   // the value wave that also computes the block after the workgroup's keys
+#endif
+#ifndef C3_PRIO_VALUE
+#define C3_PRIO_VALUE 1   // value waves
+#endif
+#ifndef C3_PRIO_KEY
+#define C3_PRIO_KEY 0     // key waves
+#endif
 // LDS: the layout of the two-role kernel, then the V fragments of the block after the workgroup's keys
 // (16 rows; the wave that computes that block has no registers to keep them in)
 template <int D, int CQT> struct Chain3Lds : ChainLds<D, CQT> {
@@ -284,7 +297,7 @@ __device__ __forceinline__ void chain3_role(const CHAIN_CONST_AS ChainArgs *args
                 constexpr bool FULL = decltype(full_tag)::value;
                 const unsigned char *Qs = smem + opaque((unsigned int)(q_slot(it) - smem) + row_frag_off());
                 const unsigned char *Gs = smem + opaque((unsigned int)(g_slot(it) - smem) + row_frag_off());
-                __builtin_amdgcn_s_setprio(1);
+                __builtin_amdgcn_s_setprio(VLDS ? C3_PRIO_EXTRA : C3_PRIO_SCORE);
                 f32x4 dp[NCBL][2];
                 float2 l2 = {0.f, 0.f};
                 if constexpr (FULL) l2 = *reinterpret_cast<const float2 *>(stat_slot(it) + 2 * n);
@@ -293,6 +306,8 @@ __device__ __forceinline__ void chain3_role(const CHAIN_CONST_AS ChainArgs *args
                 s_phase(r0, it + 1, pd, edge_tag, [&](int f, int ks) {
                     return *reinterpret_cast<const bf16x8 *>(Qs + f * 1024 + ks * 2048);
                 });
+                // (the instance beside the dV accumulators has no registers for phases that overlap)
+                if constexpr (VLDS) __builtin_amdgcn_sched_barrier(0);
                 if constexpr (FULL) {
                     unsigned char *Cs = c_stage(it), *Ps = p_stage(it);
                     // ---- convolution: C^T block cb from score blocks cb (k slots 0..3 of a lane
@@ -331,6 +346,7 @@ __device__ __forceinline__ void chain3_role(const CHAIN_CONST_AS ChainArgs *args
 #pragma unroll
                         for (int f = 0; f < 2; ++f) { prev_pd[kb][f][0] = pd[kb][f][0]; prev_pd[kb][f][1] = pd[kb][f][1]; }
                     // ---- dP^T = V dO^T - D, after the convolution (the shifted score windows are no longer live) ----
+                    if constexpr (VLDS) __builtin_amdgcn_sched_barrier(0);
                     {
                         const float2 d2 = *reinterpret_cast<const float2 *>(stat_slot(it) + BR + 2 * n);
 #pragma unroll
@@ -354,9 +370,10 @@ __device__ __forceinline__ void chain3_role(const CHAIN_CONST_AS ChainArgs *args
                         }
                     }
                     // ---- P = exp2(C - LSE) (times the dC scale), dC = P dP ----
+                    if constexpr (VLDS) __builtin_amdgcn_sched_barrier(0);
                     static_for<NCBL>([&](auto CB) {
                         constexpr int cb = decltype(CB)::value, cba = CB0 + cb;
-                        __builtin_amdgcn_s_setprio(0);
+                        __builtin_amdgcn_s_setprio(VLDS ? C3_PRIO_EXTRA : 0);
 #pragma unroll
                         for (int ob = 0; ob < 2; ++ob) {
                             f32x4 prob, dc;
@@ -448,10 +465,10 @@ __device__ __forceinline__ void chain3_role(const CHAIN_CONST_AS ChainArgs *args
 #pragma unroll
             for (int db = 0; db < DB; ++db) acc_v[m][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
         // dV^T += dO^T P of tile u (keys c0-8 .. c0+23)
-        auto dv_phase = [&](int u) {
+        auto dv_phase = [&](int u, auto prio_tag) {
             const unsigned char *Ps = smem + opaque((unsigned int)(p_stage(u) - smem) + tr_lane_off(PST, g, n));
             const unsigned char *Gs = smem + opaque((unsigned int)(g_slot(u) - smem) + tr_frag_off());
-            __builtin_amdgcn_s_setprio(1);
+            __builtin_amdgcn_s_setprio(decltype(prio_tag)::value);
             constexpr int PF = 3;
             bf16x8 pf[2], gq[PF + 1];
 #pragma unroll
@@ -468,7 +485,6 @@ __device__ __forceinline__ void chain3_role(const CHAIN_CONST_AS ChainArgs *args
                 for (int cb = 0; cb < 2; ++cb) acc_v[cb][db] = mfma_bf16(gq[db % (PF + 1)], pf[cb], acc_v[cb][db]);
                 SCHED_MFMA_ID(2, 60 + db);
             });
-            __builtin_amdgcn_s_setprio(0);
         };
         auto store_dv = [&] {
             const float inv = 1.f / dcs;
@@ -500,7 +516,8 @@ __device__ __forceinline__ void chain3_role(const CHAIN_CONST_AS ChainArgs *args
                     __syncthreads();
                     if (it + 1 < n_tiles) fetch_tile(it + 1);
                     const int u = it - 1;
-                    if (WANT_KV && it >= 1 && u < n_tiles && !is_skipped(r_begin + u * BR)) dv_phase(u);
+                    if (WANT_KV && it >= 1 && u < n_tiles && !is_skipped(r_begin + u * BR)) dv_phase(u, std::integral_constant<int, C3_PRIO_EXTRA>{});
+                    __builtin_amdgcn_sched_barrier(0);
                     tile(it);
                 }
             });
@@ -527,7 +544,7 @@ __device__ __forceinline__ void chain3_role(const CHAIN_CONST_AS ChainArgs *args
                 if (it + 1 < n_tiles) fetch_tile(it + 1);
                 const int u = it - 1;
                 const bool u_in = it >= 1 && u < n_tiles;
-                if (WANT_KV && u_in && !is_skipped(r_begin + u * BR)) dv_phase(u);
+                if (WANT_KV && u_in && !is_skipped(r_begin + u * BR)) dv_phase(u, std::integral_constant<int, C3_PRIO_VALUE>{});
                 // ---- dW, key blocks jb = 0..3 of the triples 2 pg and 2 pg + 1 (block jb = dC block jb & 1 of
                 // triple 2 pg + jb / 2, keys k0 + 64 pg - 8 + 16 jb ..), tap slots t_lo .. t_lo + NU - 1:
                 // G_t[j][j'] += sum_rows dC[row][j] S[row + t - (CQT-1)][j'] with j' in the score block
@@ -668,7 +685,7 @@ __device__ __forceinline__ void chain3_role(const CHAIN_CONST_AS ChainArgs *args
             }
             if (v_ok) {
                 bf16_t *ds_blk = ds_pair + (size_t)(r0v / BR) * (WK * BR);
-                __builtin_amdgcn_s_setprio(2);
+                __builtin_amdgcn_s_setprio(C3_PRIO_KEY);
                 // ---- dS^T of tile v: rows below it come from tile v+1.  Operand of row offset
                 // e = parity + (CQT-1 - tap slot): fragment e & 1 shifted e >> 1 lanes up. ----
                 f32x4 ds[NDB][2];
@@ -732,7 +749,6 @@ __device__ __forceinline__ void chain3_role(const CHAIN_CONST_AS ChainArgs *args
                 const unsigned char *Dsl = smem + opaque((unsigned int)(ds_tile - smem) + tr_lane_off(PST, g, n));
                 asm volatile("" ::: "memory");
                 __builtin_amdgcn_wave_barrier();
-                __builtin_amdgcn_s_setprio(1);
                 // ---- dK^T += Q^T dS ----
                 {
                     constexpr int PF = 3;
@@ -755,7 +771,6 @@ __device__ __forceinline__ void chain3_role(const CHAIN_CONST_AS ChainArgs *args
                 asm volatile("" ::: "memory");
                 __builtin_amdgcn_wave_barrier();
             }
-            __builtin_amdgcn_s_setprio(0);
         }
         __syncthreads();
         __syncthreads();
