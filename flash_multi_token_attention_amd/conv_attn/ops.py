@@ -178,7 +178,18 @@ def dq_backward(Q, K, V, dO, D, L, conv_kernel, scale, pad_q, pad_k, causal,
     nbytes = lib.convattn_dw_partial_bytes(C.byref(desc))
     if nbytes == 0:
         _lib.check(lib.convattn_validate(C.byref(desc), _lib.OP_BWD), "conv_attn.dq_backward")
-    part = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=Q.device)
+    # The dS scratch is O(Nq*Nk): above the workspace cap, or when the allocation fails, the
+    # query-stationary kernel with O(N) scratch runs instead (same results within the tolerances).
+    part = None
+    if nbytes <= max_workspace_bytes() or low_memory:
+        try:
+            part = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=Q.device)
+        except torch.OutOfMemoryError:
+            if low_memory:
+                raise
+    if part is None:
+        return dq_backward(Q, K, V, dO, D, L, conv_kernel, scale, pad_q, pad_k, causal, out_dtype, exact,
+                           low_memory=True)
     dW = torch.empty(W.shape, dtype=torch.float32, device=Q.device)
     st = _stream(Q)
     rc = lib.convattn_bwd_dq_dw(C.byref(desc), _ptr(Q), _ptr(K), _ptr(V), _ptr(dO), _ptr(D), _ptr(L),

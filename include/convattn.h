@@ -13,14 +13,16 @@
  *   - Every tensor pointer is a DEVICE address of a dense row-major array:
  *     Q [B,H,Nq,d], K,V [B,H,Nk,d], W [H,c_q,c_k] (always fp32), statistics
  *     M, L, D, LSE [B,H,Nq] (always fp32).  Pointers must be 16-byte aligned.
- *   - The library never allocates, frees or keeps device memory: the caller
- *     owns inputs, outputs and the partial buffers whose sizes the
- *     *_partial_bytes() queries return.
+ *   - The library never allocates or frees device memory: the caller owns
+ *     inputs, outputs and the work buffers whose sizes the *_bytes() queries
+ *     return.  One exception, convattn_decode_noalloc, keeps its scratch in a
+ *     built-in device array of fixed size (see its declaration).
  *   - Every launch is asynchronous on the hipStream_t passed as `stream`
  *     (NULL = the null stream); no entry point synchronises the device.
  *   - Return value: 0 = ok, < 0 = convattn_status (argument rejected before any
  *     HIP call), > 0 = hipError_t of a failed launch.
- *   - The functions are re-entrant and keep no state between calls.
+ *   - The functions are re-entrant and keep no state between calls, except
+ *     convattn_decode_noalloc: calls that overlap on one GPU share its scratch.
  *
  * Each entry point names the interface of Gusanidas/flash-multi-token-attention
  * that it replaces (paths relative to flash_multi_token_attention/).
@@ -35,7 +37,7 @@
 extern "C" {
 #endif
 
-#define CONVATTN_VERSION 100 /* major*10000 + minor*100 + patch */
+#define CONVATTN_VERSION 300 /* major*10000 + minor*100 + patch */
 
 typedef enum convattn_dtype {
     CONVATTN_BF16 = 0,
@@ -129,7 +131,13 @@ int convattn_bwd_preprocess(const convattn_desc *desc, const void *o, const void
                             const float *m, const float *l, float *D, float *lse,
                             void *stream);
 
-/* Bytes of the dW partial buffer convattn_bwd_dq_dw writes (0 on a bad descriptor). */
+/*
+ * Bytes of the work buffer convattn_bwd_dq_dw needs (0 on a bad descriptor).  On the
+ * bf16 matrix-core path with windows of up to 8 query taps this is the whole workspace of the
+ * key-stationary kernel: the bf16 dS matrix, B*H*Nq*Nk*2 bytes (2.2 GB at B4 H16 N4096),
+ * plus the dW partials and the dC scales.  With CONVATTN_FLAG_LOW_MEMORY in desc->flags
+ * (and on every other path) it is the dW partials only, O(B*H*Nq/128) floats.
+ */
 size_t convattn_dw_partial_bytes(const convattn_desc *desc);
 
 /*

@@ -36,7 +36,7 @@ def test_header_symbols_are_exported(lib):
     assert declared == set(_lib.EXPORTS)
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.convattn_version() == 100
+    assert lib.convattn_version() == 300
 
 
 def test_desc_layout_matches_header():

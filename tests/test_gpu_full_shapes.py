@@ -67,6 +67,40 @@ def test_c5_real_shape_heads_match_one_head_runs():
     torch.cuda.empty_cache()
 
 
+def test_c5_one_head_against_the_cpu_oracle():
+    # one head of the long-context workload (N = 16384) against the oracle's forward and autograd backward
+    # on the CPU (1 GB per N x N temporary), the GPU side run on that head alone (bit-equal to the head
+    # inside the full run: test above)
+    wl = synthetic.WORKLOADS["c5_long"]
+    t = synthetic.make_inputs(wl, seed=0)
+    h = 31
+    Qc, Kc, Vc, dOc = (t[k][:, h:h + 1].contiguous() for k in ("Q", "K", "V", "dO"))
+    Wc = t["W"][h:h + 1].contiguous()
+    O, M, L, dQ, dK, dV, dW = _fwd_bwd(*(x.to(DEV) for x in (Qc, Kc, Vc, dOc, Wc)), wl.scale, wl.pad_q, wl.pad_k)
+    O_ref, M_ref, L_ref = orc.forward_chunked(Qc.float(), Kc.float(), Vc.float(), Wc, True, wl.scale, rows=2048)
+    assert max_abs(O, O_ref) <= TOL_BF16
+    assert max_abs(M, M_ref) <= TOL_BF16 and rel_max(L, L_ref) <= TOL_BF16
+    ref = orc.backward_autograd(Qc.float(), Kc.float(), Vc.float(), Wc, dOc.float(), True, wl.scale)
+    errs = [max_abs(dQ, ref[0]), max_abs(dK, ref[1]), max_abs(dV, ref[2])]
+    print(f"C5 head {h} max-abs errors vs oracle: O {max_abs(O, O_ref):.4f} dQ {errs[0]:.4f} dK {errs[1]:.4f} "
+          f"dV {errs[2]:.4f} dW rel {rel_max(dW, ref[3]):.4f}")
+    assert max(errs) <= TOL_BF16
+    assert rel_max(dW, ref[3]) <= TOL_DW_REL
+
+
+def test_c2_one_pair_against_the_cpu_oracle():
+    # one (batch, head) pair of the forward-only workload (N = 2048, d = 64) inside the full run
+    wl = synthetic.WORKLOADS["c2_fwd"]
+    t = synthetic.make_inputs(wl, seed=0)
+    g = {k: v.to(DEV) for k, v in t.items()}
+    O, M, L = ops.forward(g["Q"], g["K"], g["V"], g["W"], wl.scale, wl.pad_q, wl.pad_k, True, out_dtype=torch.bfloat16)
+    for b, h in ((0, 0), (3, 15)):
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        O_ref, M_ref, L_ref = orc.forward(*(t[k][sl].float() for k in ("Q", "K", "V")), t["W"][h:h + 1], True, wl.scale)
+        assert max_abs(O[sl], O_ref) <= TOL_BF16
+        assert max_abs(M[sl], M_ref) <= TOL_BF16 and rel_max(L[sl], L_ref) <= TOL_BF16
+
+
 def test_c4_real_shape_decode():
     # B=32, H=32, Nk=8192: K and V are 2 GiB each (offsets beyond 2^31 bytes)
     wl = synthetic.WORKLOADS["c4_decode"]
@@ -171,6 +205,28 @@ def test_backward_falls_back_to_the_two_passes_when_the_workspace_is_capped(monk
     d_low = ops._desc(g[0], g[1], g[4], sc, True, torch.float32, low_memory=True)
     lib = _lib.load()
     assert lib.convattn_dw_partial_bytes(C.byref(d_low)) < lib.convattn_dw_partial_bytes(C.byref(d_fast)) // 8
+
+
+def test_dq_backward_falls_back_to_linear_scratch_when_the_workspace_is_capped(monkeypatch):
+    # the dQ + dW op alone (what the autograd function calls when only Q or the window needs a gradient):
+    # its fast path needs the O(N^2) dS scratch; above the cap it must run with O(N) scratch instead
+    Q, K, V, dO, W = rand_case(1, 2, 260, 260, 128, 6, 11, torch.bfloat16, seed=6)
+    ref = oracle_bwd(Q, K, V, W, dO, True)
+    g = [t.to(DEV) for t in (Q, K, V, dO, W)]
+    sc = scale_of(128)
+    O, M, L = ops.forward(g[0], g[1], g[2], g[4], sc, 5, 5, True, out_dtype=torch.bfloat16)
+    D, LSE = ops.bwd_preprocess(O, g[3], M, L)
+    fast = ops.dq_backward(g[0], g[1], g[2], g[3], D, LSE, g[4], sc, 5, 5, True, out_dtype=torch.float32)
+    monkeypatch.setenv("CONVATTN_MAX_WORKSPACE_BYTES", "1024")
+    asked = []
+    real_empty = torch.empty
+    monkeypatch.setattr(torch, "empty", lambda *a, **k: (asked.append(a[0]) or real_empty(*a, **k)))
+    dQ, dW = ops.dq_backward(g[0], g[1], g[2], g[3], D, LSE, g[4], sc, 5, 5, True, out_dtype=torch.float32)
+    monkeypatch.undo()
+    flat = [a for a in asked if isinstance(a, int)]
+    assert flat and max(flat) * 4 < 2 * 260 * 260 * 2      # no allocation the size of the dS matrix
+    assert max_abs(dQ, ref[0]) <= TOL_BF16 and rel_max(dW, ref[3]) <= TOL_DW_REL
+    assert max_abs(dQ, fast[0]) <= TOL_BF16 and rel_max(dW, fast[1]) <= TOL_DW_REL
 
 
 @pytest.mark.gpu

@@ -62,7 +62,9 @@ def test_backward(B, H, N, d, causal):
     ref = hc.backward_autograd(Q.float(), K.float(), V.float(), W, dO.float(), causal, sc)
     for name, got, want in zip(("dQ", "dK", "dV", "dW"), (dQ, dK, dV, dW), ref):
         assert got.dtype == torch.float32
-        tol = 2e-2 * max(1.0, float(want.abs().max()))   # D = rowsum(dO o O) is taken from the bf16 O
+        # observed 2e-3 .. 5e-3 of the gradient's scale (D = rowsum(dO o O) is taken from the bf16 O, the tile x
+        # input products round the tile to bf16): the bound leaves a factor of two, not ten
+        tol = 1e-2 * max(1.0, float(want.abs().max()))
         err = float((got.cpu() - want).abs().max())
         assert err <= tol, (name, err, tol)
 
@@ -86,7 +88,8 @@ def test_module_autograd():
     W = mod.head_conv_weights.detach().float().cpu()
     ref = hc.backward_autograd(Q.float(), K.float(), V.float(), W, dO.float(), True, None)
     for got, want in zip((q.grad, k.grad, v.grad, mod.head_conv_weights.grad), ref):
-        assert float((got.float().cpu() - want).abs().max()) <= 3e-2 * max(1.0, float(want.abs().max()))
+        # (bf16 module: the gradients themselves are rounded to bf16, 4e-3 of their scale)
+        assert float((got.float().cpu() - want).abs().max()) <= 1.5e-2 * max(1.0, float(want.abs().max()))
     out2 = head_conv_attention(q.detach(), k.detach(), v.detach(), mod.head_conv_weights.detach(), True, None)
     assert torch.equal(out2, out.detach())
 
