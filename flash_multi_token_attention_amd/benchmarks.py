@@ -22,8 +22,10 @@ scripts/plot_fwd_inference_speedup.py: decode time against the cache length) and
 head_conv_attn package; it ships no benchmark for it, its own check runs B=2, 16 heads, N=201, d=32,
 head_conv_attn/fwd_kernel.py:383-390).
 
-The reference's third line, its materialising PyTorch module, allocates [B,H,N,N] fp32
-temporaries and is not part of this package; it is timed on the CPU by ``bench.py``.
+The reference's third line, its materialising PyTorch module ([B,H,N,N] fp32 temporaries), is
+not part of this package: ``tests/bench_materialising.py`` times a restatement of it on the GPU
+and adds its two columns to a ``train`` table; ``plot`` then also draws the reference's own
+speed-up figure (fused module against materialising module) from them.
 """
 from __future__ import annotations
 
@@ -185,6 +187,24 @@ def plot(train_md: str, decode_md: str, out_dir: str) -> List[str]:
         plt.xscale("log", base=2); plt.xlabel("Sequence length"); plt.ylabel("SDPA time / conv-attention time")
         plt.title("Conv-attention against plain attention (MI355X)"); plt.grid(True, alpha=0.3); plt.legend(fontsize=7)
         save("benchmark_seq_len_speedup.png")
+        # 1b: the reference's published figure: its fused module against its materialising PyTorch module
+        # (columns added by tests/bench_materialising.py; rows without them are left out)
+        mat = {w: [r for r in per[w] if r.get("materialising fwd", "-") not in ("-", "")] for w in windows}
+        if any(mat.values()):
+            plt.figure(figsize=(10, 5))
+            for w in windows:
+                if not mat[w]:
+                    continue
+                n = [int(r["N"]) for r in mat[w]]
+                plt.plot(n, [float(r["materialising fwd"]) / float(r["conv fwd"]) for r in mat[w]], "o-", label=f"forward, {w}")
+                plt.plot(n, [float(r["materialising fwd+bwd"]) / float(r["conv fwd+bwd"]) for r in mat[w]], "s--",
+                         label=f"forward+backward, {w}")
+            plt.axhline(1.0, color="gray", linewidth=0.8)
+            plt.xscale("log", base=2); plt.yscale("log"); plt.xlabel("Sequence length")
+            plt.ylabel("materialising PyTorch time / fused time")
+            plt.title("Fused conv-attention against the materialising PyTorch module (MI355X)")
+            plt.grid(True, alpha=0.3); plt.legend(fontsize=7)
+            save("benchmark_seq_len_speedup_vs_materialising.png")
         # 2 and 3: absolute times
         for col, other, name, title in (("conv fwd", "sdpa fwd", "benchmark_seq_len_forward_times.png", "Forward"),
                                         ("conv fwd+bwd", "sdpa fwd+bwd", "benchmark_seq_len_backward_times.png", "Forward+backward")):
