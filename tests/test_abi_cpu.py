@@ -191,7 +191,11 @@ def test_benchmark_tables_parse_and_plot(tmp_path):
     assert len(rows) == len(benchmarks.TRAIN_SWEEP) and {"N", "window", "conv fwd", "sdpa fwd+bwd"} <= set(rows[0])
     assert all(float(r["conv fwd"]) > 0 for r in rows)
     files = benchmarks.plot(train, decode, str(tmp_path))
-    assert len(files) == 4 and all(os.path.getsize(f) > 10000 for f in files)
+    # speed-up against plain attention, speed-up against the materialising module (the reference's own
+    # figure; its columns come from tests/bench_materialising.py), forward times, backward times, decode
+    assert len(files) == 5 and all(os.path.getsize(f) > 10000 for f in files)
+    assert any(f.endswith("speedup_vs_materialising.png") for f in files)
+    assert float(rows[4]["materialising fwd+bwd"]) > float(rows[4]["conv fwd+bwd"])
 
 
 def test_kv_layout_rejected_before_launch(lib):
