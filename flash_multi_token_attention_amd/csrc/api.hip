@@ -127,7 +127,7 @@ const char *convattn_strerror(int code) {
         case CONVATTN_ERR_CAUSAL_SHAPE: return "causal conv-attention needs seq_len_q == seq_len_k";
         case CONVATTN_ERR_LDS: return "convolution window too large for the 160 KB of LDS at this head dimension";
         case CONVATTN_ERR_TOO_LARGE: return "batch or head count too large for one launch";
-        case CONVATTN_ERR_KV_LAYOUT: return "KV layout rejected: H must be a multiple of H_kv, page_size a power of two >= 16, strides multiples of 8 that cover a page / a sequence, the block table long enough, and the descriptor one of the streaming decode kernel (bf16, d 64 or 128, c_k <= 17)";
+        case CONVATTN_ERR_KV_LAYOUT: return "KV layout rejected: H must be a multiple of H_kv, page_size a power of two >= 16, strides multiples of 8 that cover a page / a sequence, the block table long enough, and the descriptor one of the streaming decode kernel (bf16, d 32, 64 or 128, c_k <= 17)";
         case CONVATTN_ERR_HEADMIX: return "head-mixing attention: n_heads must be 16 or 32, d_model 32, 64 or 128, inputs bf16";
         case CONVATTN_ERR_SCRATCH: return "the split partials of this decode step do not fit the library's built-in scratch (convattn_decode_noalloc): use fewer splits or convattn_decode";
         default: break;

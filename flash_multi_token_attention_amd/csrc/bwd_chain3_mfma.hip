@@ -119,7 +119,7 @@ __device__ __forceinline__ void chain3_role(const CHAIN_CONST_AS ChainArgs *args
     // of 1 KB (KBT of Q, then KBT of dO; unit 2 ks + f = the 16 row pairs of one k-step and parity).
     typedef int i32x4 __attribute__((ext_vector_type(4)));
     constexpr int KBT = Lds::tile_bytes / 1024;
-    static_assert(KBT == 2 * KS && (2 * KBT) % (2 * NP) == 0, "whole units per loading wave");
+    static_assert(KBT == 2 * KS && ((2 * KBT) % (2 * NP) == 0 || 2 * KBT < 2 * NP), "whole units per loading wave");
     auto dma_rsrc = [&](const bf16_t *ptr) {
         const unsigned long long a = reinterpret_cast<unsigned long long>(ptr);
         return (i32x4){(int)(unsigned int)a, (int)(unsigned int)(a >> 32), p.Nq * D * 2, 0x00020000};
@@ -132,6 +132,7 @@ __device__ __forceinline__ void chain3_role(const CHAIN_CONST_AS ChainArgs *args
 #pragma unroll
             for (int j0 = 0; j0 < 2 * KBT; j0 += 2 * NP) {
                 const int j = j0 + wave - NP, m = j / KBT, kb = j - m * KBT;
+                if (j >= 2 * KBT) break;   // (head dimension 32: four units for eight waves)
                 const int row = 2 * (ln >> 2) + (kb & 1), chunk = (kb >> 1) * 4 + ((ln & 3) ^ ((ln >> 4) & 3));
                 const int voff = ((r_begin + t * BR + row) * D + chunk * 8) * 2;
                 const unsigned int dst = lds0 + (m ? Lds::g_off + (t % 3) * Lds::tile_bytes : Lds::q_off + (t & 3) * Lds::tile_bytes) + kb * 1024;
@@ -843,6 +844,10 @@ hipError_t pick_shape(const Problem &p, int out_dt, const void *q, const void *k
     if (p.d == 128) {
         if (out_dt == CONVATTN_BF16) return pick_cq<128, bf16_t, WANT>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
         return pick_cq<128, float, WANT>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
+    }
+    if (p.d == 32) {
+        if (out_dt == CONVATTN_BF16) return pick_cq<32, bf16_t, WANT>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
+        return pick_cq<32, float, WANT>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
     }
     if (out_dt == CONVATTN_BF16) return pick_cq<64, bf16_t, WANT>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
     return pick_cq<64, float, WANT>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);

@@ -192,6 +192,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
 #pragma unroll
         for (int j0 = 0; j0 < 2 * KBT; j0 += 2 * NP) {
             const int j = j0 + wave, m = j / KBT, kb = j - m * KBT;
+            if (j >= 2 * KBT) break;   // (head dimension 32: four units for eight waves)
             const int row = 2 * (ln >> 2) + (kb & 1), chunk = (kb >> 1) * 4 + ((ln & 3) ^ ((ln >> 4) & 3));
             const int voff = ((r_begin + t * BR + row) * D + chunk * 8) * 2;
             const unsigned int dst = lds0 + (m ? Lds::g_off + (t % 3) * Lds::tile_bytes : Lds::q_off + (t & 3) * Lds::tile_bytes) + kb * 1024;
@@ -207,7 +208,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
         if (younger) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(NDB * 2) : "memory");
         else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     };
-    static_assert((2 * KBT) % (2 * NP) == 0, "whole units per wave");
+    static_assert((2 * KBT) % (2 * NP) == 0 || 2 * KBT < 2 * NP, "whole units per wave");
     // LSE and D of a tile: loaded by 32 threads one iteration before they are written to LDS.  STAT_ROLE: the
     // role whose wave does it (its first 32 lanes): the last consumer wave where it has the lightest
     // iteration (LIGHT), else the first producer wave.
@@ -968,6 +969,10 @@ hipError_t pick_shape(const Problem &p, int out_dt, const void *q, const void *k
     if (p.d == 128) {
         if (out_dt == CONVATTN_BF16) return pick_cq<128, bf16_t, WANT>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
         return pick_cq<128, float, WANT>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
+    }
+    if (p.d == 32) {
+        if (out_dt == CONVATTN_BF16) return pick_cq<32, bf16_t, WANT>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
+        return pick_cq<32, float, WANT>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
     }
     if (out_dt == CONVATTN_BF16) return pick_cq<64, bf16_t, WANT>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
     return pick_cq<64, float, WANT>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);

@@ -166,6 +166,10 @@ hipError_t mfma_dq_from_rows(const Problem &p, int out_dt, const void *k, const 
         if (out_dt == CONVATTN_BF16) return launch<128, bf16_t>(p, k, ds_ws, dc_scale, dq, s);
         return launch<128, float>(p, k, ds_ws, dc_scale, dq, s);
     }
+    if (p.d == 32) {
+        if (out_dt == CONVATTN_BF16) return launch<32, bf16_t>(p, k, ds_ws, dc_scale, dq, s);
+        return launch<32, float>(p, k, ds_ws, dc_scale, dq, s);
+    }
     if (out_dt == CONVATTN_BF16) return launch<64, bf16_t>(p, k, ds_ws, dc_scale, dq, s);
     return launch<64, float>(p, k, ds_ws, dc_scale, dq, s);
 }

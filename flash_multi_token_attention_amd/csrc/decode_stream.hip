@@ -345,7 +345,7 @@ __global__ __launch_bounds__(NW * 64) void decode_stream_kernel(
 }  // namespace
 
 bool decode_stream_ok(const Problem &p, int in_dt, unsigned flags) {
-    return in_dt == CONVATTN_BF16 && !(flags & CONVATTN_FLAG_EXACT) && (p.d == 64 || p.d == 128) &&
+    return in_dt == CONVATTN_BF16 && !(flags & CONVATTN_FLAG_EXACT) && (p.d == 32 || p.d == 64 || p.d == 128) &&
            p.pk <= 8 && p.c_q <= 16;
 }
 
@@ -372,6 +372,9 @@ hipError_t decode_stream_kv(const Problem &p, const KvArgs &kv, const void *q, c
     if (p.d == 128) {
         if (kv.table) CONVATTN_DECODE_PICK_HG(128, true);
         else CONVATTN_DECODE_PICK_HG(128, false);
+    } else if (p.d == 32) {
+        if (kv.table) CONVATTN_DECODE_PICK_HG(32, true);
+        else CONVATTN_DECODE_PICK_HG(32, false);
     } else {
         if (kv.table) CONVATTN_DECODE_PICK_HG(64, true);
         else CONVATTN_DECODE_PICK_HG(64, false);

@@ -184,8 +184,10 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
     // padding asks for.
     // A tile is 2 KS units of 1 KB (unit 2 ks + blk = rows 16 blk .. 16 blk + 15 of k-step ks); wave w
     // issues the units w, w + NW, ...  Lane l of a load fills chunk position l % 4 of row l / 4.
-    constexpr int UNITS = Lds::k_bytes / 1024, N_LD = UNITS / NW;
-    static_assert(UNITS == 2 * KS && UNITS % NW == 0 && NW == 4, "whole units per wave");
+    // (head dimension 32: two units, issued by the waves 0 and 1)
+    constexpr int UNITS = Lds::k_bytes / 1024, N_LD = UNITS >= NW ? UNITS / NW : 1;
+    static_assert(UNITS == 2 * KS && (UNITS % NW == 0 || UNITS < NW) && NW == 4, "whole units per wave");
+    const bool dma_wave = UNITS >= NW || wave < UNITS;
     // (K rows are read as row fragments, 16 rows of one chunk column at a time: swizzle value row / 4 mod 4;
     // V rows through transpose reads, 8 rows x 32 bytes per half wave: the same value with its two bits
     // swapped, so that rows r and r + 4 use different halves of their 64 bytes)
@@ -218,7 +220,7 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
     auto fetch_step = [&](int u) {
         const unsigned int Ks = lds_base + (u % Lds::n_buf) * Lds::buf_bytes, Vs = Ks + Lds::k_bytes;
         const int k0 = (32 * u - 8) * KST, v0 = (32 * u - 16) * KST;
-        static_for<N_LD>([&](auto I) {
+        if (dma_wave) static_for<N_LD>([&](auto I) {
             if (u == 0) {
                 dma16(k_dma, Ks, dma_off + k0, 0, I);
                 dma16(v_dma, Vs, dma_off_v + v0, 0, I);
@@ -532,6 +534,10 @@ hipError_t mfma_fwd(const Problem &p, int out_dt, const void *q, const void *k, 
     if (p.d == 128) {
         if (out_dt == CONVATTN_BF16) return pick_cq<128, bf16_t>(p, q, k, v, w, o, m, l, s);
         return pick_cq<128, float>(p, q, k, v, w, o, m, l, s);
+    }
+    if (p.d == 32) {
+        if (out_dt == CONVATTN_BF16) return pick_cq<32, bf16_t>(p, q, k, v, w, o, m, l, s);
+        return pick_cq<32, float>(p, q, k, v, w, o, m, l, s);
     }
     if (out_dt == CONVATTN_BF16) return pick_cq<64, bf16_t>(p, q, k, v, w, o, m, l, s);
     return pick_cq<64, float>(p, q, k, v, w, o, m, l, s);

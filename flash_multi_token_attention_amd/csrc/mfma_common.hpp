@@ -174,7 +174,7 @@ __device__ __forceinline__ u32x4 load_row16(const bf16_t *__restrict__ base, int
 
 // fp32-arithmetic fallbacks are chosen when this is false.
 inline bool mfma_shape_ok(const Problem &p, int in_dt, unsigned flags) {
-    return in_dt == CONVATTN_BF16 && !(flags & CONVATTN_FLAG_EXACT) && (p.d == 64 || p.d == 128) &&
+    return in_dt == CONVATTN_BF16 && !(flags & CONVATTN_FLAG_EXACT) && (p.d == 32 || p.d == 64 || p.d == 128) &&
            p.pk <= kMfmaMaxPk && p.c_q <= 11;
 }
 // The forward addresses K and V of one (batch, head) through buffer descriptors, which count
@@ -189,7 +189,10 @@ inline bool mfma_fwd_shape_ok(const Problem &p, int in_dt, unsigned flags) {
 // The backward kernels put the key taps on one 16-wide MFMA dimension.
 inline bool mfma_bwd_shape_ok(const Problem &p, int in_dt, unsigned flags) {
     // (the one-pass kernel addresses Q and dO of one (batch, head) with 32-bit byte offsets)
-    return mfma_shape_ok(p, in_dt, flags) && p.c_k <= 15 && (size_t)p.Nq * p.d * 2 < (1ull << 31) &&
+    // (head dimension 32: the key-stationary kernels only, i.e. windows of up to 8 query taps and not the
+    // low-memory dQ pass)
+    const bool d32_ok = p.d != 32 || (p.c_q <= 8 && (long long)p.B * p.H <= 65535 && !(flags & CONVATTN_FLAG_LOW_MEMORY));
+    return mfma_shape_ok(p, in_dt, flags) && d32_ok && p.c_k <= 15 && (size_t)p.Nq * p.d * 2 < (1ull << 31) &&
            ((long long)p.Nq + 16 + 127) / 128 <= kMaxGridZ && ((long long)p.Nk + 8 + 127) / 128 <= kMaxGridZ;
 }
 

@@ -242,7 +242,7 @@ int convattn_decode_strided(const convattn_desc *desc, const void *q, const void
  *   seq_lens      optional device int32 [B]: number of keys of every batch entry (1 .. desc->Nk); NULL =
  *                 desc->Nk for all.  desc->Nk is the longest sequence; splits cut every sequence evenly.
  * Strides are multiples of 8 elements.  Only descriptors that run the streaming decode kernel are
- * accepted (bf16 K and V, d 64 or 128, c_k <= 17: convattn_kernel_path(desc, CONVATTN_OP_DECODE) == 1).
+ * accepted (bf16 K and V, d 32, 64 or 128, c_k <= 17: convattn_kernel_path(desc, CONVATTN_OP_DECODE) == 1).
  */
 typedef struct convattn_kv_layout {
     int32_t H_kv;

@@ -24,6 +24,10 @@ FWD_SHAPES = [
     (1, 1, 130, 128, 6, 17),
     (1, 2, 31, 64, 2, 3),
     (1, 1, 1, 64, 6, 11),
+    # head dimension 32 (the reference dispatches 32, 64 and 128: kernels/fwd_wrapper.cu:69-95)
+    (2, 2, 300, 32, 6, 11),
+    (1, 2, 161, 32, 3, 3),
+    (1, 1, 200, 32, 11, 11),
 ]
 
 
@@ -87,6 +91,10 @@ BWD_SHAPES = [
     (1, 1, 130, 128, 6, 15),
     (1, 2, 31, 64, 2, 3),
     (1, 1, 1, 64, 6, 11),
+    # head dimension 32: windows of up to 8 query taps run the key-stationary kernels
+    (2, 2, 300, 32, 6, 11),
+    (1, 2, 161, 32, 3, 3),
+    (1, 1, 200, 32, 8, 9),
 ]
 
 
@@ -197,6 +205,8 @@ def test_module_autograd_matches_oracle_autograd():
     (3, 1000, 128, 3, 5, 7),
     (6, 64, 64, 6, 11, 64),
     (6, 130, 128, 16, 17, 2),
+    (16, 240, 32, 5, 5, 4),      # the reference's own decode test (scripts/test_fwd_inference_conv_attn.py:31-56)
+    (6, 1000, 32, 6, 11, 2),
 ])
 @pytest.mark.parametrize("causal", [False, True])
 def test_decode_bf16_stream(r, Nk, d, c_q, c_k, splits, causal):
