@@ -6,20 +6,9 @@
 #include <mutex>
 
 #include "common.hpp"
-#include <stdlib.h>
-
 #include "mfma_common.hpp"
 
 using namespace convattn;
-
-// CONVATTN_CHAIN3=0 in the environment selects the two-waves-per-SIMD backward (development switch)
-bool convattn::chain3_enabled() {
-    static const bool on = [] {
-        const char *e = getenv("CONVATTN_CHAIN3");
-        return !(e && e[0] == '0');
-    }();
-    return on;
-}
 
 namespace {
 

@@ -1,4 +1,7 @@
-// Whole backward of conv-attention on bf16 MFMA (gfx950): the score chain stays in registers.
+// Whole backward of conv-attention on bf16 MFMA (gfx950), windows of 7 and 8 query taps: the score chain
+// stays in registers.  (Windows of up to 6 query taps run the three-role kernel of bwd_chain3_mfma.hip,
+// which shares this file's building blocks through chain_common.hpp; the per-(batch, head) dC scale
+// kernels of both live here.)
 //
 // Key-stationary: a workgroup of 8 waves owns 128 keys of one (batch, head) and walks down the
 // query rows in tiles of 32.  Pair p (waves p and p+4, one SIMD) owns keys c0 = k0 + 32p .. c0+31
@@ -17,11 +20,8 @@
 // One workgroup barrier per tile; Q and dO tiles go from global memory straight into LDS (buffer
 // loads with the LDS modifier, one tile ahead), in a layout that serves both the 128-bit row
 // fragment reads of the producers and the 64-bit transpose reads of dV / dK (see ChainLds).
-// The transposed convolution of a pair's 32 keys needs dC on the 16 keys after them as well: that
-// block is the first block of the next pair, so (windows of up to 6 query taps) only the last pair
-// of a workgroup computes it itself and the other consumers read it from the next pair's stage;
-// the last pair's consumer, which shares its SIMD with that heavier producer, leaves dW to the
-// other three consumers and stages the LSE / D values of the tiles instead.
+// The transposed convolution of a pair's 32 keys needs dC on the 16 keys after them as well: every
+// pair computes that block itself.
 //
 // dW[a][b] = sum_i sum_j dC[i][j] S_m[i+a-pq][j+b-pk] is computed as G_a = dC^T S(rows shifted by
 // a), a [key j] x [key j'] product contracted over the rows on the matrix cores; only its
@@ -43,52 +43,12 @@ using namespace chain;
 
 
 constexpr int NT = 2 * NP * 64;  // 512 threads
-#ifndef CHAIN_PF
-#define CHAIN_PF 3
-#endif
-#ifndef CHAIN_PRIO_P
-#define CHAIN_PRIO_P 1
-#endif
-#ifndef CHAIN_PRIO_C
-#define CHAIN_PRIO_C 1
-#endif
-#ifndef CHAIN_PRIO_TC
-#define CHAIN_PRIO_TC 2
-#endif
-#ifndef CHAIN_PRIO_CEND
-#define CHAIN_PRIO_CEND 0
-#endif
-#ifndef CHAIN_ABLATE
-#define CHAIN_ABLATE 0
-#endif
-#ifdef CHAIN_PHASE_BARRIERS
-#define CHAIN_SCHED_BARRIER __builtin_amdgcn_sched_barrier(0)
-#else
-#define CHAIN_SCHED_BARRIER
-#endif
-
 #if !defined(CONVATTN_CHAIN_UNIT) || CONVATTN_CHAIN_UNIT == 3
 #define CONVATTN_CHAIN_UNIT_IS_ALL 1
 #else
 #define CONVATTN_CHAIN_UNIT_IS_ALL 0
 #endif
-
-#ifdef CHAIN_TS
-__device__ long long g_chain_ts[8][64][12];
-#define TS(i)                                                                                     \
-    do {                                                                                          \
-        if (lane == 0 && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == CHAIN_TS && it < 64) \
-            g_chain_ts[wave][it][i] = clock64();                                                  \
-    } while (0)
-#define TSX(a, b)                                                                          \
-    do {                                                                                   \
-        if (lane == 0 && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == CHAIN_TS)     \
-            g_chain_ts[wave][a][b] = clock64();                                            \
-    } while (0)
-#else
-#define TS(i)
-#define TSX(a, b)
-#endif
+constexpr int kPF = 3;   // dO^T / Q^T fragments read ahead of their MFMAs in the dV / dK phases
 
 // One role of the workgroup (ROLE 0 = producer waves, 1 = consumer waves).  The two roles have
 // disjoint register sets of 256 each and are both inlined into the kernel: as called functions
@@ -122,14 +82,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
     const int g = lane >> 4, n = lane & 15;
     constexpr bool producer = ROLE == 0;
     constexpr bool WANT_KV = (WANT & 1) != 0, WANT_QW = (WANT & 2) != 0;
-    // LIGHT: only the last pair's producer computes the C / dP / dC block after its own keys (the others'
-    // consumers read it from the next pair's stage); its consumer in turn takes no part in dW, which the
-    // other three share (2 CQT (pair group, tap slot) units, a multiple of 6).  The instance with 8 tap
-    // slots has no registers for a third of the units per wave: there every pair computes its own block.
-    constexpr bool LIGHT = CQT <= 6;
-    static_assert(!LIGHT || (2 * CQT) % 6 == 0, "whole dW units per wave and half");
     const int pr = wave & (NP - 1);
-    TSX(0, 10);
 
     auto q_slot = [&](int t) { return smem + Lds::q_off + (t & 3) * Lds::tile_bytes; };
     auto g_slot = [&](int t) { return smem + Lds::g_off + (t % 3) * Lds::tile_bytes; };
@@ -187,7 +140,6 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
     const i32x4 q_dma = dma_rsrc(Qb), g_dma = dma_rsrc(dOb);
     const unsigned int lds0 = (unsigned int)(unsigned long long)(__attribute__((address_space(3))) unsigned char *)smem;
     auto fetch_tile = [&](int t) {
-        if (CHAIN_ABLATE & 256) return;
         const int ln = (int)opaque((unsigned int)lane);
 #pragma unroll
         for (int j0 = 0; j0 < 2 * KBT; j0 += 2 * NP) {
@@ -209,14 +161,13 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
         else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     };
     static_assert((2 * KBT) % (2 * NP) == 0 || 2 * KBT < 2 * NP, "whole units per wave");
-    // LSE and D of a tile: loaded by 32 threads one iteration before they are written to LDS.  STAT_ROLE: the
-    // role whose wave does it (its first 32 lanes): the last consumer wave where it has the lightest
-    // iteration (LIGHT), else the first producer wave.
-    constexpr bool STAT_ROLE = (ROLE == 1) == LIGHT;
+    // LSE and D of a tile: loaded by the first 32 lanes of the first producer wave one iteration before they
+    // are written to LDS.
+    constexpr bool STAT_ROLE = ROLE == 0;
     // (a wave-uniform test, i.e. a branch: the other waves of the role must not even touch `ls` / `dd`, whose
     // reuse as load destinations makes the compiler wait for every outstanding vector memory operation of the
     // wave, the dS stores of the last iteration among them)
-    const bool stat_wave = STAT_ROLE && wave == (LIGHT ? 2 * NP - 1 : 0);
+    const bool stat_wave = STAT_ROLE && wave == 0;
     float ls = 0.f, dd = 0.f;
     auto load_stats = [&](int r0) {
         if constexpr (STAT_ROLE) {
@@ -292,13 +243,10 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
         stage_stats(0);
         load_stats(r_begin + BR);
 
-        // The C / dP / dC block after a pair's own keys (keys c0+24 .. c0+39) is the first block of the next
-        // pair, whose producer computes it anyway: only the last pair of the workgroup (HEAVY) computes it
-        // itself, and with it the fourth S^T block; the consumers of the other pairs read that block from
-        // the next pair's stage.
-        auto producer_loop = [&](auto heavy_tag) {
-        constexpr bool HEAVY = decltype(heavy_tag)::value;
-        constexpr int PNSB = HEAVY ? NSB : NSB - 1, PNCB = HEAVY ? NCB : NCB - 1;
+        // Every pair computes the C / dP / dC block after its own keys (keys c0+24 .. c0+39) itself, and with it
+        // the fourth S^T block.
+        {
+        constexpr int PNSB = NSB, PNCB = NCB;
         // packed fp16 scores of the previous tile: [block][fragment][dword]
         unsigned int prev_pd[NSB][2][2];
 
@@ -311,7 +259,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
 #pragma unroll
                 for (int f = 0; f < 2; ++f) acc[kb][f] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int ks = 0; ks < ((CHAIN_ABLATE & 64) ? 0 : KS); ++ks) {
+            for (int ks = 0; ks < KS; ++ks) {
                 bf16x8 qf[2];
 #pragma unroll
                 for (int f = 0; f < 2; ++f) qf[f] = load_qf(f, ks);
@@ -350,19 +298,14 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
         {
             s_phase(r_begin - BR, 0, prev_pd, std::true_type{}, [&](int f, int ks) { return q_above[f][ks]; });
         }
-
-        TSX(0, 11);
         for (int it = 0; it <= n_tiles + 1; ++it) {
             const int r0 = r_begin + it * BR;
-            TS(0);
             tiles_landed(false);
             __syncthreads();
-            TS(1);
             // (the LSE / D loads before the tile loads: the wait above is for the youngest loads of the wave)
             if (it + 1 < n_tiles) stage_stats(it + 1);
             load_stats(r0 + 2 * BR);
             if (it + 1 < n_tiles) fetch_tile(it + 1);
-            TS(2);
             // dC of a tile that has none (entirely above the diagonal, or the one after the last):
             // zeros, so that the consumers read every tile alike
             auto zero_dc = [&] {
@@ -377,9 +320,6 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
             };
             if (it == n_tiles) zero_dc();
             if (it >= n_tiles) continue;
-#if defined(CHAIN_SKIP_ROLE) && CHAIN_SKIP_ROLE == 0
-            continue;
-#endif
 
             auto ptile = [&](auto edge_tag, auto full_tag) {
                 constexpr bool EDGE = decltype(edge_tag)::value;
@@ -387,21 +327,16 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                 // row fragments: lane n of fragment f reads row 2n + f, 16 bytes at column 32 ks + 8 g
                 const unsigned char *Qs = smem + opaque((unsigned int)(q_slot(it) - smem) + row_frag_off());
                 const unsigned char *Gs = smem + opaque((unsigned int)(g_slot(it) - smem) + row_frag_off());
-                // (with the light producers the consumers are the longer role: they get the issue slot first)
-                if constexpr (LIGHT) __builtin_amdgcn_s_setprio(0);
-                else __builtin_amdgcn_s_setprio(CHAIN_PRIO_P);
+                __builtin_amdgcn_s_setprio(1);
                 f32x4 dp[NCB][2];
                 float2 l2 = {0.f, 0.f};
                 if constexpr (FULL) l2 = *reinterpret_cast<const float2 *>(stat_slot(it) + 2 * n);
-                TS(4);
                 // ---- S^T ----
                 unsigned int pd[NSB][2][2];
                 s_phase(r0, it + 1, pd, edge_tag, [&](int f, int ks) {
                     return *reinterpret_cast<const bf16x8 *>(Qs + f * 1024 + ks * 2048);
                 });
-                CHAIN_SCHED_BARRIER;
-                TS(3);
-                if constexpr (FULL) {
+                                if constexpr (FULL) {
                     unsigned char *Cs = c_stage(it), *Ps = p_stage(it);
                     // ---- convolution: C^T block cb from score blocks cb (k slots 0..3 of a lane
                     // group) and cb+1 (4..7).  Operand of row offset delta = DL - (CQT-1): fragment
@@ -414,7 +349,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                         c[cb][1] = (f32x4){-l2.y, -l2.y, -l2.y, -l2.y};
                     }
                     f16x8 tf_prev = (f16x8)(_Float16)0.f;
-                    static_for<(CHAIN_ABLATE & 16) ? 0 : CQT + 1>([&](auto DL) {
+                    static_for<CQT + 1>([&](auto DL) {
                         constexpr int t0 = decltype(DL)::value;
                         constexpr int delta = t0 - (CQT - 1);
                         constexpr int f = delta & 1, s = (f - delta) / 2;
@@ -439,7 +374,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                         for (int f = 0; f < 2; ++f) { prev_pd[kb][f][0] = pd[kb][f][0]; prev_pd[kb][f][1] = pd[kb][f][1]; }
                     // ---- dP^T = V dO^T - D, after the convolution: the shifted score windows are no
                     // longer live then (with dP first, some instances of the kernel needed scratch) ----
-                    if constexpr (!(CHAIN_ABLATE & 32)) {
+                    {
                         const float2 d2 = *reinterpret_cast<const float2 *>(stat_slot(it) + BR + 2 * n);
 #pragma unroll
                         for (int cb = 0; cb < PNCB; ++cb) {
@@ -458,10 +393,8 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                                 for (int f = 0; f < 2; ++f) dp[cb][f] = mfma_bf16(vf[cb][ks], gf[f], dp[cb][f]);
                         }
                     }
-                    CHAIN_SCHED_BARRIER;
-                    TS(5);
-                    // ---- P = exp2(C - LSE) (times the dC scale), dC = P dP ----
-                    static_for<(CHAIN_ABLATE & 128) ? 0 : PNCB>([&](auto CB) {
+                                        // ---- P = exp2(C - LSE) (times the dC scale), dC = P dP ----
+                    static_for<PNCB>([&](auto CB) {
                         constexpr int cb = decltype(CB)::value;
                         __builtin_amdgcn_s_setprio(0);
 #pragma unroll
@@ -501,12 +434,8 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
             if (is_skipped(r0)) ptile(std::true_type{}, std::false_type{});
             else if (is_edge(r0)) ptile(std::true_type{}, std::true_type{});
             else ptile(std::false_type{}, std::true_type{});
-            TS(6);
         }
-        };
-        if (!LIGHT || pr == NP - 1) producer_loop(std::true_type{});
-        else producer_loop(std::false_type{});
-        TSX(1, 10);
+        }
         __syncthreads();  // the consumers' barrier before they hand over their dW accumulators
         __syncthreads();  // ... and the one after it
         // ---- dW partial of this workgroup: G[m][n] of half x belongs to key tap b = n - m + 16 x - 8 + pk;
@@ -540,19 +469,12 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
             *reinterpret_cast<f16x8 *>(bands + t * 1024) = band_frag<CQT>(t, w_head, cq, ck, pk, g, n, true, p.scale);
         stage_stats(0);
         load_stats(r_begin + BR);
-        // dW: a unit is the key blocks of two pairs (pair group) times one tap slot.  LIGHT: the waves 0 .. 2 take
-        // 2 CQT / 3 consecutive units each, in two passes of NU units of one pair group; otherwise every wave
-        // takes one pair group and half of the tap slots in one pass.
-        constexpr int NU = LIGHT ? CQT / 3 : (CQT + 1) / 2;   // units per pass
-        constexpr int NPASS = LIGHT ? 2 : 1, TH = NU * NPASS;
-        int dw_pg[NPASS], dw_t[NPASS];                         // pair group and first tap slot of each pass
-#pragma unroll
-        for (int ps = 0; ps < NPASS; ++ps) {
-            const int q = LIGHT ? pr * TH + ps * NU : 0;
-            dw_pg[ps] = LIGHT ? q / CQT : pr >> 1;
-            dw_t[ps] = LIGHT ? q - dw_pg[ps] * CQT : (pr & 1) * NU;
-        }
-        const bool dw_wave = !LIGHT || pr < NP - 1;
+        // dW: a unit is the key blocks of two pairs (pair group) times one tap slot; every wave takes one pair
+        // group and half of the tap slots, in one pass.
+        constexpr int NU = (CQT + 1) / 2;   // units per pass
+        constexpr int NPASS = 1, TH = NU * NPASS;
+        const int dw_pg[NPASS] = {pr >> 1}, dw_t[NPASS] = {(pr & 1) * NU};   // pair group and first tap slot
+        constexpr bool dw_wave = true;
         f32x4 acc_k[NDB][DB], acc_v[2][DB];
 #pragma unroll
         for (int m = 0; m < 2; ++m)
@@ -571,25 +493,17 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
             for (int f = 0; f < 2; ++f) prev_dc[cb][f][0] = prev_dc[cb][f][1] = 0u;
         const int n_kt = gridDim.z * NP, kt = blockIdx.z * NP + pr;
         bf16_t *ds_pair = dS_ws + (bh * n_kt + kt) * (size_t)n_rt * (WK * BR);
-
-        TSX(0, 11);
         bool ds_stored = false;  // the last iteration stored a dS block (after its tile loads)
         for (int it = 0; it <= n_tiles + 1; ++it) {
-            TS(0);
             tiles_landed(ds_stored);
             ds_stored = false;
             __syncthreads();
-            TS(1);
             // (the LSE / D loads before the tile loads: the counted wait above relies on that order)
             if (it + 1 < n_tiles) stage_stats(it + 1);
             load_stats(r_begin + (it + 2) * BR);
             if (it + 1 < n_tiles) fetch_tile(it + 1);
-            TS(2);
             const int u = it - 1, v = it - 2;
             const int r0u = r_begin + u * BR, r0v = r_begin + v * BR;
-#if defined(CHAIN_SKIP_ROLE) && CHAIN_SKIP_ROLE == 1
-            continue;
-#endif
             const bool u_in = it >= 1 && u < n_tiles;
             const bool u_ok = u_in && !is_skipped(r0u);
             const bool v_ok = it >= 2 && !is_skipped(r0v);
@@ -597,14 +511,14 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
             // Order of the iteration: dV (operands of the staged tiles only, so the first MFMAs
             // start while the dC loads are in flight), dS, dW (independent of dS: its MFMAs cover
             // the round trip of dS through LDS), dK.
-            if (WANT_KV && u_ok && !(CHAIN_ABLATE & 4)) {
+            if (WANT_KV && u_ok) {
                 const unsigned char *Ps = smem + opaque((unsigned int)(p_stage(u) - smem) + tr_lane_off(PST, g, n));
                 const unsigned char *Gs = smem + opaque((unsigned int)(g_slot(u) - smem) + tr_frag_off());
-                __builtin_amdgcn_s_setprio(CHAIN_PRIO_C);
+                __builtin_amdgcn_s_setprio(1);
                 // ---- dV^T += dO^T P (keys c0-8 .. c0+23) ----
                 // the dO^T fragment of head-dim block db + PF is read while block db is multiplied: the
                 // MFMAs of PF blocks cover the LDS latency
-                constexpr int PF = CHAIN_PF;
+                constexpr int PF = kPF;
                 bf16x8 pf[2], gq[PF + 1];
 #pragma unroll
                 for (int cb = 0; cb < 2; ++cb) pf[cb] = read_tr(Ps, PST, cb * 16);
@@ -621,17 +535,14 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                     SCHED_MFMA_ID(2, 60 + db);
                 });
             }
-            CHAIN_SCHED_BARRIER;
-            TS(3);
-            // packed dC^T of tile u, as the producer's lanes held it (zeros when the tile has none)
+                        // packed dC^T of tile u, as the producer's lanes held it (zeros when the tile has none)
             unsigned int cur_dc[NCB][2][2];
             {
                 // read unconditionally: the producer writes zeros for a tile without dC; what the first
                 // iteration reads (nothing written yet) is dropped before any use
                 const unsigned char *Cl = smem + opaque((unsigned int)(c_stage(max(u, 0)) - smem) + 2 * n * CST + 4 * g * 2);
-                // the block after the pair's own keys: the first block of the next pair's stage (the last
-                // pair's producer writes it to its own stage)
-                const unsigned char *Cn = Cl + ((!LIGHT || pr == NP - 1) ? 2 * 32 : Lds::pair_bytes);
+                // the block after the pair's own keys: the third block of the pair's own stage
+                const unsigned char *Cn = Cl + 2 * 32;
 #pragma unroll
                 for (int cb = 0; cb < NCB; ++cb)
 #pragma unroll
@@ -641,11 +552,10 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                         cur_dc[cb][f][1] = t2[1];
                     }
             }
-            TS(7);
-            if (v_ok && !(CHAIN_ABLATE & 512)) {
+            if (v_ok) {
                 const bool edge = is_edge(r0v);
                 bf16_t *ds_blk = ds_pair + (size_t)(r0v / BR) * (WK * BR);
-                __builtin_amdgcn_s_setprio(CHAIN_PRIO_TC);
+                __builtin_amdgcn_s_setprio(2);
                 // ---- dS^T of tile v: rows below it come from tile v+1.  Operand of row offset
                 // e = parity + (CQT-1 - tap slot): fragment e & 1 shifted e >> 1 lanes up. ----
                 f32x4 ds[NDB][2];
@@ -658,7 +568,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                 tbq[0] = band_of(0);
                 tbq[1] = band_of(CQT >= 2 ? 1 : 0);
                 tbq[2] = tbq[3] = tbq[0];
-                static_for<(CHAIN_ABLATE & 2) ? 0 : CQT + 1>([&](auto E) {
+                static_for<CQT + 1>([&](auto E) {
                     constexpr int e = decltype(E)::value, f = e & 1, s = e >> 1;
                     // tap slot CQT-1-e for parity 0 (this step's band), CQT-e for parity 1 (the last step's)
                     if constexpr (e + 2 <= CQT - 1) tbq[(e + 2) % 4] = band_of(e + 2);
@@ -675,7 +585,6 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                         if constexpr (e >= 1) ds[sb][1] = mfma_f16(tb_prev, __builtin_bit_cast(f16x8, bv), ds[sb][1]);
                     }
                 });
-                TS(8);
 #pragma unroll
                 for (int sb = 0; sb < NDB; ++sb)
 #pragma unroll
@@ -698,19 +607,16 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                         }
                         if constexpr (WANT_KV) *reinterpret_cast<bf16x4 *>(ds_tile + (2 * n + ob) * PST + (sb * 16 + 4 * g) * 2) = sv;
                     }
-                TS(9);
             }
 #pragma unroll
             for (int cb = 0; cb < NCB; ++cb)
 #pragma unroll
                 for (int f = 0; f < 2; ++f) { prev_dc[cb][f][0] = cur_dc[cb][f][0]; prev_dc[cb][f][1] = cur_dc[cb][f][1]; }
-            CHAIN_SCHED_BARRIER;
-            TS(4);
-            // ---- dW, key blocks jb = 0..3 of the pairs 2 pg and 2 pg + 1 (block jb = dC block jb & 1 of
+                        // ---- dW, key blocks jb = 0..3 of the pairs 2 pg and 2 pg + 1 (block jb = dC block jb & 1 of
             // pair 2 pg + jb / 2, keys k0 + 64 pg - 8 + 16 jb ..), tap slots t_lo .. t_lo + TH - 1:
             // G_t[j][j'] += sum_rows dC[row][j] S[row + t - (CQT-1)][j'] with j' in the score block
             // 8 keys before the dC block (x = 0) and the one 8 keys after it (x = 1) ----
-            if (WANT_QW && u_in && dw_wave && !(CHAIN_ABLATE & 1)) static_for<NPASS>([&](auto PS) {
+            if (WANT_QW && u_in && dw_wave) static_for<NPASS>([&](auto PS) {
                 constexpr int ps = decltype(PS)::value;
                 const int pg = dw_pg[ps], t_lo = dw_t[ps];
                 // Ring rows of this lane's two transpose reads at the wave's first tap slot: tile row 0
@@ -783,17 +689,15 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                     for (int tt = 0; tt < NU; ++tt) { b0[tt] = b1[tt]; b1[tt] = b2[tt]; }
                 });
             });
-            CHAIN_SCHED_BARRIER;
-            TS(5);
-            if (WANT_KV && v_ok && !(CHAIN_ABLATE & 8)) {
+                        if (WANT_KV && v_ok) {
                 const unsigned char *Qs = smem + opaque((unsigned int)(q_slot(v) - smem) + tr_frag_off());
                 const unsigned char *Dsl = smem + opaque((unsigned int)(ds_tile - smem) + tr_lane_off(PST, g, n));
                 asm volatile("" ::: "memory");
                 __builtin_amdgcn_wave_barrier();
-                __builtin_amdgcn_s_setprio(CHAIN_PRIO_C);
+                __builtin_amdgcn_s_setprio(1);
                 // ---- dK^T += Q^T dS ----
                 {
-                    constexpr int PF = CHAIN_PF;
+                    constexpr int PF = kPF;
                     bf16x8 sf[2], qq[PF + 1];
                     // (Q^T does not depend on the dS tile: its first fragments are on their way first)
 #pragma unroll
@@ -814,11 +718,8 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                 asm volatile("" ::: "memory");
                 __builtin_amdgcn_wave_barrier();
             }
-            __builtin_amdgcn_s_setprio(CHAIN_PRIO_CEND);
-            TS(6);
+            __builtin_amdgcn_s_setprio(0);
         }
-
-        TSX(1, 10);
         // ---- dW accumulators of this wave to LDS as [pair group][tap slot][x][m][n], once every
         // wave is done with the tiles ----
         __syncthreads();
@@ -870,8 +771,6 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
         }
 
     }  // consumer
-
-    TSX(1, 11);
 }
 
 template <int D, int CQT, typename TO, int WANT>
@@ -957,8 +856,7 @@ template <int D, typename TO, int WANT>
 hipError_t pick_cq(const Problem &p, const void *q, const void *k, const void *v, const void *d_o,
                    const float *Dl, const float *lse, const float *w, const float *dc_scale, void *dk, void *dv,
                    void *ds_ws, float *dw_part, hipStream_t s) {
-    if (p.c_q <= 3) return launch_chain<D, 3, TO, WANT>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
-    if (p.c_q <= 6) return launch_chain<D, 6, TO, WANT>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
+    // (windows of up to 6 query taps run the three-role kernel of bwd_chain3_mfma.hip)
     return launch_chain<D, 8, TO, WANT>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
 }
 
@@ -980,11 +878,6 @@ hipError_t pick_shape(const Problem &p, int out_dt, const void *q, const void *k
 
 }  // namespace
 
-#ifdef CHAIN_TS
-extern "C" int convattn_debug_chain_ts(long long *host) {
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_chain_ts), sizeof(long long) * 8 * 64 * 12);
-}
-#endif
 
 #if CONVATTN_CHAIN_UNIT_IS_ALL
 hipError_t mfma_dc_scale(const Problem &p, const void *d_o, const void *v, float *dc_scale, hipStream_t s) {

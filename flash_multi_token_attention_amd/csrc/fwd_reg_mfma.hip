@@ -53,29 +53,8 @@ constexpr float kMaxSlack = 6.f;  // log2 units a score may exceed its row's exp
 // window's halo, the other 33-CQT are its output rows.
 constexpr int wave_rows(int cqt) { return 33 - cqt; }
 
-#ifndef FWD_PFV
-#define FWD_PFV 2   // V^T fragments read ahead of their MFMAs in the P V phase
-#endif
-#ifdef FWD_TS
-__device__ long long g_fwd_ts[4][64][8];
-#define FTS(i)                                                                                     \
-    do {                                                                                           \
-        if (lane == 0 && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == FWD_TS && u < 64)     \
-            g_fwd_ts[wave][u][i] = clock64();                                                      \
-    } while (0)
-#define FTSX(a, b)                                                                        \
-    do {                                                                                  \
-        if (lane == 0 && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == FWD_TS)      \
-            g_fwd_ts[wave][a][b] = clock64();                                             \
-    } while (0)
-#else
-#define FTS(i)
-#define FTSX(a, b)
-#endif
-
-#ifndef FWD_NBUF
-#define FWD_NBUF 2   // LDS buffers: 2 = the rows of step u+1 arrive during step u (3: two steps ahead; measured: no faster)
-#endif
+constexpr int kFwdPfv = 2;    // V^T fragments read ahead of their MFMAs in the P V phase
+constexpr int kFwdNbuf = 2;   // LDS buffers: the rows of step u+1 arrive during step u (3, two steps ahead, measured no faster)
 template <int D> struct FwdLds {
     // K / V rows go from global memory straight into LDS (buffer loads with the LDS modifier: the
     // 64 lanes of a load fill 1 KB of consecutive LDS, which rules out padded rows).  A tile of 32
@@ -87,7 +66,7 @@ template <int D> struct FwdLds {
     static constexpr int KST = D * 2;              // bytes of a row in global memory
     static constexpr int k_bytes = BK * KST;
     static constexpr int buf_bytes = 2 * k_bytes;  // K rows, then V rows
-    static constexpr int n_buf = FWD_NBUF;         // steps u, u+1 (and u+2) resident or on their way
+    static constexpr int n_buf = kFwdNbuf;         // steps u, u+1 (and u+2) resident or on their way
     static constexpr int total = n_buf * buf_bytes;
 };
 
@@ -106,7 +85,6 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;  // wave-uniform for the compiler too
     const int g = lane >> 4, n = lane & 15;
-    FTSX(0, 6);
 
     // x = head, y = batch, z = query tile: the dispatcher hands out every (batch, head) of the
     // longest (causal) tiles first, so the tail of the launch is made of short tiles
@@ -319,10 +297,8 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
         for (int f = 0; f < 2; ++f)
 #pragma unroll
             for (int dw = 0; dw < 2; ++dw) carry[f][dw] = pd[1][f][dw];
-
-        FTS(3);
-        // V^T fragments of the first FWD_PFV head-dim blocks: in flight during the softmax
-        constexpr int PFV = FWD_PFV < DB ? FWD_PFV : DB;
+        // V^T fragments of the first kFwdPfv head-dim blocks: in flight during the softmax
+        constexpr int PFV = kFwdPfv < DB ? kFwdPfv : DB;
         bf16x8 vf[PFV + 1];
         auto load_vf = [&](int buf, int db) {
             bf16x4 lo = lds_tr64((lds_byte_ptr)(size_t)(va[db & 1] + (db >> 1) * 2048));
@@ -400,7 +376,6 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
         // ---- O^T += V^T P^T: V^T fragments through the LDS transpose read, P^T straight from
         //      the softmax registers (k slot 8g+e <-> key 4g+e of output block 0 for e < 4, of
         //      output block 1 for e >= 4) ----
-        FTS(4);
         __builtin_amdgcn_s_setprio(1);
         bf16x8 pf[2];
 #pragma unroll
@@ -420,7 +395,6 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
             for (int ob = 0; ob < 2; ++ob) acc_o[ob][db] = mfma_bf16(vf[db % (PFV + 1)], pf[ob], acc_o[ob][db]);
             SCHED_MFMA(2);
         }
-        FTS(5);
     };
 
     const int k_end = causal ? min(p.Nk, i0 + BQ) : p.Nk;
@@ -435,14 +409,11 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
         constexpr int KIND = decltype(kind)::value;
 #pragma unroll 1
         for (int u = ua; u < ub; ++u) {
-            FTS(0);
             // this wave's rows of step u have landed (with three buffers those of step u + 1 may be on their way)
             if constexpr (Lds::n_buf == 3) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * N_LD) : "memory");
             else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();  // step u-1 is done everywhere: its buffer is free, and step u's is written
-            FTS(1);
             fetch_step(u + Lds::n_buf - 1);
-            FTS(2);
             if constexpr (KIND != 2) step(u, std::integral_constant<bool, KIND == 1>{});
             const int to_other = (u % Lds::n_buf == Lds::n_buf - 1) ? -(Lds::n_buf - 1) * Lds::buf_bytes : Lds::buf_bytes;
             ka += to_other;
@@ -454,13 +425,10 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
     const int u_tail = p.Nk < 24 ? 1 : (p.Nk - 24) / 32 + 1;    // first u >= 1 with 32u + 24 > Nk
     const int u1 = min(causal ? min(u_diag, u_tail) : u_tail, n_steps);
     const int u2 = max(u1, causal ? min((i0w + WR + 15) / 32 + 1, n_steps) : n_steps);  // 32u - 16 > i0w + WR - 1
-    FTSX(0, 7);
     run(0, 1, std::integral_constant<int, 1>{});
     run(1, u1, std::integral_constant<int, 0>{});
     run(u1, u2, std::integral_constant<int, 1>{});
     run(u2, n_steps, std::integral_constant<int, 2>{});
-
-    FTSX(1, 6);
     // ---- epilogue: finish the row sums and maxima, normalise, store O, M, L ----
 #pragma unroll
     for (int ob = 0; ob < 2; ++ob) {
@@ -493,7 +461,6 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
             }
         }
     }
-    FTSX(1, 7);
 }
 
 template <int D, int CQT, typename TO>
@@ -523,11 +490,6 @@ hipError_t pick_cq(const Problem &p, const void *q, const void *k, const void *v
 
 }  // namespace
 
-#ifdef FWD_TS
-extern "C" int convattn_debug_fwd_ts(long long *host) {
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_fwd_ts), sizeof(long long) * 4 * 64 * 8);
-}
-#endif
 
 hipError_t mfma_fwd(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
                     const float *w, void *o, float *m, float *l, hipStream_t s) {

@@ -299,12 +299,11 @@ CHAIN_DECL(mfma_bwd_chain3_kv);
 CHAIN_DECL(mfma_bwd_chain3_qw);
 CHAIN_DECL(mfma_bwd_chain3_all);
 #undef CHAIN_DECL
-bool chain3_enabled();
 inline hipError_t mfma_bwd_chain(const Problem &p, int out_dt, int want, const void *q, const void *k, const void *v,
                                  const void *d_o, const float *Dl, const float *lse, const float *w,
                                  const float *dc_scale, void *dk, void *dv, void *ds_ws, float *dw_part,
                                  hipStream_t s) {
-    if (p.c_q <= 6 && chain3_enabled()) {
+    if (p.c_q <= 6) {
         if (want == 1) return mfma_bwd_chain3_kv(p, out_dt, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
         if (want == 2) return mfma_bwd_chain3_qw(p, out_dt, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
         return mfma_bwd_chain3_all(p, out_dt, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
