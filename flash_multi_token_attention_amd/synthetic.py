@@ -101,10 +101,11 @@ def executed_mfma_flops(wl: Workload, two_pass: bool = False) -> Dict[str, objec
     forward: a wave owns 33 - T output rows (T = 3 or 6 tap slots) of a 32-row score tile and walks
       the keys in 32-key steps up to its last row + 16: per step S^T 2 (row fragments) x 2 (key
       blocks) x d/32, convolution 4 T, P V 2 x d/16 MFMAs.
-    key-stationary backward: a wave pair owns 32 keys and walks 32-row tiles from the first row that
+    key-stationary backward: a wave triple owns 32 keys and walks 32-row tiles from the first row that
       sees its keys: per tile S^T 6 d/32 (48 keys for 32 owned), convolution 4 T (32 keys), dP 4 d/32,
-      transposed convolution 4 T, dV and dK 2 d/16 each, dW 4 T MFMAs; the last of a workgroup's four
-      pairs also computes the 16 keys after its own (S^T 8 d/32, convolution 6 T, dP 6 d/32).
+      transposed convolution 4 T, dV and dK 2 d/16 each, dW 4 T MFMAs; for the last of a workgroup's
+      four triples a second score chain computes the 16 keys after its own (S^T 4 d/32 for the two
+      16-key blocks around them, convolution 2 T, dP 2 d/32).
     dQ = dS K: 2 x d/16 per 32 rows x 32 keys below the diagonal (nothing wasted but the diagonal
       blocks' upper halves).
     """
@@ -118,7 +119,9 @@ def executed_mfma_flops(wl: Workload, two_pass: bool = False) -> Dict[str, objec
         steps = min((w0 + rows + 15) // 32 + 1, (wg_end + 16 + 31) // 32)
         fwd += steps * (4 * d // 32 + 4 * T + 2 * d // 16)
     consumer = 4 * T + 4 * d // 16 + 4 * T             # transposed convolution, dV and dK, dW
-    light, heavy = 6 * d // 32 + 4 * T + 4 * d // 32, 8 * d // 32 + 6 * T + 6 * d // 32
+    light = 6 * d // 32 + 4 * T + 4 * d // 32
+    extra = 4 * d // 32 + 2 * T + 2 * d // 32           # the score chain of the block after the workgroup's keys
+    heavy = light + extra
     full = kv = qw = s_only = 0
     for c0 in range(0, (N + 8 + 127) // 128 * 128, 32):   # one wave pair per 32 keys
         k0 = c0 // 128 * 128
@@ -130,7 +133,7 @@ def executed_mfma_flops(wl: Workload, two_pass: bool = False) -> Dict[str, objec
         full += (n_t - skipped) * (producer + consumer)
         kv += (n_t - skipped) * (producer + consumer - 4 * T)          # dK / dV pass: no dW
         qw += (n_t - skipped) * (producer + consumer - 4 * d // 16)    # dQ + dW pass: no dV, dK
-        s_only += (skipped + 1) * (8 if last else 6) * d // 32         # + the 32 rows above the first tile
+        s_only += (skipped + 1) * (10 if last else 6) * d // 32        # + the 32 rows above the first tile
     dq = sum((min(N, (r // 128 + 1) * 128) + 63) // 64 * 2 for r in range(0, N, 32)) * 2 * d // 16
     out = {"fwd": fwd * mf * bh}
     if wl.backward:
