@@ -149,6 +149,8 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
             const int voff = ((r_begin + t * BR + row) * D + chunk * 8) * 2;
             const unsigned int dst = lds0 + (m ? Lds::g_off + (t % 3) * Lds::tile_bytes : Lds::q_off + (t & 3) * Lds::tile_bytes) + kb * 1024;
             const i32x4 rsrc = m ? g_dma : q_dma;
+            // (M0 is written here and read by the load that follows; nothing else of this kernel uses it,
+            // and it is not declared clobbered: the compiler keeps no value in M0 across an asm statement)
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                          :: "s"(dst), "v"(voff), "s"(rsrc) : "memory");
         }
@@ -156,6 +158,8 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
     // Every tile this wave has asked for is in LDS (to be followed by the workgroup barrier).  Vector
     // memory operations complete in the order of their issue: `younger` = the global stores the wave
     // has issued since the tile loads (the dS block of an iteration: NDB * 2), which need not be waited for.
+    // The count holds only while a wave issues exactly those stores, and no other vector memory operation,
+    // between its loads and this wait: the statistics loads are issued before the tile loads.
     auto tiles_landed = [&](bool younger) {
         if (younger) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(NDB * 2) : "memory");
         else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");

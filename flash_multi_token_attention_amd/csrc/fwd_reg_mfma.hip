@@ -189,6 +189,7 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
     // LDS; the step's first row is the scalar offset of the load
     auto dma16 = [&](const i32x4 &rsrc, unsigned int lds_addr, int voffset, int soffset, auto I) {
         constexpr int i = decltype(I)::value;
+        // (M0 is written here and read by the load that follows; nothing else of this kernel uses it)
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen offset:%4 lds"
                      :: "s"(__builtin_amdgcn_readfirstlane((int)lds_addr + i * (4096 - 128))), "v"(voffset), "s"(rsrc),
                         "s"(__builtin_amdgcn_readfirstlane(soffset)), "n"(i * 128) : "memory");
@@ -409,7 +410,8 @@ __global__ __launch_bounds__(NW * 64, 2) void fwd_reg_mfma_kernel(
         constexpr int KIND = decltype(kind)::value;
 #pragma unroll 1
         for (int u = ua; u < ub; ++u) {
-            // this wave's rows of step u have landed (with three buffers those of step u + 1 may be on their way)
+            // this wave's rows of step u have landed (with three buffers those of step u + 1 may be on their way:
+            // 2 * N_LD loads per step, and the loop body issues no other vector memory operation before this wait)
             if constexpr (Lds::n_buf == 3) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * N_LD) : "memory");
             else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();  // step u-1 is done everywhere: its buffer is free, and step u's is written

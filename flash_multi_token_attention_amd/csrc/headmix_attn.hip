@@ -655,17 +655,6 @@ __global__ __launch_bounds__(256) void headmix_dw_reduce_kernel(int n_part, int 
     if (wave == 0 && idx < hh) dW[idx] = (red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]);
 }
 
-template <auto Kern> hipError_t allow_lds(int bytes) {
-    static bool done[64] = {};
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return e;
-    if (dev < 64 && done[dev]) return hipSuccess;
-    e = hipFuncSetAttribute(reinterpret_cast<const void *>(Kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-    if (e == hipSuccess && dev < 64) done[dev] = true;
-    return e;
-}
-
 template <int H, int D>
 hipError_t launch_fwd(const HmArgs &a, int out_dt, const void *q, const void *k, const void *v, const float *w, void *o,
                       float *l, float *m, hipStream_t s) {
@@ -673,12 +662,12 @@ hipError_t launch_fwd(const HmArgs &a, int out_dt, const void *q, const void *k,
     static_assert(lds <= 160 * 1024, "LDS budget");
     dim3 grid((a.N + HT - 1) / HT, a.B);
     if (out_dt == CONVATTN_BF16) {
-        hipError_t e = allow_lds<headmix_fwd_kernel<H, D, bf16_t>>(lds);
+        hipError_t e = set_max_lds_once<headmix_fwd_kernel<H, D, bf16_t>>(lds);
         if (e != hipSuccess) return e;
         headmix_fwd_kernel<H, D, bf16_t><<<grid, HW * 64, lds, s>>>(a, (const bf16_t *)q, (const bf16_t *)k,
                                                                      (const bf16_t *)v, w, (bf16_t *)o, l, m);
     } else {
-        hipError_t e = allow_lds<headmix_fwd_kernel<H, D, float>>(lds);
+        hipError_t e = set_max_lds_once<headmix_fwd_kernel<H, D, float>>(lds);
         if (e != hipSuccess) return e;
         headmix_fwd_kernel<H, D, float><<<grid, HW * 64, lds, s>>>(a, (const bf16_t *)q, (const bf16_t *)k,
                                                                    (const bf16_t *)v, w, (float *)o, l, m);
@@ -692,7 +681,7 @@ hipError_t launch_bwd(const HmArgs &a, const void *q, const void *k, const void 
     constexpr int lds = HmLds<H, D, bwd_ahead<H, D, WHAT>() ? H / HW : (bwd_frag_staging<H, D, WHAT>() ? 3 : 1)>::total;
     static_assert(lds <= 160 * 1024, "LDS budget");
     static_assert(HW * H * H * 4 <= HmLds<H, D>::arr_bytes, "room for the dW accumulators of the waves");
-    hipError_t e = allow_lds<headmix_bwd_kernel<H, D, WHAT>>(lds);
+    hipError_t e = set_max_lds_once<headmix_bwd_kernel<H, D, WHAT>>(lds);
     if (e != hipSuccess) return e;
     dim3 grid((a.N + HT - 1) / HT, a.B, WHAT == 1 ? H / 16 : 1);
     headmix_bwd_kernel<H, D, WHAT><<<grid, HW * 64, lds, s>>>(a, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v,

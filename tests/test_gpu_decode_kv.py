@@ -51,7 +51,7 @@ def test_gqa_dense_and_cache_view(H, H_kv, c_q, causal):
         assert torch.equal(plain[0], same[0]) and torch.equal(plain[1], same[1]) and torch.equal(plain[2], same[2])
 
 
-@pytest.mark.parametrize("d,page,H,H_kv", [(128, 16, 4, 4), (128, 64, 8, 2), (64, 128, 4, 1)])
+@pytest.mark.parametrize("d,page,H,H_kv", [(128, 16, 4, 4), (128, 64, 8, 2), (64, 128, 4, 1), (32, 32, 8, 2)])
 @pytest.mark.parametrize("causal", [False, True])
 def test_paged_cache_with_ragged_lengths(d, page, H, H_kv, causal):
     B, c_q, c_k = 3, 6, 11
