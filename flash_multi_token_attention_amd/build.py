@@ -33,10 +33,6 @@ UNITS = [
     ("reduce_kernels.hip", "reduce_kernels", []),
     ("fwd_reg_mfma.hip", "fwd_reg_mfma", []),
     ("bwd_dq_mfma.hip", "bwd_dq_mfma", VGPR_FORM),
-    ("bwd_dkdv_mfma.hip", "bwd_dkdv_mfma_narrow", ["-DCONVATTN_DKDV_UNIT=0"]),
-    ("bwd_dkdv_mfma.hip", "bwd_dkdv_mfma_wide", ["-DCONVATTN_DKDV_UNIT=1"]),
-    ("bwd_ws_mfma.hip", "bwd_ws_mfma", []),
-    ("bwd_dq_gemm.hip", "bwd_dq_gemm", []),
     ("bwd_chain_mfma.hip", "bwd_chain_mfma_all", ["-DCONVATTN_CHAIN_UNIT=3"]),
     ("bwd_chain_mfma.hip", "bwd_chain_mfma_kv", ["-DCONVATTN_CHAIN_UNIT=1"]),
     ("bwd_chain_mfma.hip", "bwd_chain_mfma_qw", ["-DCONVATTN_CHAIN_UNIT=2"]),

@@ -157,27 +157,26 @@ int convattn_bwd_preprocess(const convattn_desc *desc, const void *o, const void
                                static_cast<hipStream_t>(stream));
 }
 
-// Workspace of the one-pass backward on the MFMA path: dS blocks, dW partials and (windows of up
-// to 8 query taps) the dC scale of every (batch, head), each part 256-byte aligned.
+// Workspace of the one-pass backward on the MFMA path: dS blocks, dW partials and the dC scale of
+// every (batch, head), each part 256-byte aligned.
 struct FusedWs {
     size_t ds_bytes, part_off, scale_off, total;
-    bool chain;
 };
 static FusedWs fused_ws(const Problem &p) {
     FusedWs w;
-    w.chain = chain_ok(p);
-    w.ds_bytes = w.chain ? chain_ds_bytes(p) : mfma_ds_bytes(p);
+    w.ds_bytes = chain_ds_bytes(p);
     w.part_off = align256(w.ds_bytes);
     w.scale_off = w.part_off + align256(fused_dw_bytes(p));
-    w.total = w.scale_off + (w.chain ? align256(chain_scale_bytes(p)) : 0);
+    w.total = w.scale_off + align256(chain_scale_bytes(p));
     return w;
 }
 
-// The dQ + dW pass on the chain path (windows of up to 8 query taps) is the key-stationary kernel
-// without its dK / dV half plus the dQ = dS K product: its "dW partial buffer" is the one-pass
-// backward's workspace (dS blocks, dW partials, dC scales).
+// The dQ + dW pass on the MFMA path is the key-stationary kernel without its dK / dV half plus the
+// dQ = dS K product: its "dW partial buffer" is the one-pass backward's workspace (dS blocks, dW
+// partials, dC scales).  With CONVATTN_FLAG_LOW_MEMORY it is the query-stationary kernel of
+// bwd_dq_mfma.hip, whose buffer holds dW partials only.
 static bool dq_dw_uses_chain(const convattn_desc *desc, const Problem &p) {
-    return pick_path(desc, p, CONVATTN_OP_BWD) == 1 && chain_ok(p) && !(desc->flags & CONVATTN_FLAG_LOW_MEMORY);
+    return pick_path(desc, p, CONVATTN_OP_BWD) == 1 && !(desc->flags & CONVATTN_FLAG_LOW_MEMORY);
 }
 
 size_t convattn_dw_partial_bytes(const convattn_desc *desc) {
@@ -235,10 +234,8 @@ int convattn_bwd_dkdv(const convattn_desc *desc, const void *q, const void *k, c
     REQUIRE_PTR(q); REQUIRE_PTR(k); REQUIRE_PTR(v); REQUIRE_PTR(d_o); REQUIRE_PTR(D);
     REQUIRE_PTR(lse); REQUIRE_PTR(w); REQUIRE_PTR(dk); REQUIRE_PTR(dv);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (pick_path(desc, p, CONVATTN_OP_BWD) == 1 && chain_ok(p))   // the key-stationary kernel without dS and dW; it scales dC by D
+    if (pick_path(desc, p, CONVATTN_OP_BWD) == 1)   // the key-stationary kernel without dS and dW; it scales dC by D
         return (int)mfma_bwd_chain(p, desc->out_dtype, 1, q, k, v, d_o, D, lse, w, nullptr, dk, dv, nullptr, nullptr, s);
-    if (pick_path(desc, p, CONVATTN_OP_BWD) == 1)
-        return (int)mfma_bwd_dkdv(p, desc->out_dtype, q, k, v, d_o, D, lse, w, dk, dv, s);
     return (int)generic_bwd_dkdv(p, desc->in_dtype, desc->out_dtype, q, k, v, d_o, D, lse, w, dk, dv, s);
 }
 
@@ -263,8 +260,6 @@ int convattn_bwd_fused_dkdv(const convattn_desc *desc, const void *q, const void
     unsigned char *ws = static_cast<unsigned char *>(workspace);
     const FusedWs lay = fused_ws(p);
     float *part = reinterpret_cast<float *>(ws + lay.part_off);
-    if (!lay.chain)
-        return (int)mfma_bwd_fused_ws(p, desc->out_dtype, q, k, v, d_o, D, lse, w, dk, dv, ws, part, s);
     float *scale = reinterpret_cast<float *>(ws + lay.scale_off);
     hipError_t e = mfma_dc_scale(p, d_o, v, scale, s);
     if (e != hipSuccess) return (int)e;
@@ -286,10 +281,6 @@ int convattn_bwd_fused_dq(const convattn_desc *desc, const void *q, const void *
                                       static_cast<float *>(workspace), s);
     }
     const FusedWs lay = fused_ws(p);
-    if (!lay.chain) {
-        REQUIRE_PTR(D);
-        return (int)mfma_dq_from_ds(p, desc->out_dtype, k, workspace, D, dq, s);
-    }
     const float *scale = reinterpret_cast<const float *>(static_cast<const unsigned char *>(workspace) + lay.scale_off);
     return (int)mfma_dq_from_rows(p, desc->out_dtype, k, workspace, scale, dq, s);
 }

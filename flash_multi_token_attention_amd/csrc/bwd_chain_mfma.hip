@@ -1,5 +1,5 @@
-// Whole backward of conv-attention on bf16 MFMA (gfx950), windows of 7 and 8 query taps: the score chain
-// stays in registers.  (Windows of up to 6 query taps run the three-role kernel of bwd_chain3_mfma.hip,
+// Whole backward of conv-attention on bf16 MFMA (gfx950), windows of 7 to 11 query taps (instances of 8 and
+// 12 tap slots): the score chain stays in registers.  (Windows of up to 6 query taps run the three-role kernel of bwd_chain3_mfma.hip,
 // which shares this file's building blocks through chain_common.hpp; the per-(batch, head) dC scale
 // kernels of both live here.)
 //
@@ -211,16 +211,22 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
     // trip to memory instead of several.
     fetch_tile(0);
     load_stats(r_begin);
+    // bands of the window (direct: times scale * log2 e, the convolved scores come out in log2 units; flipped:
+    // times the softmax scale); the first barrier of the tile loop publishes them
+    if constexpr (Lds::compact_bands)
+        band_tab_build<CQT>(smem + Lds::band_off, W + (size_t)h * cq * ck, cq, ck, pk, p.scale * kLog2e, p.scale, tid, NT);
+    // lane's part of a band's address: the tap slot is a constant offset from one address register
+    const unsigned int band_lane = Lds::compact_bands ? band_tab_lane_off(g, n) : lane * 16;
+    auto read_band = [&](const unsigned char *lane_ptr, int slot) {   // (slot: a constant after unrolling)
+        if constexpr (Lds::compact_bands) return band_tab_read(lane_ptr + slot * Lds::band_slot);
+        else return *reinterpret_cast<const f16x8 *>(lane_ptr + slot * Lds::band_slot);
+    };
 
     if constexpr (producer) {
         // ================================ producer ================================
         const bf16_t *Kb = K + bh * p.Nk * D;
         const bf16_t *Vb = V + bh * p.Nk * D;
-        // bands (times scale * log2 e: the convolved scores come out in log2 units) in LDS, one KB
-        // per tap slot, the slots dealt out to the four waves; the first barrier of the tile loop
-        // publishes them
-        // lane's 16 bytes of a band: the tap slot is a constant offset from one address register
-        const unsigned char *bands = smem + opaque((unsigned int)Lds::band_off + lane * 16);
+        const unsigned char *bands = smem + opaque((unsigned int)Lds::band_off + band_lane);
         bf16x8 kf[NSB][KS];  // K rows c0-16 .. c0+47
         bf16x8 vf[NCB][KS];  // V rows c0-8 .. c0+39
 #pragma unroll
@@ -241,9 +247,11 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks)
                 q_above[f][ks] = __builtin_bit_cast(bf16x8, load_row16_nb<D>(Qb, r_begin - BR + 2 * n + f, p.Nq, ks * 32 + g * 8));
-        for (int t = pr; t < CQT; t += NP)
-            *reinterpret_cast<f16x8 *>(smem + Lds::band_off + t * 1024 + lane * 16) =
-                band_frag<CQT>(t, W + (size_t)h * cq * ck, cq, ck, pk, g, n, false, p.scale * kLog2e);
+        // (ready-made fragments: one KB per tap slot, the slots dealt out to the four waves)
+        if constexpr (!Lds::compact_bands)
+            for (int t = pr; t < CQT; t += NP)
+                *reinterpret_cast<f16x8 *>(smem + Lds::band_off + t * 1024 + lane * 16) =
+                    band_frag<CQT>(t, W + (size_t)h * cq * ck, cq, ck, pk, g, n, false, p.scale * kLog2e);
         stage_stats(0);
         load_stats(r_begin + BR);
 
@@ -272,7 +280,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
 #pragma unroll
                     for (int f = 0; f < 2; ++f) acc[kb][f] = mfma_bf16(kf[kb][ks], qf[f], acc[kb][f]);
             }
-            const int rbase = (tp * BR) % S_RING;
+            const int rbase = (tp * BR) % Lds::ring_rows;
 #pragma unroll
             for (int kb = 0; kb < PNSB; ++kb)
 #pragma unroll
@@ -292,7 +300,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                     pd[kb][f][1] = two[1];
                     if (WANT_QW && kb < 3) {
                         const int rr = rbase + 2 * n + f;
-                        *reinterpret_cast<u32x2 *>(s_ring + (rr >= S_RING ? rr - S_RING : rr) * SST + (kb * 16 + 4 * g) * 2) =
+                        *reinterpret_cast<u32x2 *>(s_ring + (rr >= Lds::ring_rows ? rr - Lds::ring_rows : rr) * SST + (kb * 16 + 4 * g) * 2) =
                             (u32x2){pd[kb][f][0], pd[kb][f][1]};
                     }
                 }
@@ -358,7 +366,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                         constexpr int delta = t0 - (CQT - 1);
                         constexpr int f = delta & 1, s = (f - delta) / 2;
                         f16x8 tf_cur = tf_prev;
-                        if constexpr (t0 < CQT) tf_cur = *reinterpret_cast<const f16x8 *>(bands + t0 * 1024);
+                        if constexpr (t0 < CQT) tf_cur = read_band(bands, t0);
                         unsigned int sh[NSB][2];
 #pragma unroll
                         for (int kb = 0; kb < PNSB; ++kb)
@@ -467,17 +475,22 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
     } else {
         // ================================ consumer ================================
         const float *w_head = W + (size_t)h * cq * ck;
-        // flipped bands (times the softmax scale) in LDS, one KB per tap slot, dealt out to the four waves
-        unsigned char *bands = smem + opaque((unsigned int)Lds::band_off + CQT * 1024 + lane * 16);
-        for (int t = pr; t < CQT; t += NP)
-            *reinterpret_cast<f16x8 *>(bands + t * 1024) = band_frag<CQT>(t, w_head, cq, ck, pk, g, n, true, p.scale);
+        // flipped bands, after the direct ones
+        unsigned char *bands = smem + opaque((unsigned int)Lds::band_off + CQT * Lds::band_slot + band_lane);
+        if constexpr (!Lds::compact_bands)
+            for (int t = pr; t < CQT; t += NP)
+                *reinterpret_cast<f16x8 *>(bands + t * 1024) = band_frag<CQT>(t, w_head, cq, ck, pk, g, n, true, p.scale);
         stage_stats(0);
         load_stats(r_begin + BR);
         // dW: a unit is the key blocks of two pairs (pair group) times one tap slot; every wave takes one pair
-        // group and half of the tap slots, in one pass.
-        constexpr int NU = (CQT + 1) / 2;   // units per pass
-        constexpr int NPASS = 1, TH = NU * NPASS;
-        const int dw_pg[NPASS] = {pr >> 1}, dw_t[NPASS] = {(pr & 1) * NU};   // pair group and first tap slot
+        // group and half of the tap slots, in one pass (two for more than 8 tap slots: the operands of a
+        // pass are in registers three key blocks deep).
+        static_assert(CQT % 2 == 0, "half of the tap slots per wave");
+        constexpr int NPASS = CQT > 8 ? 2 : 1, TH = CQT / 2, NU = TH / NPASS;   // units per pass
+        static_assert(NU * NPASS == TH, "whole units per pass");
+        int dw_pg[NPASS], dw_t[NPASS];   // pair group and first tap slot
+#pragma unroll
+        for (int ps = 0; ps < NPASS; ++ps) { dw_pg[ps] = pr >> 1; dw_t[ps] = (pr & 1) * TH + ps * NU; }
         constexpr bool dw_wave = true;
         f32x4 acc_k[NDB][DB], acc_v[2][DB];
 #pragma unroll
@@ -567,7 +580,7 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                 for (int sb = 0; sb < NDB; ++sb) ds[sb][0] = ds[sb][1] = (f32x4){0.f, 0.f, 0.f, 0.f};
                 // flipped bands: the fragment of step e + 2 is read during step e (two steps of MFMAs
                 // cover the LDS latency; read one step ahead, every step waited for its band)
-                auto band_of = [&](int e) { return *reinterpret_cast<const f16x8 *>(bands + (CQT - 1 - e) * 1024); };
+                auto band_of = [&](int e) { return read_band(bands, CQT - 1 - e); };
                 f16x8 tbq[4];   // bands of steps e-1 .. e+2
                 tbq[0] = band_of(0);
                 tbq[1] = band_of(CQT >= 2 ? 1 : 0);
@@ -624,16 +637,16 @@ __device__ __forceinline__ void chain_role(const CHAIN_CONST_AS ChainArgs *args_
                 constexpr int ps = decltype(PS)::value;
                 const int pg = dw_pg[ps], t_lo = dw_t[ps];
                 // Ring rows of this lane's two transpose reads at the wave's first tap slot: tile row 0
-                // at tap slot 0 is ring row wbase; the TH tap slots are consecutive rows (mod S_RING).
-                const int wbase = ((u + 1) * BR - (CQT - 1) + S_RING) % S_RING;
+                // at tap slot 0 is ring row wbase; the TH tap slots are consecutive rows (mod the ring's rows).
+                const int wbase = ((u + 1) * BR - (CQT - 1) + Lds::ring_rows) % Lds::ring_rows;
                 const unsigned int c_lane = opaque(tr_lane_off(CST, g, n));
                 const unsigned int ring0 = Lds::pair_off + 2 * pg * Lds::pair_bytes + 4 * (n & 3) * 2;
                 unsigned int a_lo[NU], a_hi[NU];
 #pragma unroll
                 for (int tt = 0; tt < NU; ++tt) {
                     const unsigned int ra = wbase + 4 * g + (n >> 2) + min(t_lo + tt, CQT - 1), rb = ra + 16;
-                    a_lo[tt] = opaque(ring0 + min(ra, ra - S_RING) * SST);
-                    a_hi[tt] = opaque(ring0 + min(rb, rb - S_RING) * SST);
+                    a_lo[tt] = opaque(ring0 + min(ra, ra - Lds::ring_rows) * SST);
+                    a_hi[tt] = opaque(ring0 + min(rb, rb - Lds::ring_rows) * SST);
                 }
                 // score block jb' = 0..4 of the group: block jb' & 1 (or 2 for the last) of pair 2 pg + jb' / 2
                 // (blocks 0..3: a constant offset from the lane's address; block 4 is block 0 of the pair
@@ -797,7 +810,7 @@ __global__ __launch_bounds__(NT) void bwd_chain_kernel(ChainArgs args) {
 constexpr int kScaleChunks = 32;
 __global__ __launch_bounds__(256) void dc_scale_partial_kernel(int Nq, int Nk, int d, const bf16_t *__restrict__ dO,
                                                                const bf16_t *__restrict__ V, float *__restrict__ part) {
-    const size_t bh = blockIdx.y;
+    const size_t bh = (size_t)blockIdx.z * gridDim.y + blockIdx.y;   // y = head, z = batch
     __shared__ float red[2][4];
 #pragma unroll
     for (int which = 0; which < 2; ++which) {
@@ -861,7 +874,8 @@ hipError_t pick_cq(const Problem &p, const void *q, const void *k, const void *v
                    const float *Dl, const float *lse, const float *w, const float *dc_scale, void *dk, void *dv,
                    void *ds_ws, float *dw_part, hipStream_t s) {
     // (windows of up to 6 query taps run the three-role kernel of bwd_chain3_mfma.hip)
-    return launch_chain<D, 8, TO, WANT>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
+    if (p.c_q <= 8) return launch_chain<D, 8, TO, WANT>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
+    return launch_chain<D, 12, TO, WANT>(p, q, k, v, d_o, Dl, lse, w, dc_scale, dk, dv, ds_ws, dw_part, s);
 }
 
 template <int WANT>
@@ -887,7 +901,7 @@ hipError_t pick_shape(const Problem &p, int out_dt, const void *q, const void *k
 hipError_t mfma_dc_scale(const Problem &p, const void *d_o, const void *v, float *dc_scale, hipStream_t s) {
     // dc_scale holds {s, log2 s} per (batch, head), then the partial maxima
     float *part = dc_scale + (size_t)p.B * p.H * 2;
-    dc_scale_partial_kernel<<<dim3(kScaleChunks, p.B * p.H), 256, 0, s>>>(p.Nq, p.Nk, p.d, (const bf16_t *)d_o,
+    dc_scale_partial_kernel<<<dim3(kScaleChunks, p.H, p.B), 256, 0, s>>>(p.Nq, p.Nk, p.d, (const bf16_t *)d_o,
                                                                           (const bf16_t *)v, part);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;

@@ -17,6 +17,7 @@ constexpr int NCB = 3;           // C / dP / dC blocks: keys c0-8+16cb
 constexpr int NDB = 2;           // dS blocks: keys c0+16sb
 constexpr int SST = 112;         // bytes per row of the S tile in LDS (48 keys fp16 + 16)
 constexpr int S_RING = 72;       // rows of the S ring: a tile being written, the tile before it and 8 rows more (>= c_q - 1)
+constexpr int kBandTab = 352;    // bytes of a compact band table: 44 slots of 4 fp16 (see band_tab_build)
 constexpr int CST = 112;         // bytes per row of the dC tile (48 keys fp16 + 16)
 constexpr int PST = 72;          // bytes per row of the P and dS tiles (32 keys bf16 + 8)
 static_assert(BKW == kKvKeysPerWg && WK == kChainKeys && BR == kChainRows, "dS workspace layout");
@@ -34,16 +35,21 @@ template <int D, int CQT> struct ChainLds {
     static constexpr int g_off = q_off + q_slots * tile_bytes, g_slots = 3;  // tiles it-1 .. it+1
     static constexpr int stat_off = g_off + g_slots * tile_bytes;   // LSE and D of a tile: two slots
     static constexpr int stat_bytes = 2 * (2 * BR * 4);
-    static constexpr int band_off = stat_off + stat_bytes;          // bands, then flipped bands: one KB per tap slot
-    static constexpr int band_bytes = 2 * CQT * 1024;
+    // bands, then flipped bands: one KB of ready-made fragments per tap slot, or (windows of more than 8
+    // query taps, where those do not fit) one compact table per tap slot that the lanes read their fragments from
+    static constexpr bool compact_bands = CQT > 8;
+    static constexpr int band_slot = compact_bands ? kBandTab : 1024;
+    static constexpr int band_off = stat_off + stat_bytes;
+    static constexpr int band_bytes = 2 * CQT * band_slot;
     static constexpr int pair_off = band_off + band_bytes;
-    static constexpr int s_bytes = S_RING * SST;
+    static constexpr int ring_rows = CQT > 9 ? S_RING + 4 : S_RING;   // >= 64 + CQT - 1
+    static constexpr int s_bytes = ring_rows * SST;
     static constexpr int c_bytes = 2 * BR * CST;
     static constexpr int p_bytes = 2 * BR * PST;
     static constexpr int ds_bytes = BR * PST;
     static constexpr int pair_bytes = s_bytes + c_bytes + p_bytes + ds_bytes;
     static constexpr int total = pair_off + NP * pair_bytes;
-    static_assert(CQT * 2 * 1024 <= pair_bytes, "room for the dW accumulators");
+    static_assert(2 * CQT * 2 * 1024 <= NP * pair_bytes, "room for the dW accumulators (they take the place of the pairs' tiles)");
 };
 
 // A lane-dependent LDS offset the compiler may not fold or hoist: what is added to it afterwards
@@ -130,6 +136,35 @@ __device__ __forceinline__ f16x8 band_frag(int t, const float *__restrict__ w_he
 #pragma unroll
     for (int e = 0; e < 8; ++e) f[e] = (_Float16)(v[e] * mul);
     return f;
+}
+
+// The same bands as compact tables.  A fragment is Toeplitz in (slot, lane): its value at k slot e of lane
+// (g, n) is T[x] with x = kappa(e, g) - n in [-15, 31], T[x] = w[a][pk +- (x - 8)] (zero outside the window),
+// and the eight k slots of a lane are x0 .. x0+3 and x0+16 .. x0+19 with x0 = 4g - n.  A table holds T as 44
+// slots of 4 fp16: slot 4k + r (k = 0..10, r = 0..3) = T[4k + r - 15 .. 4k + r - 12], so that lane (g, n) finds
+// its two groups at the slots 4k + r and 4(k + 4) + r with k = g - n/4 + 3, r = 3 - n%4: two aligned 8-byte
+// reads, 128 bytes apart, and the 28 distinct addresses of a wave fall into distinct banks.
+__device__ __forceinline__ unsigned int band_tab_lane_off(int g, int n) {
+    return (unsigned int)(((g - (n >> 2) + 3) * 4 + 3 - (n & 3)) * 8);
+}
+__device__ __forceinline__ f16x8 band_tab_read(const unsigned char *lane_ptr) {
+    const u32x2 lo = *reinterpret_cast<const u32x2 *>(lane_ptr), hi = *reinterpret_cast<const u32x2 *>(lane_ptr + 128);
+    return __builtin_bit_cast(f16x8, (u32x4){lo[0], lo[1], hi[0], hi[1]});
+}
+// Tables of all tap slots: CQT direct ones (times mul_direct), then CQT flipped ones (times mul_flipped), built
+// by all `nthreads` threads of the workgroup; a barrier has to follow before they are read.
+template <int CQT>
+__device__ __forceinline__ void band_tab_build(unsigned char *tabs, const float *__restrict__ w_head, int c_q, int c_k,
+                                               int pk, float mul_direct, float mul_flipped, int tid, int nthreads) {
+    constexpr int PER = kBandTab / 2;   // fp16 entries per table
+    for (int i = tid; i < 2 * CQT * PER; i += nthreads) {
+        const int td = i / PER, q = i - td * PER, flip = td >= CQT, t = td - flip * CQT;
+        const int a = t - (CQT - c_q), x = q - (q >> 2) * 3 - 15;   // entry e of slot s: x = s + e - 15
+        const int bb = flip ? pk - (x - kKeyHalo) : pk + (x - kKeyHalo);
+        float v = 0.f;
+        if (a >= 0 && bb >= 0 && bb < c_k) v = w_head[a * c_k + bb] * (flip ? mul_flipped : mul_direct);
+        reinterpret_cast<_Float16 *>(tabs)[i] = (_Float16)v;
+    }
 }
 
 // Kernel arguments as one block: each role reads them from the kernel argument segment with

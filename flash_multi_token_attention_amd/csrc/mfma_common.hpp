@@ -189,9 +189,8 @@ inline bool mfma_fwd_shape_ok(const Problem &p, int in_dt, unsigned flags) {
 // The backward kernels put the key taps on one 16-wide MFMA dimension.
 inline bool mfma_bwd_shape_ok(const Problem &p, int in_dt, unsigned flags) {
     // (the one-pass kernel addresses Q and dO of one (batch, head) with 32-bit byte offsets)
-    // (head dimension 32: the key-stationary kernels only, i.e. windows of up to 8 query taps and not the
-    // low-memory dQ pass)
-    const bool d32_ok = p.d != 32 || (p.c_q <= 8 && (long long)p.B * p.H <= 65535 && !(flags & CONVATTN_FLAG_LOW_MEMORY));
+    // (head dimension 32: the key-stationary kernels only, i.e. not the low-memory dQ pass)
+    const bool d32_ok = p.d != 32 || !(flags & CONVATTN_FLAG_LOW_MEMORY);
     return mfma_shape_ok(p, in_dt, flags) && d32_ok && p.c_k <= 15 && (size_t)p.Nq * p.d * 2 < (1ull << 31) &&
            ((long long)p.Nq + 16 + 127) / 128 <= kMaxGridZ && ((long long)p.Nk + 8 + 127) / 128 <= kMaxGridZ;
 }
@@ -241,42 +240,15 @@ inline int mfma_dq_tiles(const Problem &p) { return (p.Nq + kMfmaDqRows - 1) / k
 hipError_t mfma_bwd_dq_dw(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
                           const void *d_o, const float *Dl, const float *lse, const float *w, void *dq,
                           float *dw_part, hipStream_t s);
-hipError_t mfma_bwd_dkdv(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
-                         const void *d_o, const float *Dl, const float *lse, const float *w, void *dk,
-                         void *dv, hipStream_t s);
 
-// ---- whole backward in one pass over the score tiles ----
-// The key-stationary kernel's workgroups cover 128 keys each (+ 8: the dV ranges start 8 keys
-// early).  Besides dK and dV it leaves one dW partial per workgroup and dS as bf16 blocks
-// [key tile of 32][row tile of 64][32 keys][64 rows]; mfma_dq_from_ds multiplies those blocks
-// with K.  dS of a row is finished 16 rows after the row itself, so the row tiles are shifted:
-// row tile rt holds rows 64 rt - 16 .. 64 rt + 47.
-constexpr int kKvKeysPerWg = 128, kDsKeys = 32, kDsRows = 64, kDsRowShift = 16;
-// Inside a dS block the 64 rows of a key are stored in the order the producing lanes hold
-// them: position 32k + 8g + 4h + r holds the block's row 32k + 16h + 4g + r.
-__host__ __device__ inline int ds_row_of_pos(int pos) {
-    return (pos & 32) | ((pos & 4) << 2) | ((pos >> 3 & 3) << 2) | (pos & 3);
-}
+// ---- whole backward with the score chain in registers (bwd_chain_mfma.hip, bwd_chain3_mfma.hip, bwd_dq_rows.hip) ----
+constexpr int kKvKeysPerWg = 128;
 inline int mfma_kv_tiles(const Problem &p) { return (p.Nk + 8 + kKvKeysPerWg - 1) / kKvKeysPerWg; }
-inline int mfma_ds_key_tiles(const Problem &p) { return mfma_kv_tiles(p) * (kKvKeysPerWg / kDsKeys); }
-__host__ __device__ inline int mfma_ds_row_tiles(const Problem &p) { return (p.Nq + kDsRowShift + kDsRows - 1) / kDsRows; }
-inline size_t mfma_ds_bytes(const Problem &p) {
-    return (size_t)p.B * p.H * mfma_ds_key_tiles(p) * mfma_ds_row_tiles(p) * kDsKeys * kDsRows * 2;
-}
-// bwd_ws_mfma.hip: 8-wave workgroups, producer / consumer wave pairs, two waves per SIMD.
-hipError_t mfma_bwd_fused_ws(const Problem &p, int out_dt, const void *q, const void *k, const void *v,
-                             const void *d_o, const float *Dl, const float *lse, const float *w, void *dk,
-                             void *dv, void *ds_ws, float *dw_part, hipStream_t s);
-hipError_t mfma_dq_from_ds(const Problem &p, int out_dt, const void *k, const void *ds_ws, const float *Dl,
-                           void *dq, hipStream_t s);
-
-// ---- whole backward with the score chain in registers (bwd_chain_mfma.hip, bwd_dq_rows.hip) ----
-// Windows of up to 8 query taps.  The key-stationary kernel's workgroups cover 128 keys each (+ 8:
+// The key-stationary kernel's workgroups cover 128 keys each (+ 8:
 // the dV ranges start 8 keys early); it leaves one dW partial per workgroup and dS as bf16 blocks
 // [key tile of 32][row tile of 32][32 rows][32 keys], which mfma_dq_from_rows multiplies with K.
 // dc_scale holds {s, log2 s} per (batch, head): the power of two dC is carried at (mfma_dc_scale).
-constexpr int kChainKeys = 32, kChainRows = 32, kChainMaxCq = 8;
-inline bool chain_ok(const Problem &p) { return p.c_q <= kChainMaxCq && (long long)p.B * p.H <= 65535; }
+constexpr int kChainKeys = 32, kChainRows = 32;
 inline int chain_key_tiles(const Problem &p) { return mfma_kv_tiles(p) * (kKvKeysPerWg / kChainKeys); }
 __host__ __device__ inline int chain_row_tiles(const Problem &p) { return (p.Nq + kChainRows - 1) / kChainRows; }
 inline size_t chain_ds_bytes(const Problem &p) {

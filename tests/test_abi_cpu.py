@@ -112,10 +112,9 @@ def test_fused_backward_workspace_size(lib):
     # 8 query taps: the same layout (88 taps per dW partial)
     n = lib.convattn_bwd_fused_workspace_bytes(C.byref(desc(c_q=8)))
     assert n == 2 * 4 * 8 * 4 * 32 * 32 * 2 + (2 * 4 * 2 * 88 * 4 + 255) // 256 * 256 + (2 * 4 * 66 * 4 + 255) // 256 * 256
-    # more than 8 query taps: dS blocks of 32 keys x 64 rows for 8 key tiles x ceil((128 + 16) / 64) row
-    # tiles, then the dW partials
+    # ... also for 9 to 11 query taps
     n = lib.convattn_bwd_fused_workspace_bytes(C.byref(desc(c_q=9)))
-    assert n == 2 * 4 * 8 * 3 * 32 * 64 * 2 + (2 * 4 * 2 * 99 * 4 + 255) // 256 * 256
+    assert n == 2 * 4 * 8 * 4 * 32 * 32 * 2 + (2 * 4 * 2 * 99 * 4 + 255) // 256 * 256 + (2 * 4 * 66 * 4 + 255) // 256 * 256
     # fp32 inputs run the two fp32 passes: the workspace is only the dW partial buffer
     f32 = desc(in_dtype=_lib.F32, out_dtype=_lib.F32)
     assert lib.convattn_bwd_fused_workspace_bytes(C.byref(f32)) == lib.convattn_dw_partial_bytes(C.byref(f32))

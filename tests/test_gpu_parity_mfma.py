@@ -91,10 +91,15 @@ BWD_SHAPES = [
     (1, 1, 130, 128, 6, 15),
     (1, 2, 31, 64, 2, 3),
     (1, 1, 1, 64, 6, 11),
-    # head dimension 32: windows of up to 8 query taps run the key-stationary kernels
+    # windows of 9 to 11 query taps: the 12-slot instance of the key-stationary kernel
+    (1, 2, 330, 128, 11, 11),
+    (1, 1, 257, 128, 9, 7),
+    (2, 2, 150, 64, 10, 15),
+    # head dimension 32
     (2, 2, 300, 32, 6, 11),
     (1, 2, 161, 32, 3, 3),
     (1, 1, 200, 32, 8, 9),
+    (1, 2, 200, 32, 11, 11),
 ]
 
 
