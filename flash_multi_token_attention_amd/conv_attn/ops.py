@@ -30,7 +30,9 @@ def _ptr(t: Optional[torch.Tensor]):
 
 
 def _stream(t: torch.Tensor):
-    return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+    # (the raw handle of torch's current stream on the tensor's device; torch.cuda.current_stream()
+    # builds a Stream object per call, which costs more than the launch it is asked for)
+    return C.c_void_p(torch._C._cuda_getCurrentRawStream(t.get_device()))
 
 
 def _check_input(t: torch.Tensor, name: str) -> None:

@@ -24,7 +24,7 @@ def _ptr(t: torch.Tensor):
 
 
 def _stream(t: torch.Tensor):
-    return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+    return C.c_void_p(torch._C._cuda_getCurrentRawStream(t.get_device()))
 
 
 def _bf16(t: torch.Tensor, name: str) -> torch.Tensor:
