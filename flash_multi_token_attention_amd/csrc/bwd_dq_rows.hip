@@ -61,14 +61,17 @@ __global__ __launch_bounds__(NW * 64) void dq_rows_kernel(Problem p, const bf16_
     const int n_steps = (k_end + BKS - 1) / BKS;
     const bool row_ok = rt < n_rt;
 
-    // two register sets: the loads of steps s+1 and s+2 are in flight while step s is multiplied
-    u32x4 kr_a[K_LD], sr_a[2][2], kr_b[K_LD], sr_b[2][2];
-    auto load_step = [&](int s, u32x4 (&kr)[K_LD], u32x4 (&sr)[2][2]) {
+    // the dS loads of steps s+1 and s+2 (two register sets) and the K loads of step s+1 (K comes from the
+    // L2, which the other row tiles of the head keep it in) are in flight while step s is multiplied
+    u32x4 kr[K_LD], sr_a[2][2], sr_b[2][2];
+    auto load_k = [&](int s) {
 #pragma unroll
         for (int i = 0; i < K_LD; ++i) {
             const int c = tid + i * NW * 64, row = c / CPR, cc = c % CPR;
             kr[i] = load_row16_clamped<D>(Kb, s * BKS + row, p.Nk, cc * 8);
         }
+    };
+    auto load_ds = [&](int s, u32x4 (&sr)[2][2]) {
 #pragma unroll
         for (int kp = 0; kp < 2; ++kp) {
             const int kt = s * 2 + kp;
@@ -84,7 +87,7 @@ __global__ __launch_bounds__(NW * 64) void dq_rows_kernel(Problem p, const bf16_
         }
     };
 
-    auto run_step = [&](int s, u32x4 (&kr)[K_LD], u32x4 (&sr)[2][2]) {
+    auto run_step = [&](int s, u32x4 (&sr)[2][2]) {
         unsigned char *Ks = smem + (s & 1) * Lds::k_bytes;
 #pragma unroll
         for (int i = 0; i < K_LD; ++i) {
@@ -101,7 +104,8 @@ __global__ __launch_bounds__(NW * 64) void dq_rows_kernel(Problem p, const bf16_
             for (int ob = 0; ob < 2; ++ob) sf[kp][ob] = __builtin_bit_cast(bf16x8, zero_unless(ok, sr[kp][ob]));
         }
         __syncthreads();
-        load_step(s + 2, kr, sr);
+        load_k(s + 1);
+        load_ds(s + 2, sr);
         if (causal && s * BKS > rw + 31) return;  // every key of the step is after the wave's rows
 
 #pragma unroll
@@ -117,11 +121,12 @@ __global__ __launch_bounds__(NW * 64) void dq_rows_kernel(Problem p, const bf16_
             }
         }
     };
-    load_step(0, kr_a, sr_a);
-    load_step(1, kr_b, sr_b);
+    load_k(0);
+    load_ds(0, sr_a);
+    load_ds(1, sr_b);
     for (int s = 0; s < n_steps; s += 2) {
-        run_step(s, kr_a, sr_a);
-        if (s + 1 < n_steps) run_step(s + 1, kr_b, sr_b);
+        run_step(s, sr_a);
+        if (s + 1 < n_steps) run_step(s + 1, sr_b);
     }
 
     // lane n of block ob = row 2 n + ob of the wave's 32; 4 consecutive head-dim columns per block
