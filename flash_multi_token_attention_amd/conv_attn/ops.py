@@ -171,7 +171,7 @@ def dq_backward(Q, K, V, dO, D, L, conv_kernel, scale, pad_q, pad_k, causal,
                 out_dtype=torch.float32, exact=False, low_memory=False) -> Tuple[torch.Tensor, torch.Tensor]:
     """-> (dQ [B,H,N,d], dconv_kernel [H,c_q,c_k] fp32).  ``L`` is the log-sum-exp
     M + log L and ``D`` is rowsum(dO * O), as the reference passes them.  On the MFMA path the
-    scratch of this op holds the bf16 dS matrix (B*H*Nq*Nk*2 bytes); ``low_memory`` runs the
+    scratch of this op holds the bf16 dS matrix (B*H*Nq*Nk*2 bytes, causal: half of that); ``low_memory`` runs the
     slower query-stationary kernel whose scratch is O(N)."""
     W, D, L, desc = _bwd_common(Q, K, V, dO, D, L, conv_kernel, scale, pad_q, pad_k, causal,
                                 out_dtype, exact, low_memory)
@@ -227,7 +227,7 @@ def backward(Q, K, V, dO, D, L, conv_kernel, scale, pad_q, pad_k, causal,
     """-> (dQ, dK, dV, dconv_kernel) from one pass over the score tiles: the results of
     ``dq_backward`` + ``dkdv_backward`` (same arguments) without computing the scores, the
     convolution and dC twice.  Needs a workspace the size of the bf16 dS matrix
-    (B*H*Nq*Nk*2 bytes: 2.2 GB at B4 H16 N4096, 17 GB at B1 H32 N16384).  A workspace above
+    (B*H*Nq*Nk*2 bytes, causal: half of that: 1.1 GB at B4 H16 N4096, 8.6 GB at B1 H32 N16384).  A workspace above
     ``max_workspace_bytes()`` is avoided by running the pass once per group of heads of one batch
     entry (every (batch, head) pair is independent; dconv_kernel is summed over the batch in index
     order); when a single pair does not fit or the allocation fails, the two passes with O(N)

@@ -652,7 +652,9 @@ __device__ __forceinline__ void chain3_role(const CHAIN_CONST_AS ChainArgs *args
 #pragma unroll
             for (int f = 0; f < 2; ++f) prev_dc[cb][f][0] = prev_dc[cb][f][1] = 0u;
         const int n_kt = gridDim.z * NP, kt = blockIdx.z * NP + pr;
-        bf16_t *ds_pair = dS_ws + (bh * n_kt + kt) * (size_t)n_rt * (WK * BR);
+        // (causal: the pair's first block is row tile kt - 1)
+        bf16_t *ds_pair = dS_ws + (bh * (size_t)chain_ds_block_off(causal, n_rt, n_kt) + (size_t)chain_ds_block_off(causal, n_rt, kt) -
+                                   chain_ds_first_rt(causal, kt)) * (WK * BR);
 
         bool ds_stored = false;  // the last iteration stored a dS block (after its tile loads)
         for (int it = 0; it <= n_tiles + 1; ++it) {

@@ -49,7 +49,7 @@ __global__ __launch_bounds__(NW * 64) void dq_rows_kernel(Problem p, const bf16_
     const bool causal = p.causal != 0;
     const size_t bh = (size_t)b * p.H + h;
     const bf16_t *Kb = K + bh * p.Nk * D;
-    const bf16_t *ws = dS_ws + bh * n_kt * n_rt * (size_t)BLK;
+    const bf16_t *ws = dS_ws + bh * (size_t)chain_ds_block_off(causal, n_rt, n_kt) * BLK;
 
     f32x4 acc[2][DB];
 #pragma unroll
@@ -75,7 +75,9 @@ __global__ __launch_bounds__(NW * 64) void dq_rows_kernel(Problem p, const bf16_
 #pragma unroll
         for (int kp = 0; kp < 2; ++kp) {
             const int kt = s * 2 + kp;
-            const size_t blk = (size_t)min(kt, n_kt - 1) * n_rt + min(rt, n_rt - 1);
+            // (a block that does not exist: any block that does; the registers are cleared before their use)
+            const int rt_c = min(rt, n_rt - 1), kt_c = causal ? min(kt, rt_c) : min(kt, n_kt - 1);
+            const size_t blk = (size_t)chain_ds_block_off(causal, n_rt, kt_c) + rt_c - chain_ds_first_rt(causal, kt_c);
 #pragma unroll
             for (int ob = 0; ob < 2; ++ob) {
                 // every dS block is read once: non-temporal, so that it does not push K out of the caches.

@@ -251,8 +251,18 @@ inline int mfma_kv_tiles(const Problem &p) { return (p.Nk + 8 + kKvKeysPerWg - 1
 constexpr int kChainKeys = 32, kChainRows = 32;
 inline int chain_key_tiles(const Problem &p) { return mfma_kv_tiles(p) * (kKvKeysPerWg / kChainKeys); }
 __host__ __device__ inline int chain_row_tiles(const Problem &p) { return (p.Nq + kChainRows - 1) / kChainRows; }
+// The dS blocks of one (batch, head) are kept as [key tile][row tile]; under the causal mask key tile kt has
+// only the row tiles from kt - 1 on (the rows before them see none of its keys), and only those are kept.
+__host__ __device__ inline int chain_ds_first_rt(bool causal, int kt) { return causal && kt > 1 ? kt - 1 : 0; }
+// blocks before key tile kt (with kt = the number of key tiles: blocks of a (batch, head))
+__host__ __device__ inline long long chain_ds_block_off(bool causal, int n_rt, int kt) {
+    if (!causal || kt <= 1) return (long long)kt * n_rt;
+    const long long k = kt < n_rt + 1 ? kt : n_rt + 1;   // key tiles from n_rt + 1 on have no blocks
+    return k * n_rt - (k - 1) * (k - 2) / 2;
+}
 inline size_t chain_ds_bytes(const Problem &p) {
-    return (size_t)p.B * p.H * chain_key_tiles(p) * chain_row_tiles(p) * kChainKeys * kChainRows * 2;
+    return (size_t)p.B * p.H * (size_t)chain_ds_block_off(p.causal != 0, chain_row_tiles(p), chain_key_tiles(p)) *
+           kChainKeys * kChainRows * 2;
 }
 // {s, log2 s} per (batch, head) followed by 32 x 2 partial maxima per (batch, head)
 inline size_t chain_scale_bytes(const Problem &p) { return (size_t)p.B * p.H * (2 + 64) * sizeof(float); }

@@ -134,7 +134,7 @@ int convattn_bwd_preprocess(const convattn_desc *desc, const void *o, const void
 /*
  * Bytes of the work buffer convattn_bwd_dq_dw needs (0 on a bad descriptor).  On the
  * bf16 matrix-core path this is the whole workspace of the
- * key-stationary kernel: the bf16 dS matrix, B*H*Nq*Nk*2 bytes (2.2 GB at B4 H16 N4096),
+ * key-stationary kernel: the bf16 dS matrix, B*H*Nq*Nk*2 bytes (causal: its lower triangle, 1.1 GB at B4 H16 N4096),
  * plus the dW partials and the dC scales.  With CONVATTN_FLAG_LOW_MEMORY in desc->flags
  * (and on every other path) it is the dW partials only, O(B*H*Nq/128) floats.
  */

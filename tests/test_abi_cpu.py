@@ -104,17 +104,22 @@ def test_dw_partial_size_matches_tiling(lib):
 
 
 def test_fused_backward_workspace_size(lib):
-    # bf16, N = 128, d = 64, 6 query taps: dS blocks of 32 rows x 32 keys bf16 for ceil((128 + 8) / 128) * 4
-    # key tiles x ceil(128 / 32) row tiles per (batch, head), then one dW partial per 128-key workgroup,
-    # then {scale, log2 scale} of dC and 32 x 2 partial maxima per (batch, head); each part 256-aligned
-    n = lib.convattn_bwd_fused_workspace_bytes(C.byref(desc()))
-    assert n == 2 * 4 * 8 * 4 * 32 * 32 * 2 + (2 * 4 * 2 * 66 * 4 + 255) // 256 * 256 + (2 * 4 * 66 * 4 + 255) // 256 * 256
-    # 8 query taps: the same layout (88 taps per dW partial)
+    # bf16, N = 128, d = 64, 6 query taps: dS blocks of 32 rows x 32 keys bf16, ceil((128 + 8) / 128) * 4 = 8 key tiles x
+    # ceil(128 / 32) = 4 row tiles per (batch, head) without a mask; under the causal mask key tile kt keeps the row
+    # tiles from kt - 1 on: 4 + 4 + 3 + 2 + 1 = 14 blocks.  Then one dW partial per 128-key workgroup, then
+    # {scale, log2 scale} of dC and 32 x 2 partial maxima per (batch, head); each part 256-aligned
+    tail = (2 * 4 * 2 * 66 * 4 + 255) // 256 * 256 + (2 * 4 * 66 * 4 + 255) // 256 * 256
+    assert lib.convattn_bwd_fused_workspace_bytes(C.byref(desc(causal=0))) == 2 * 4 * 8 * 4 * 32 * 32 * 2 + tail
+    assert lib.convattn_bwd_fused_workspace_bytes(C.byref(desc())) == 2 * 4 * 14 * 32 * 32 * 2 + tail
+    # (N = 4096: 128 + sum(128 .. 1) = 8384 of 132 x 128 = 16896 blocks)
+    big = desc(B=1, H=1, Nq=4096, Nk=4096)
+    tail_big = (33 * 66 * 4 + 255) // 256 * 256 + (66 * 4 + 255) // 256 * 256   # 33 workgroups of 128 keys
+    assert lib.convattn_bwd_fused_workspace_bytes(C.byref(big)) == 8384 * 32 * 32 * 2 + tail_big
+    # 8 query taps: the same layout (88 taps per dW partial), also for 9 to 11 query taps
     n = lib.convattn_bwd_fused_workspace_bytes(C.byref(desc(c_q=8)))
-    assert n == 2 * 4 * 8 * 4 * 32 * 32 * 2 + (2 * 4 * 2 * 88 * 4 + 255) // 256 * 256 + (2 * 4 * 66 * 4 + 255) // 256 * 256
-    # ... also for 9 to 11 query taps
+    assert n == 2 * 4 * 14 * 32 * 32 * 2 + (2 * 4 * 2 * 88 * 4 + 255) // 256 * 256 + (2 * 4 * 66 * 4 + 255) // 256 * 256
     n = lib.convattn_bwd_fused_workspace_bytes(C.byref(desc(c_q=9)))
-    assert n == 2 * 4 * 8 * 4 * 32 * 32 * 2 + (2 * 4 * 2 * 99 * 4 + 255) // 256 * 256 + (2 * 4 * 66 * 4 + 255) // 256 * 256
+    assert n == 2 * 4 * 14 * 32 * 32 * 2 + (2 * 4 * 2 * 99 * 4 + 255) // 256 * 256 + (2 * 4 * 66 * 4 + 255) // 256 * 256
     # fp32 inputs run the two fp32 passes: the workspace is only the dW partial buffer
     f32 = desc(in_dtype=_lib.F32, out_dtype=_lib.F32)
     assert lib.convattn_bwd_fused_workspace_bytes(C.byref(f32)) == lib.convattn_dw_partial_bytes(C.byref(f32))
