@@ -29,7 +29,10 @@ namespace {
 
 typedef short short4_t __attribute__((ext_vector_type(4)));
 
-constexpr int HW = 8;            // waves per workgroup
+// waves per workgroup: one per head with 16 heads (half the accumulators and fragments per wave, four waves per
+// SIMD to hide the latencies between the phases) where 128 registers per wave hold that without much scratch
+// (the forward, and the backward up to d = 64); otherwise 8 (two or four heads per wave)
+template <int H, int D, bool BWD> constexpr int kHmWaves = (H == 16 && (!BWD || D <= 64)) ? 16 : 8;
 constexpr int HT = 16;           // rows / keys per tile
 constexpr int SST = 20;          // floats per row of a score tile in LDS
 constexpr int HST = HT * SST + 16;   // floats per head of a score array (== 16 mod 32: see the reads in phase 2)
@@ -44,7 +47,7 @@ struct HmArgs {
 };
 
 // XT: staging tiles per wave (1, or one per head of the wave where K tiles are staged a phase early)
-template <int H, int D, int XT = 1> struct HmLds {
+template <int H, int D, int XT, int HW> struct HmLds {
     static constexpr int WST = H + 4;                       // floats per row of W
     static constexpr int XST = D * 2 + 32;                  // bytes per row of a staged bf16 tile
     static constexpr int arr_bytes = H * HST * 4;           // one score array
@@ -147,24 +150,38 @@ __device__ __forceinline__ void tile_times_staged(f32x4 (&acc)[D / 16], const fl
                                                              acc[db], 0, 0, 0);
 }
 
-// Max / sum over the 16 lanes of a lane group (all of them get the result).
+// Max / sum over the 16 lanes of a lane group (all of them get the result, bit for bit: at every step the
+// lanes are paired the same way from either side).  Rotations of the row of 16 by 8, 4, 2 and 1 lanes as DPP
+// moves: vector-ALU speed, where a shuffle through the LDS crossbar costs its latency eight times in a row.
+template <int ROR> __device__ __forceinline__ float row16_rot(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x120 + ROR, 0xf, 0xf, true));
+}
 __device__ __forceinline__ float row16_max(float v) {
-#pragma unroll
-    for (int o = 8; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 16));
-    return v;
+    v = fmaxf(v, row16_rot<8>(v));
+    v = fmaxf(v, row16_rot<4>(v));
+    v = fmaxf(v, row16_rot<2>(v));
+    return fmaxf(v, row16_rot<1>(v));
 }
 __device__ __forceinline__ float row16_sum(float v) {
-#pragma unroll
-    for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, 16);
-    return v;
+    v += row16_rot<8>(v);
+    v += row16_rot<4>(v);
+    v += row16_rot<2>(v);
+    return v + row16_rot<1>(v);
 }
 
-template <int H> __device__ __forceinline__ void load_w(float *Wl, int wst, const float *__restrict__ W, int tid) {
+// Workgroup barrier for data that is exchanged through LDS only: waits for this wave's LDS operations, not for
+// its global loads (__syncthreads() drains those too, which would expose the latency of every load that is
+// issued ahead of its use at the next barrier).
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+template <int H, int HW> __device__ __forceinline__ void load_w(float *Wl, int wst, const float *__restrict__ W, int tid) {
     for (int i = tid; i < H * H; i += HW * 64) Wl[(i / H) * wst + (i % H)] = W[i];
 }
 
 // Phase 1: scaled scores of the heads wave, wave + 8, ... for rows i0.. and keys j0.. -> S[h'][i][j]
-template <int H, int D>
+template <int H, int D, int HW>
 __device__ __forceinline__ void scores_phase(float *S, const HmArgs &a, const bf16_t *__restrict__ Qb,
                                              const bf16_t *__restrict__ Kb, int i0, int j0, int wave, int g, int n) {
 #pragma unroll
@@ -193,11 +210,12 @@ __device__ __forceinline__ void mix_row(f32x4 (&out)[H / 16], const float *Wl, i
 
 // ------------------------------------------------------------------ forward
 template <int H, int D, typename TO>
-__global__ __launch_bounds__(HW * 64) void headmix_fwd_kernel(HmArgs a, const bf16_t *__restrict__ Q,
+__global__ __launch_bounds__((kHmWaves<H, D, false> * 64)) void headmix_fwd_kernel(HmArgs a, const bf16_t *__restrict__ Q,
                                                               const bf16_t *__restrict__ K, const bf16_t *__restrict__ V,
                                                               const float *__restrict__ W, TO *__restrict__ O,
                                                               float *__restrict__ L, float *__restrict__ M) {
-    using Lds = HmLds<H, D>;
+    constexpr int HW = kHmWaves<H, D, false>;
+    using Lds = HmLds<H, D, 1, HW>;
     constexpr int DB = D / 16, HPW = H / HW, RPW = HT / HW;  // heads and rows per wave
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     float *S = reinterpret_cast<float *>(smem + Lds::s_off);
@@ -209,7 +227,7 @@ __global__ __launch_bounds__(HW * 64) void headmix_fwd_kernel(HmArgs a, const bf
     const size_t bo = (size_t)b * a.H * a.N * D;
     const bf16_t *Qb = Q + bo, *Kb = K + bo, *Vb = V + bo;
 
-    load_w<H>(Wl, Lds::WST, W, tid);
+    load_w<H, HW>(Wl, Lds::WST, W, tid);
     f32x4 acc_o[HPW][DB];
 #pragma unroll
     for (int t = 0; t < HPW; ++t)
@@ -242,21 +260,31 @@ __global__ __launch_bounds__(HW * 64) void headmix_fwd_kernel(HmArgs a, const bf
 
     const int j_end = a.causal ? min(a.N, i0 + HT) : a.N;
     for (int j0 = 0; j0 < j_end; j0 += HT) {
-        __syncthreads();   // the last tile's P has been used (and, first, W is in place)
+        lds_barrier();   // the last tile's P has been used (and, first, W is in place)
         if constexpr (AHEAD) {
+            // (the products first: they wait for the K fragments, which were asked for a tile ago; a wait placed
+            // after this tile's loads would be for those as well)
+            f32x4 sc[HPW];
+#pragma unroll
+            for (int t = 0; t < HPW; ++t) sc[t] = frags_dot<D>(qf[t], kf[t]);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int t = 0; t < HPW; ++t) {
                 const int h = wave + t * HW;
-                load_chunks<D>(vr[t], Vb + (size_t)h * a.N * D, j0, a.N, lane);
-                const f32x4 sc = frags_dot<D>(qf[t], kf[t]);
-#pragma unroll
-                for (int r = 0; r < 4; ++r) S[h * HST + (4 * g + r) * SST + n] = sc[r] * a.scale;
                 load_frags<D>(kf[t], Kb + (size_t)h * a.N * D, j0 + HT, a.N, g, n);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) S[h * HST + (4 * g + r) * SST + n] = sc[t][r] * a.scale;
             }
         } else {
-            scores_phase<H, D>(S, a, Qb, Kb, i0, j0, wave, g, n);
+            scores_phase<H, D, HW>(S, a, Qb, Kb, i0, j0, wave, g, n);
         }
-        __syncthreads();
+        lds_barrier();
+        // (the V rows of the tile are asked for here rather than with the K fragments: the vector memory pipe of
+        // the CU takes a workgroup's loads one after the other, and this phase has no other use for it)
+        if constexpr (AHEAD) {
+#pragma unroll
+            for (int t = 0; t < HPW; ++t) load_chunks<D>(vr[t], Vb + (size_t)(wave + t * HW) * a.N * D, j0, a.N, lane);
+        }
 #pragma unroll
         for (int rl = 0; rl < RPW; ++rl) {
             const int i = wave * RPW + rl;
@@ -279,7 +307,7 @@ __global__ __launch_bounds__(HW * 64) void headmix_fwd_kernel(HmArgs a, const bf
                     if (n == 0) al[h * HT + i] = alpha;
                 }
         }
-        __syncthreads();
+        lds_barrier();
 #pragma unroll
         for (int t = 0; t < HPW; ++t) {
             const int h = wave + t * HW;
@@ -334,13 +362,14 @@ __global__ __launch_bounds__(HW * 64) void headmix_fwd_kernel(HmArgs a, const bf
 }
 
 template <int H, int D, int WHAT> constexpr bool bwd_ahead() {
-    return WHAT == 0 && (H / HW) * (D / 32) <= 8 && HmLds<H, D, H / HW>::total <= 160 * 1024;
+    constexpr int HW = kHmWaves<H, D, true>;
+    return WHAT == 0 && (H / HW) * (D / 32) <= 8 && HmLds<H, D, H / HW, HW>::total <= 160 * 1024;
 }
 // dK + dV, where LDS allows three staging tiles per wave: the Q and dO tiles of the products with dS^T
 // and P^T are staged from the row fragments that the score and dP products load anyway, and the
 // fragments of two heads are loaded before the first of them is used.
 template <int H, int D, int WHAT> constexpr bool bwd_frag_staging() {
-    return WHAT == 1 && HmLds<H, D, 3>::total <= 160 * 1024;
+    return WHAT == 1 && HmLds<H, D, 3, kHmWaves<H, D, true>>::total <= 160 * 1024;
 }
 template <int D>
 __device__ __forceinline__ void stage_frags(unsigned char *xt, int xst, const bf16x8 (&f)[D / 32], int g, int n) {
@@ -355,20 +384,28 @@ __device__ __forceinline__ void stage_frags(unsigned char *xt, int xst, const bf
 // WHAT = 0: dQ and the dW partial of a row tile (grid: row tiles x batch);
 // WHAT = 1: dK and dV of 16 heads (blockIdx.z) of a key tile (grid: key tiles x batch x H / 16).
 template <int H, int D, int WHAT>
-__global__ __launch_bounds__(HW * 64) void headmix_bwd_kernel(HmArgs a, const bf16_t *__restrict__ Q,
+__global__ __launch_bounds__((kHmWaves<H, D, true> * 64)) void headmix_bwd_kernel(HmArgs a, const bf16_t *__restrict__ Q,
                                                               const bf16_t *__restrict__ K, const bf16_t *__restrict__ V,
                                                               const float *__restrict__ W, const bf16_t *__restrict__ dO,
                                                               const float *__restrict__ LSE, const float *__restrict__ Dl,
                                                               float *__restrict__ out0, float *__restrict__ out1) {
+    constexpr int HW = kHmWaves<H, D, true>;
     constexpr int DB = D / 16, HPW = H / HW, RPW = HT / HW, HB = H / 16;
-    constexpr int OPW = 2;   // WHAT = 1: heads of this workgroup's 16 that a wave accumulates for
+    constexpr int OPW = 16 / HW;   // WHAT = 1: heads of this workgroup's 16 that a wave accumulates for
+    constexpr int PU = HPW >= 2 ? 2 : 1;   // heads whose fragments are loaded before the first of them is used
     // dQ + dW, where registers and LDS allow: the Q / dO fragments of the wave's heads stay resident, the
     // K / V fragments of a key tile are loaded while the tile before it is worked on, dP is taken in the
     // score phase and the K tile is staged for the last phase from the fragments (no second load).
     constexpr bool AHEAD = bwd_ahead<H, D, WHAT>();
     constexpr bool FSTAGE = bwd_frag_staging<H, D, WHAT>();
     constexpr int XTILES = AHEAD ? HPW : (FSTAGE ? 3 : 1);   // FSTAGE: tile 0 = dO of the head at hand, 1 + x = Q of output head x
-    using Lds = HmLds<H, D, XTILES>;
+    using Lds = HmLds<H, D, XTILES, HW>;
+    // (where loads are issued a tile ahead of their use the barriers must not wait for them; the other instances
+    // measured faster with the full barrier)
+    auto tile_barrier = [] {
+        if constexpr (AHEAD) lds_barrier();
+        else __syncthreads();
+    };
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     float *S = reinterpret_cast<float *>(smem + Lds::s_off);
     float *P = reinterpret_cast<float *>(smem + Lds::p_off);
@@ -381,7 +418,7 @@ __global__ __launch_bounds__(HW * 64) void headmix_bwd_kernel(HmArgs a, const bf
     const bf16_t *Qb = Q + bo, *Kb = K + bo, *Vb = V + bo, *Gb = dO + bo;
     const int fixed0 = (WHAT == 0 ? gridDim.x - 1 - blockIdx.x : blockIdx.x) * HT;   // own row tile (0) or key tile (1)
 
-    load_w<H>(Wl, Lds::WST, W, tid);
+    load_w<H, HW>(Wl, Lds::WST, W, tid);
     constexpr int NACC = WHAT == 0 ? HPW : 2 * OPW;
     f32x4 acc[NACC][DB];   // WHAT 0: dQ of the wave's heads; WHAT 1: dK then dV of its output heads
 #pragma unroll
@@ -421,7 +458,7 @@ __global__ __launch_bounds__(HW * 64) void headmix_bwd_kernel(HmArgs a, const bf
     const int hi = WHAT == 0 ? (a.causal ? min(a.N, fixed0 + HT) : a.N) : a.N;
     for (int o0 = lo; o0 < hi; o0 += HT) {
         const int i0 = WHAT == 0 ? fixed0 : o0, j0 = WHAT == 0 ? o0 : fixed0;
-        __syncthreads();   // the last tile's dS has been used (and, first, W and the statistics are in place)
+        tile_barrier();   // the last tile's dS has been used (and, first, W and the statistics are in place)
         if (WHAT == 1) load_stats(i0);
         f32x4 dp_early[NF];
         if constexpr (AHEAD) {
@@ -441,16 +478,16 @@ __global__ __launch_bounds__(HW * 64) void headmix_bwd_kernel(HmArgs a, const bf
             }
         } else if constexpr (FSTAGE) {
 #pragma unroll
-            for (int t0 = 0; t0 < HPW; t0 += 2) {
-                bf16x8 xq[2][D / 32], xk[2][D / 32];
+            for (int t0 = 0; t0 < HPW; t0 += PU) {
+                bf16x8 xq[PU][D / 32], xk[PU][D / 32];
 #pragma unroll
-                for (int u = 0; u < 2; ++u) {
+                for (int u = 0; u < PU; ++u) {
                     const size_t ho = (size_t)(wave + (t0 + u) * HW) * a.N * D;
                     load_frags<D>(xq[u], Qb + ho, i0, a.N, g, n);
                     load_frags<D>(xk[u], Kb + ho, j0, a.N, g, n);
                 }
 #pragma unroll
-                for (int u = 0; u < 2; ++u) {
+                for (int u = 0; u < PU; ++u) {
                     const int t = t0 + u, h = wave + t * HW;
                     const f32x4 sc = frags_dot<D>(xq[u], xk[u]);
 #pragma unroll
@@ -459,9 +496,9 @@ __global__ __launch_bounds__(HW * 64) void headmix_bwd_kernel(HmArgs a, const bf
                 }
             }
         } else {
-            scores_phase<H, D>(S, a, Qb, Kb, i0, j0, wave, g, n);
+            scores_phase<H, D, HW>(S, a, Qb, Kb, i0, j0, wave, g, n);
         }
-        __syncthreads();
+        tile_barrier();
         // ---- P = exp(Z - LSE), rows of this wave ----
 #pragma unroll
         for (int rl = 0; rl < RPW; ++rl) {
@@ -477,20 +514,20 @@ __global__ __launch_bounds__(HW * 64) void headmix_bwd_kernel(HmArgs a, const bf
                     P[h * HST + i * SST + n] = visible ? __expf(z[hb][r] - lse_s[h * HT + i]) : 0.f;
                 }
         }
-        __syncthreads();
+        tile_barrier();
         // ---- heads of this wave: dP = dO V^T, (dV += P^T dO), dZ = P (dP - D) in place of P ----
         if constexpr (FSTAGE) {
 #pragma unroll
-            for (int t0 = 0; t0 < HPW; t0 += 2) {
-                bf16x8 xg[2][D / 32], xv[2][D / 32];
+            for (int t0 = 0; t0 < HPW; t0 += PU) {
+                bf16x8 xg[PU][D / 32], xv[PU][D / 32];
 #pragma unroll
-                for (int u = 0; u < 2; ++u) {
+                for (int u = 0; u < PU; ++u) {
                     const size_t ho = (size_t)(wave + (t0 + u) * HW) * a.N * D;
                     load_frags<D>(xg[u], Gb + ho, i0, a.N, g, n);
                     load_frags<D>(xv[u], Vb + ho, j0, a.N, g, n);
                 }
 #pragma unroll
-                for (int u = 0; u < 2; ++u) {
+                for (int u = 0; u < PU; ++u) {
                     const int t = t0 + u, h = wave + t * HW;
                     const f32x4 dp = frags_dot<D>(xg[u], xv[u]);
                     if (h / 16 == hs) {
@@ -528,7 +565,7 @@ __global__ __launch_bounds__(HW * 64) void headmix_bwd_kernel(HmArgs a, const bf
             }
         }
         }
-        __syncthreads();
+        tile_barrier();
         // ---- rows of this wave: dW += dZ S^T over its elements, then dS = scale W^T dZ in place ----
 #pragma unroll
         for (int rl = 0; rl < RPW; ++rl) {
@@ -551,7 +588,7 @@ __global__ __launch_bounds__(HW * 64) void headmix_bwd_kernel(HmArgs a, const bf
 #pragma unroll
                 for (int r = 0; r < 4; ++r) P[(hb * 16 + 4 * g + r) * HST + i * SST + n] = ds[hb][r] * a.scale;
         }
-        __syncthreads();
+        tile_barrier();
         // ---- heads of this wave: dQ += dS K, or dK += dS^T Q ----
         if constexpr (WHAT == 0) {
 #pragma unroll
@@ -658,7 +695,7 @@ __global__ __launch_bounds__(256) void headmix_dw_reduce_kernel(int n_part, int 
 template <int H, int D>
 hipError_t launch_fwd(const HmArgs &a, int out_dt, const void *q, const void *k, const void *v, const float *w, void *o,
                       float *l, float *m, hipStream_t s) {
-    constexpr int lds = HmLds<H, D>::total;
+    constexpr int HW = kHmWaves<H, D, false>, lds = HmLds<H, D, 1, HW>::total;
     static_assert(lds <= 160 * 1024, "LDS budget");
     dim3 grid((a.N + HT - 1) / HT, a.B);
     if (out_dt == CONVATTN_BF16) {
@@ -678,9 +715,10 @@ hipError_t launch_fwd(const HmArgs &a, int out_dt, const void *q, const void *k,
 template <int H, int D, int WHAT>
 hipError_t launch_bwd(const HmArgs &a, const void *q, const void *k, const void *v, const float *w, const void *d_o,
                       const float *lse, const float *Dl, float *out0, float *out1, hipStream_t s) {
-    constexpr int lds = HmLds<H, D, bwd_ahead<H, D, WHAT>() ? H / HW : (bwd_frag_staging<H, D, WHAT>() ? 3 : 1)>::total;
+    constexpr int HW = kHmWaves<H, D, true>;
+    constexpr int lds = HmLds<H, D, bwd_ahead<H, D, WHAT>() ? H / HW : (bwd_frag_staging<H, D, WHAT>() ? 3 : 1), HW>::total;
     static_assert(lds <= 160 * 1024, "LDS budget");
-    static_assert(HW * H * H * 4 <= HmLds<H, D>::arr_bytes, "room for the dW accumulators of the waves");
+    static_assert(HW * H * H * 4 <= HmLds<H, D, 1, HW>::arr_bytes, "room for the dW accumulators of the waves");
     hipError_t e = set_max_lds_once<headmix_bwd_kernel<H, D, WHAT>>(lds);
     if (e != hipSuccess) return e;
     dim3 grid((a.N + HT - 1) / HT, a.B, WHAT == 1 ? H / 16 : 1);
