@@ -248,13 +248,17 @@ __global__ __launch_bounds__((kHmWaves<H, D, false> * 64)) void headmix_fwd_kern
     // the latency of these loads.
     constexpr bool AHEAD = HPW * (D / 32) <= 8;
     constexpr int NCH = (HT * D / 8 + 63) / 64;
-    bf16x8 qf[AHEAD ? HPW : 1][D / 32], kf[AHEAD ? HPW : 1][D / 32];
-    u32x4 vr[AHEAD ? HPW : 1][NCH];
+    // (K rows as whole rows, 1 KB of consecutive memory per load, and from the wave's staging tile into the
+    // fragments: a fragment load straight from memory takes 64 bytes of each of 16 rows, half of every cache line
+    // it touches, and the vector memory pipe of the CU, which a workgroup's loads pass one after the other, is what
+    // the score phase waits for)
+    bf16x8 qf[AHEAD ? HPW : 1][D / 32];
+    u32x4 kr[AHEAD ? HPW : 1][NCH], vr[AHEAD ? HPW : 1][NCH];
     if constexpr (AHEAD) {
 #pragma unroll
         for (int t = 0; t < HPW; ++t) {
             load_frags<D>(qf[t], Qb + (size_t)(wave + t * HW) * a.N * D, i0, a.N, g, n);
-            load_frags<D>(kf[t], Kb + (size_t)(wave + t * HW) * a.N * D, 0, a.N, g, n);
+            load_chunks<D>(kr[t], Kb + (size_t)(wave + t * HW) * a.N * D, 0, a.N, lane);
         }
     }
 
@@ -266,12 +270,20 @@ __global__ __launch_bounds__((kHmWaves<H, D, false> * 64)) void headmix_fwd_kern
             // after this tile's loads would be for those as well)
             f32x4 sc[HPW];
 #pragma unroll
-            for (int t = 0; t < HPW; ++t) sc[t] = frags_dot<D>(qf[t], kf[t]);
+            for (int t = 0; t < HPW; ++t) {
+                stage_chunks<D>(xt, Lds::XST, kr[t], lane);
+                bf16x8 kf[D / 32];
+#pragma unroll
+                for (int blk = 0; blk < D / 32; ++blk)
+                    kf[blk] = *reinterpret_cast<const bf16x8 *>(xt + n * Lds::XST + (blk * 32 + 8 * g) * 2);
+                sc[t] = frags_dot<D>(qf[t], kf);
+                __builtin_amdgcn_wave_barrier();
+            }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int t = 0; t < HPW; ++t) {
                 const int h = wave + t * HW;
-                load_frags<D>(kf[t], Kb + (size_t)h * a.N * D, j0 + HT, a.N, g, n);
+                load_chunks<D>(kr[t], Kb + (size_t)h * a.N * D, j0 + HT, a.N, lane);
 #pragma unroll
                 for (int r = 0; r < 4; ++r) S[h * HST + (4 * g + r) * SST + n] = sc[t][r] * a.scale;
             }
