@@ -415,7 +415,7 @@ __global__ __launch_bounds__((kHmWaves<H, D, true> * 64)) void headmix_bwd_kerne
     // (where loads are issued a tile ahead of their use the barriers must not wait for them; the other instances
     // measured faster with the full barrier)
     auto tile_barrier = [] {
-        if constexpr (AHEAD) lds_barrier();
+        if constexpr (AHEAD || FSTAGE) lds_barrier();
         else __syncthreads();
     };
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -468,6 +468,32 @@ __global__ __launch_bounds__((kHmWaves<H, D, true> * 64)) void headmix_bwd_kerne
     // the other axis: keys up to the diagonal (dQ) or rows from the diagonal on (dK / dV)
     const int lo = WHAT == 0 ? 0 : (a.causal ? fixed0 : 0);
     const int hi = WHAT == 0 ? (a.causal ? min(a.N, fixed0 + HT) : a.N) : a.N;
+    // dK + dV with fragment staging: the fragments of the first pair of heads are asked for two phases before
+    // their products (Q / K of the next row tile during the last two phases of this one, dO / V during the
+    // probability phase), in the registers that the other pair of fragment sets has just left
+    constexpr int NPF = FSTAGE ? PU : 1;
+    bf16x8 pq[NPF][D / 32], pk[NPF][D / 32], pg[NPF][D / 32], pv[NPF][D / 32];
+    auto prefetch_qk = [&](int i0n) {
+        if constexpr (FSTAGE) {
+#pragma unroll
+            for (int u = 0; u < PU; ++u) {
+                const size_t ho = (size_t)(wave + u * HW) * a.N * D;
+                load_frags<D>(pq[u], Qb + ho, i0n, a.N, g, n);
+                load_frags<D>(pk[u], Kb + ho, fixed0, a.N, g, n);
+            }
+        }
+    };
+    auto prefetch_gv = [&](int i0n) {
+        if constexpr (FSTAGE) {
+#pragma unroll
+            for (int u = 0; u < PU; ++u) {
+                const size_t ho = (size_t)(wave + u * HW) * a.N * D;
+                load_frags<D>(pg[u], Gb + ho, i0n, a.N, g, n);
+                load_frags<D>(pv[u], Vb + ho, fixed0, a.N, g, n);
+            }
+        }
+    };
+    prefetch_qk(lo);
     for (int o0 = lo; o0 < hi; o0 += HT) {
         const int i0 = WHAT == 0 ? fixed0 : o0, j0 = WHAT == 0 ? o0 : fixed0;
         tile_barrier();   // the last tile's dS has been used (and, first, W and the statistics are in place)
@@ -494,9 +520,14 @@ __global__ __launch_bounds__((kHmWaves<H, D, true> * 64)) void headmix_bwd_kerne
                 bf16x8 xq[PU][D / 32], xk[PU][D / 32];
 #pragma unroll
                 for (int u = 0; u < PU; ++u) {
-                    const size_t ho = (size_t)(wave + (t0 + u) * HW) * a.N * D;
-                    load_frags<D>(xq[u], Qb + ho, i0, a.N, g, n);
-                    load_frags<D>(xk[u], Kb + ho, j0, a.N, g, n);
+                    if (t0 == 0) {
+#pragma unroll
+                        for (int blk = 0; blk < D / 32; ++blk) { xq[u][blk] = pq[u][blk]; xk[u][blk] = pk[u][blk]; }
+                    } else {
+                        const size_t ho = (size_t)(wave + (t0 + u) * HW) * a.N * D;
+                        load_frags<D>(xq[u], Qb + ho, i0, a.N, g, n);
+                        load_frags<D>(xk[u], Kb + ho, j0, a.N, g, n);
+                    }
                 }
 #pragma unroll
                 for (int u = 0; u < PU; ++u) {
@@ -511,6 +542,7 @@ __global__ __launch_bounds__((kHmWaves<H, D, true> * 64)) void headmix_bwd_kerne
             scores_phase<H, D, HW>(S, a, Qb, Kb, i0, j0, wave, g, n);
         }
         tile_barrier();
+        prefetch_gv(i0);
         // ---- P = exp(Z - LSE), rows of this wave ----
 #pragma unroll
         for (int rl = 0; rl < RPW; ++rl) {
@@ -534,9 +566,14 @@ __global__ __launch_bounds__((kHmWaves<H, D, true> * 64)) void headmix_bwd_kerne
                 bf16x8 xg[PU][D / 32], xv[PU][D / 32];
 #pragma unroll
                 for (int u = 0; u < PU; ++u) {
-                    const size_t ho = (size_t)(wave + (t0 + u) * HW) * a.N * D;
-                    load_frags<D>(xg[u], Gb + ho, i0, a.N, g, n);
-                    load_frags<D>(xv[u], Vb + ho, j0, a.N, g, n);
+                    if (t0 == 0) {
+#pragma unroll
+                        for (int blk = 0; blk < D / 32; ++blk) { xg[u][blk] = pg[u][blk]; xv[u][blk] = pv[u][blk]; }
+                    } else {
+                        const size_t ho = (size_t)(wave + (t0 + u) * HW) * a.N * D;
+                        load_frags<D>(xg[u], Gb + ho, i0, a.N, g, n);
+                        load_frags<D>(xv[u], Vb + ho, j0, a.N, g, n);
+                    }
                 }
 #pragma unroll
                 for (int u = 0; u < PU; ++u) {
@@ -578,6 +615,9 @@ __global__ __launch_bounds__((kHmWaves<H, D, true> * 64)) void headmix_bwd_kerne
         }
         }
         tile_barrier();
+        // (unconditionally, past the last row too, where the loads are switched off lane by lane: fragments that
+        // may or may not be replaced here would have to stay in their registers through the whole tile)
+        if constexpr (WHAT == 1) prefetch_qk(o0 + HT);
         // ---- rows of this wave: dW += dZ S^T over its elements, then dS = scale W^T dZ in place ----
 #pragma unroll
         for (int rl = 0; rl < RPW; ++rl) {
