@@ -178,6 +178,27 @@ def test_one_pass_backward_workspace_garbage_and_tile_edges():
         assert rel_max(out[3], ref[3]) <= TOL_DW_REL, N
 
 
+@pytest.mark.parametrize("one_pass", [False, True])
+def test_backward_more_than_65535_batch_head_pairs(one_pass):
+    # B * H beyond a grid dimension's 65535 (every kernel of the backward puts heads and batch entries on
+    # separate grid dimensions).  Every (batch, head) pair is computed on its own: the last heads of the big
+    # run must equal, bit for bit, a run of those heads alone, and a sample of pairs the CPU oracle.
+    B, H, N, d, c_q, c_k = 2, 33000, 2, 32, 3, 3
+    Q, K, V, dO, W = rand_case(B, H, N, N, d, c_q, c_k, torch.bfloat16, seed=11)
+    g = [t.to(DEV) for t in (Q, K, V, dO, W)]
+    assert ops.kernel_path(g[0], g[1], g[4], True, op="bwd") == "mfma"
+    big = _run_bwd(*g, True, torch.float32, one_pass)
+    sl = slice(H - 40, H)
+    part = _run_bwd(*(t[:, sl].contiguous() for t in g[:4]), g[4][sl].contiguous(), True, torch.float32, one_pass)
+    for got, want in zip(big[:3], part[:3]):
+        assert torch.equal(got[:, sl], want)
+    assert torch.equal(big[3][sl], part[3])
+    ref = oracle_bwd(Q[:, sl], K[:, sl], V[:, sl], W[sl], dO[:, sl], True)
+    for got, want in zip(part[:3], ref[:3]):
+        assert max_abs(got, want) <= TOL_BF16
+    assert rel_max(part[3], ref[3]) <= TOL_DW_REL
+
+
 def test_module_autograd_matches_oracle_autograd():
     from flash_multi_token_attention_amd.conv_attn import ConvAttentionCUDA
     B, H, N, d, c_q, c_k = 2, 4, 192, 128, 6, 11
