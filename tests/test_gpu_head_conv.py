@@ -69,6 +69,25 @@ def test_backward(B, H, N, d, causal):
         assert err <= tol, (name, err, tol)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_other_input_dtypes_are_used_as_bf16(dtype):
+    # float32 and float16 tensors are converted to bfloat16 (the kernels' operand type): the results are those of
+    # the converted inputs, bit for bit; O comes back in the dtype of q
+    Q, K, V, dO, W = _case(2, 16, 90, 64, seed=5)
+    ops = _ops()
+    lo = [t.to(DEV) for t in (Q, K, V, W, dO)]
+    hi = [t.to(dtype) if t.dtype == torch.bfloat16 else t for t in lo]
+    O, L, M = ops.forward(*lo[:4], scale=0.125, causal=True)
+    O2, L2, M2 = ops.forward(*hi[:4], scale=0.125, causal=True)
+    # (O is rounded once, to the dtype of q: within a bf16 rounding of the bf16 result; the statistics are the same)
+    assert O2.dtype == dtype and torch.equal(L2, L) and torch.equal(M2, M)
+    assert float((O2.float() - O.float()).abs().max()) <= 2.0 ** -8 * max(1.0, float(O.float().abs().max()))
+    for fn in (ops.bwd_dq_dw, ops.bwd_dkdv):
+        a = fn(*lo[:4], O, lo[4], L, M, causal=True, scale=0.125)
+        b = fn(*hi[:4], O, hi[4], L, M, causal=True, scale=0.125)
+        assert all(torch.equal(x, y) for x, y in zip(a, b))
+
+
 def test_identity_map_is_plain_attention():
     Q, K, V, _, _ = _case(1, 16, 100, 64, seed=9)
     O, _, _ = _ops().forward(Q.to(DEV), K.to(DEV), V.to(DEV), torch.eye(16, device=DEV), scale=0.125, causal=True)
