@@ -78,26 +78,58 @@ __global__ __launch_bounds__(256) void dw_reduce_kernel(int B, int H, int n_tile
         dW[(size_t)h * ntap + tap] = (red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]);
 }
 
-// One workgroup per (batch, head): m = max m_s, l = sum l_s e^{m_s - m},
-// o = sum o_s e^{m_s - m} / l.
+// Merge of the decode splits: m = max m_s, l = sum l_s e^{m_s - m}, o = sum o_s e^{m_s - m} / l.
+// A workgroup takes 32 output columns of one (batch, head).  All 256 threads scan the splits'
+// (m_s, l_s) together (every workgroup of a head repeats this: at most 1024 pairs); for the
+// outputs thread (g, c) adds the splits g, g+8, ... of column c, so a split's row is read with
+// 128-byte loads and eight rows are in flight per pass, and the eight sums are added in order of g.
 template <typename TO>
-__global__ void combine_kernel(int n_splits, int d, const float *__restrict__ O_part,
-                               const float *__restrict__ M_part, const float *__restrict__ L_part,
-                               TO *__restrict__ O, float *__restrict__ M, float *__restrict__ L) {
+__global__ __launch_bounds__(256) void combine_kernel(int n_splits, int d, const float *__restrict__ O_part,
+                                                      const float *__restrict__ M_part,
+                                                      const float *__restrict__ L_part, TO *__restrict__ O,
+                                                      float *__restrict__ M, float *__restrict__ L) {
+    __shared__ float red_m[4], red_l[4], acc[8][32];
     const size_t bh = blockIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const float *mp = M_part + bh * n_splits;
     const float *lp = L_part + bh * n_splits;
     float m = kNegInf;
-    for (int s = 0; s < n_splits; ++s) m = fmaxf(m, mp[s]);
+    for (int s = tid; s < n_splits; s += 256) m = fmaxf(m, mp[s]);
+#pragma unroll
+    for (int x = 32; x >= 1; x >>= 1) m = fmaxf(m, __shfl_xor(m, x));
+    if (lane == 0) red_m[wave] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(red_m[0], red_m[1]), fmaxf(red_m[2], red_m[3]));
     float l = 0.f;
-    for (int s = 0; s < n_splits; ++s) l += (mp[s] == kNegInf) ? 0.f : lp[s] * __expf(mp[s] - m);
-    for (int c = threadIdx.x; c < d; c += blockDim.x) {
-        float o = 0.f;
-        for (int s = 0; s < n_splits; ++s)
-            if (mp[s] != kNegInf) o = fmaf(O_part[(bh * n_splits + s) * d + c], __expf(mp[s] - m), o);
-        O[bh * d + c] = from_f32<TO>(o / l);
+    for (int s = tid; s < n_splits; s += 256) {
+        const float ms = mp[s];
+        if (ms != kNegInf) l = fmaf(lp[s], __expf(ms - m), l);
     }
-    if (threadIdx.x == 0) { M[bh] = m; L[bh] = l; }
+#pragma unroll
+    for (int x = 32; x >= 1; x >>= 1) l += __shfl_xor(l, x);
+    if (lane == 0) red_l[wave] = l;
+    __syncthreads();
+    l = (red_l[0] + red_l[1]) + (red_l[2] + red_l[3]);
+
+    const int c = tid & 31, g = tid >> 5, col = blockIdx.y * 32 + c;
+    float o = 0.f;
+    if (col < d) {
+        const float *op = O_part + bh * n_splits * d + col;
+#pragma unroll 4
+        for (int s = g; s < n_splits; s += 8) {
+            const float ms = mp[s];
+            if (ms != kNegInf) o = fmaf(op[(size_t)s * d], __expf(ms - m), o);
+        }
+    }
+    acc[g][c] = o;
+    __syncthreads();
+    if (tid < 32 && col < d) {
+        float sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sum += acc[i][c];
+        O[bh * d + col] = from_f32<TO>(sum / l);
+    }
+    if (tid == 0 && blockIdx.y == 0) { M[bh] = m; L[bh] = l; }
 }
 
 }  // namespace
@@ -123,11 +155,11 @@ hipError_t dw_reduce(const Problem &p, int n_tiles, const float *dw_part, float 
 
 hipError_t decode_combine(const Problem &p, int out_dt, const float *o_part, const float *m_part,
                           const float *l_part, void *o, float *m, float *l, hipStream_t s) {
-    const unsigned grid = (unsigned)(p.B * p.H);
+    const dim3 grid((unsigned)(p.B * p.H), (unsigned)((p.d + 31) / 32));
     if (out_dt == CONVATTN_BF16)
-        combine_kernel<bf16_t><<<grid, 128, 0, s>>>(p.n_splits, p.d, o_part, m_part, l_part, (bf16_t *)o, m, l);
+        combine_kernel<bf16_t><<<grid, 256, 0, s>>>(p.n_splits, p.d, o_part, m_part, l_part, (bf16_t *)o, m, l);
     else
-        combine_kernel<float><<<grid, 128, 0, s>>>(p.n_splits, p.d, o_part, m_part, l_part, (float *)o, m, l);
+        combine_kernel<float><<<grid, 256, 0, s>>>(p.n_splits, p.d, o_part, m_part, l_part, (float *)o, m, l);
     return hipGetLastError();
 }
 
