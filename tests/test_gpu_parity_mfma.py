@@ -233,6 +233,7 @@ def test_module_autograd_matches_oracle_autograd():
     (6, 130, 128, 16, 17, 2),
     (16, 240, 32, 5, 5, 4),      # the reference's own decode test (scripts/test_fwd_inference_conv_attn.py:31-56)
     (6, 1000, 32, 6, 11, 2),
+    (11, 40000, 64, 11, 11, 700),  # more splits than the merge kernel has threads (a long cache as in scripts/benchmark_fwd_inference_conv_attn.py)
 ])
 @pytest.mark.parametrize("causal", [False, True])
 def test_decode_bf16_stream(r, Nk, d, c_q, c_k, splits, causal):
