@@ -44,6 +44,9 @@ import sys
 TRAIN_SUITE = [(256, 3), (512, 3), (1024, 3), (2048, 7), (2048, 11), (4096, 11), (8192, 11)]
 TRAIN_SWEEP = [(n, k) for k in (3, 7, 11) for n in (256, 512, 1024, 2048, 4096, 8192)]
 DECODE_SWEEP = [1024, 4096, 16384, 65536]
+# the configuration of the reference's decode figure (scripts/plot_fwd_inference_speedup.py:59-70):
+# batch 2, 2 heads, 16 query rows, head dim 64, 7x7 window, 32 key splits, not causal
+DECODE_REF_SWEEP = [512, 1024, 2048, 4096]
 
 
 def time_ms(fn: Callable[[], None], iters: int = 20, warmup: int = 5) -> float:
@@ -98,18 +101,19 @@ def train_case(B: int, H: int, N: int, d: int, k: int, iters: int) -> dict:
     return r
 
 
-def decode_case(B: int, H: int, Nk: int, d: int, c_q: int, c_k: int, iters: int) -> dict:
+def decode_case(B: int, H: int, Nk: int, d: int, c_q: int, c_k: int, iters: int, q_rows: int = 0,
+                k_splits: int = 0) -> dict:
     from .conv_attn.inference import fwd_conv_attn_inference
     dev = "cuda:0"
     g = torch.Generator().manual_seed(42)
-    Q = torch.randn(B, H, c_q, d, generator=g).to(torch.bfloat16).to(dev)
+    Q = torch.randn(B, H, q_rows or c_q, d, generator=g).to(torch.bfloat16).to(dev)
     K, V = (torch.randn(B, H, Nk, d, generator=g).to(torch.bfloat16).to(dev) for _ in range(2))
     W = (0.02 * torch.randn(H, c_q, c_k, generator=g)).to(dev)
     scale = 1.0 / math.sqrt(d)
     q_last = Q[:, :, -1:, :].contiguous()
 
     def conv():
-        fwd_conv_attn_inference(Q, K, V, W, 0, scale, c_q - 1, (c_k - 1) // 2, False)
+        fwd_conv_attn_inference(Q, K, V, W, k_splits, scale, c_q - 1, (c_k - 1) // 2, False)
 
     def sdpa():
         F.scaled_dot_product_attention(q_last, K, V, scale=scale)
@@ -147,6 +151,8 @@ def parse_table(path: str) -> List[dict]:
     for line in open(path):
         line = line.strip()
         if not line.startswith("|"):
+            if head is not None:
+                break   # the end of the first table
             continue
         cells = [c.strip() for c in line.strip("|").split("|")]
         if head is None:
@@ -291,6 +297,16 @@ def main(argv=None) -> None:
         for Nk in (DECODE_SWEEP[:2] if a.quick else DECODE_SWEEP):
             r = decode_case(B, H, Nk, d, 11, 11, a.iters)
             emit(f"| {Nk} | {r['conv']:.4f} | {r['sdpa']:.4f} | {r['conv_gbs']:.0f} |")
+        if not (a.batch or a.heads or a.head_dim):
+            emit("")
+            emit("The configuration of the reference's decode figure (B=2 H=2 d=64, 16 query rows, 7x7 window, "
+                 "k_splits=32, not causal):")
+            emit("")
+            emit("| Nk | conv decode | sdpa last row |")
+            emit("|---|---|---|")
+            for Nk in (DECODE_REF_SWEEP[:2] if a.quick else DECODE_REF_SWEEP):
+                r = decode_case(2, 2, Nk, 64, 7, 7, a.iters, q_rows=16, k_splits=32)
+                emit(f"| {Nk} | {r['conv']:.4f} | {r['sdpa']:.4f} |")
     if a.md:
         with open(a.md, "w") as f:
             f.write("\n".join(lines) + "\n")

@@ -19,6 +19,7 @@ def fwd_conv_attn_inference(Q, K, V, conv_kernel, k_splits, scale, pad_q, pad_k,
     """
     if Q.shape[2] > 16:
         raise ValueError(f"Q sequence length must be <= 16 for inference, got {Q.shape[2]}")
-    ops._weights(conv_kernel, Q.shape[1], pad_q, pad_k, Q.device)  # checks pad_q / pad_k
+    if conv_kernel.dim() != 3 or pad_q != conv_kernel.shape[1] - 1 or pad_k != (conv_kernel.shape[2] - 1) // 2:
+        ops._weights(conv_kernel, Q.shape[1], pad_q, pad_k, Q.device)  # raises, naming what is wrong
     O, M, L, _ = ops.decode(Q, K, V, conv_kernel, k_splits, scale, causal)
     return O, M, L
