@@ -78,7 +78,28 @@ __global__ __launch_bounds__(256) void dw_reduce_kernel(int B, int H, int n_tile
         dW[(size_t)h * ntap + tap] = (red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]);
 }
 
-// Merge of the decode splits: m = max m_s, l = sum l_s e^{m_s - m}, o = sum o_s e^{m_s - m} / l.
+// Merge of a few decode splits: one workgroup per (batch, head), one thread per output column walks the splits.
+template <typename TO>
+__global__ void combine_few_kernel(int n_splits, int d, const float *__restrict__ O_part,
+                                   const float *__restrict__ M_part, const float *__restrict__ L_part,
+                                   TO *__restrict__ O, float *__restrict__ M, float *__restrict__ L) {
+    const size_t bh = blockIdx.x;
+    const float *mp = M_part + bh * n_splits;
+    const float *lp = L_part + bh * n_splits;
+    float m = kNegInf;
+    for (int s = 0; s < n_splits; ++s) m = fmaxf(m, mp[s]);
+    float l = 0.f;
+    for (int s = 0; s < n_splits; ++s) l += (mp[s] == kNegInf) ? 0.f : lp[s] * __expf(mp[s] - m);
+    for (int c = threadIdx.x; c < d; c += blockDim.x) {
+        float o = 0.f;
+        for (int s = 0; s < n_splits; ++s)
+            if (mp[s] != kNegInf) o = fmaf(O_part[(bh * n_splits + s) * d + c], __expf(mp[s] - m), o);
+        O[bh * d + c] = from_f32<TO>(o / l);
+    }
+    if (threadIdx.x == 0) { M[bh] = m; L[bh] = l; }
+}
+
+// Merge of many decode splits: m = max m_s, l = sum l_s e^{m_s - m}, o = sum o_s e^{m_s - m} / l.
 // A workgroup takes 32 output columns of one (batch, head).  All 256 threads scan the splits'
 // (m_s, l_s) together (every workgroup of a head repeats this: at most 1024 pairs); for the
 // outputs thread (g, c) adds the splits g, g+8, ... of column c, so a split's row is read with
@@ -155,6 +176,16 @@ hipError_t dw_reduce(const Problem &p, int n_tiles, const float *dw_part, float 
 
 hipError_t decode_combine(const Problem &p, int out_dt, const float *o_part, const float *m_part,
                           const float *l_part, void *o, float *m, float *l, hipStream_t s) {
+    // (a serving step with many (batch, head) pairs has a handful of splits: the walk over them is shorter than
+    // the second kernel's two reductions; few pairs over a long cache have hundreds)
+    if (p.n_splits <= 8) {
+        const unsigned few = (unsigned)(p.B * p.H);
+        if (out_dt == CONVATTN_BF16)
+            combine_few_kernel<bf16_t><<<few, 128, 0, s>>>(p.n_splits, p.d, o_part, m_part, l_part, (bf16_t *)o, m, l);
+        else
+            combine_few_kernel<float><<<few, 128, 0, s>>>(p.n_splits, p.d, o_part, m_part, l_part, (float *)o, m, l);
+        return hipGetLastError();
+    }
     const dim3 grid((unsigned)(p.B * p.H), (unsigned)((p.d + 31) / 32));
     if (out_dt == CONVATTN_BF16)
         combine_kernel<bf16_t><<<grid, 256, 0, s>>>(p.n_splits, p.d, o_part, m_part, l_part, (bf16_t *)o, m, l);
