@@ -1,5 +1,6 @@
 """Seeded random shapes through the C ABI against the CPU oracle: the MFMA training kernels
-(forward, one-pass and two-pass backward) and the decode stream with every kind of split count.
+(forward, one-pass and two-pass backward), the decode stream with every kind of split count and
+the head-mixing kernels.
 The fixed lists of the other test files sit on the tile edges; these draws cover the combinations
 between them.  Each case prints its shape before it runs."""
 import random
@@ -69,3 +70,34 @@ def test_random_decode_shapes_match_oracle():
         O, M, L, _ = ops.decode(g[0], g[1], g[2], g[3], splits, scale_of(d), causal, out_dtype=out_dtype)
         assert max_abs(O, O_ref) <= TOL_BF16, case
         assert max_abs(M, M_ref) <= 1e-3 and rel_max(L, L_ref) <= 1e-3, case
+
+
+def test_random_head_mixing_shapes_match_oracle():
+    import math
+    from flash_multi_token_attention_amd.head_conv_attn import ops
+    from oracle import head_conv_oracle as hc
+    rnd = random.Random(777)
+    for case in range(40):
+        H = rnd.choice([16, 32])
+        d = rnd.choice([32, 64, 128])
+        N = rnd.choice([1, 15, 16, 17, 31, 33, 64, 100, 127, 129, 200, 257, 300])
+        B = rnd.choice([1, 2, 3])
+        causal = rnd.random() < 0.6
+        w_scale = rnd.choice([0.3, 1.0])
+        print(f"case {case}: B{B} H{H} N{N} d{d} causal={causal} w_scale={w_scale}", flush=True)
+        g = torch.Generator().manual_seed(1000 + case)
+        Q, K, V, dO = (torch.randn(B, H, N, d, generator=g).to(torch.bfloat16) for _ in range(4))
+        W = w_scale * torch.randn(H, H, generator=g) / math.sqrt(H) + torch.eye(H)
+        sc = 1.0 / math.sqrt(d)
+        t = [x.to(DEV) for x in (Q, K, V, W, dO)]
+        O, L, M = ops.forward(t[0], t[1], t[2], t[3], scale=sc, causal=causal)
+        Or, Lr, Mr = hc.forward(Q.float(), K.float(), V.float(), W, causal, sc)
+        assert float((O.float().cpu() - Or).abs().max()) <= TOL_BF16, case
+        assert float((M.cpu() - Mr).abs().max()) <= 1e-3 and float(((L.cpu() - Lr).abs() / Lr).max()) <= 1e-3, case
+        dQ, dW = ops.bwd_dq_dw(t[0], t[1], t[2], t[3], O, t[4], L, M, causal=causal, scale=sc)
+        dK, dV = ops.bwd_dkdv(t[0], t[1], t[2], t[3], O, t[4], L, M, causal=causal, scale=sc)
+        ref = hc.backward_autograd(Q.float(), K.float(), V.float(), W, dO.float(), causal, sc)
+        for name, got, want in zip(("dQ", "dK", "dV", "dW"), (dQ, dK, dV, dW), ref):
+            tol = 1e-2 * max(1.0, float(want.abs().max()))
+            err = float((got.cpu() - want).abs().max())
+            assert err <= tol, (case, name, err, tol)
