@@ -29,10 +29,11 @@ namespace {
 
 typedef short short4_t __attribute__((ext_vector_type(4)));
 
-// waves per workgroup: one per head with 16 heads (half the accumulators and fragments per wave, four waves per
-// SIMD to hide the latencies between the phases) where 128 registers per wave hold that without much scratch
-// (the forward, and the backward up to d = 64); otherwise 8 (two or four heads per wave)
-template <int H, int D, bool BWD> constexpr int kHmWaves = (H == 16 && (!BWD || D <= 64)) ? 16 : 8;
+// waves per workgroup: 16 in the forward (one or two heads per wave: half the accumulators and fragments per
+// wave, four waves per SIMD to hide the latencies between the phases) and in the backward with 16 heads up to
+// d = 64, where 128 registers per wave hold that without much scratch; otherwise 8 (two or four heads per wave;
+// with 32 heads the dW accumulators of 16 waves would not fit the LDS either)
+template <int H, int D, bool BWD> constexpr int kHmWaves = (!BWD || (H == 16 && D <= 64)) ? 16 : 8;
 constexpr int HT = 16;           // rows / keys per tile
 constexpr int SST = 20;          // floats per row of a score tile in LDS
 constexpr int HST = HT * SST + 16;   // floats per head of a score array (== 16 mod 32: see the reads in phase 2)
@@ -47,13 +48,13 @@ struct HmArgs {
 };
 
 // XT: staging tiles per wave (1, or one per head of the wave where K tiles are staged a phase early)
-template <int H, int D, int XT, int HW> struct HmLds {
+template <int H, int D, int XT, int HW, int ARRS = 2> struct HmLds {
     static constexpr int WST = H + 4;                       // floats per row of W
     static constexpr int XST = D * 2 + 32;                  // bytes per row of a staged bf16 tile
     static constexpr int arr_bytes = H * HST * 4;           // one score array
     static constexpr int s_off = 0;                         // S (forward: then P in place)
     static constexpr int p_off = s_off + arr_bytes;         // backward: P, then dZ, then dS
-    static constexpr int w_off = p_off + arr_bytes;
+    static constexpr int w_off = s_off + ARRS * arr_bytes;   // (the forward has no second array)
     static constexpr int x_off = w_off + H * WST * 4;       // per-wave staging tiles
     static constexpr int stat_off = x_off + HW * XT * HT * XST;  // three [H][16] float arrays
     static constexpr int total = stat_off + 3 * H * HT * 4;
@@ -215,7 +216,7 @@ __global__ __launch_bounds__((kHmWaves<H, D, false> * 64)) void headmix_fwd_kern
                                                               const float *__restrict__ W, TO *__restrict__ O,
                                                               float *__restrict__ L, float *__restrict__ M) {
     constexpr int HW = kHmWaves<H, D, false>;
-    using Lds = HmLds<H, D, 1, HW>;
+    using Lds = HmLds<H, D, 1, HW, 1>;
     constexpr int DB = D / 16, HPW = H / HW, RPW = HT / HW;  // heads and rows per wave
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     float *S = reinterpret_cast<float *>(smem + Lds::s_off);
@@ -245,8 +246,10 @@ __global__ __launch_bounds__((kHmWaves<H, D, false> * 64)) void headmix_fwd_kern
     // Where the registers allow it the Q fragments of the wave's heads stay resident, the K fragments
     // of a tile are loaded while the tile before it is worked on, and the V rows of a tile are on their
     // way during its score and softmax phases: a workgroup fills its CU alone, so nothing else hides
-    // the latency of these loads.
-    constexpr bool AHEAD = HPW * (D / 32) <= 8;
+    // the latency of these loads.  (16 heads only: with 32 heads the softmax state of the mixed rows takes twice
+    // the registers, the fragments held ahead went to scratch memory and cost more than they hid: B2 N2048 d64
+    // 2.17 ms with them, 1.05 ms without.)
+    constexpr bool AHEAD = HPW * (D / 32) <= 8 && H == 16;
     constexpr int NCH = (HT * D / 8 + 63) / 64;
     // (K rows as whole rows, 1 KB of consecutive memory per load, and from the wave's staging tile into the
     // fragments: a fragment load straight from memory takes 64 bytes of each of 16 rows, half of every cache line
@@ -747,7 +750,7 @@ __global__ __launch_bounds__(256) void headmix_dw_reduce_kernel(int n_part, int 
 template <int H, int D>
 hipError_t launch_fwd(const HmArgs &a, int out_dt, const void *q, const void *k, const void *v, const float *w, void *o,
                       float *l, float *m, hipStream_t s) {
-    constexpr int HW = kHmWaves<H, D, false>, lds = HmLds<H, D, 1, HW>::total;
+    constexpr int HW = kHmWaves<H, D, false>, lds = HmLds<H, D, 1, HW, 1>::total;
     static_assert(lds <= 160 * 1024, "LDS budget");
     dim3 grid((a.N + HT - 1) / HT, a.B);
     if (out_dt == CONVATTN_BF16) {
