@@ -248,14 +248,15 @@ __global__ __launch_bounds__((kHmWaves<H, D, false> * 64)) void headmix_fwd_kern
     // way during its score and softmax phases: a workgroup fills its CU alone, so nothing else hides
     // the latency of these loads.  (16 heads only: with 32 heads the softmax state of the mixed rows takes twice
     // the registers, the fragments held ahead went to scratch memory and cost more than they hid: B2 N2048 d64
-    // 2.17 ms with them, 1.05 ms without.)
+    // 2.17 ms with them, 1.05 ms without, 0.82 ms with Q alone resident and K as whole rows.)
     constexpr bool AHEAD = HPW * (D / 32) <= 8 && H == 16;
+    constexpr bool QRES = !AHEAD;   // the Q fragments alone stay resident
     constexpr int NCH = (HT * D / 8 + 63) / 64;
     // (K rows as whole rows, 1 KB of consecutive memory per load, and from the wave's staging tile into the
     // fragments: a fragment load straight from memory takes 64 bytes of each of 16 rows, half of every cache line
     // it touches, and the vector memory pipe of the CU, which a workgroup's loads pass one after the other, is what
     // the score phase waits for)
-    bf16x8 qf[AHEAD ? HPW : 1][D / 32];
+    bf16x8 qf[(AHEAD || QRES) ? HPW : 1][D / 32];
     u32x4 kr[AHEAD ? HPW : 1][NCH], vr[AHEAD ? HPW : 1][NCH];
     if constexpr (AHEAD) {
 #pragma unroll
@@ -263,6 +264,10 @@ __global__ __launch_bounds__((kHmWaves<H, D, false> * 64)) void headmix_fwd_kern
             load_frags<D>(qf[t], Qb + (size_t)(wave + t * HW) * a.N * D, i0, a.N, g, n);
             load_chunks<D>(kr[t], Kb + (size_t)(wave + t * HW) * a.N * D, 0, a.N, lane);
         }
+    }
+    if constexpr (QRES) {
+#pragma unroll
+        for (int t = 0; t < HPW; ++t) load_frags<D>(qf[t], Qb + (size_t)(wave + t * HW) * a.N * D, i0, a.N, g, n);
     }
 
     const int j_end = a.causal ? min(a.N, i0 + HT) : a.N;
@@ -289,6 +294,25 @@ __global__ __launch_bounds__((kHmWaves<H, D, false> * 64)) void headmix_fwd_kern
                 load_chunks<D>(kr[t], Kb + (size_t)h * a.N * D, j0 + HT, a.N, lane);
 #pragma unroll
                 for (int r = 0; r < 4; ++r) S[h * HST + (4 * g + r) * SST + n] = sc[t][r] * a.scale;
+            }
+        } else if constexpr (QRES) {
+#pragma unroll
+            for (int t = 0; t < HPW; ++t) {
+                const int h = wave + t * HW;
+                // (K as whole rows through the wave's staging tile, as above)
+                bf16x8 kf[D / 32];
+                {
+                    u32x4 kc[NCH];
+                    load_chunks<D>(kc, Kb + (size_t)h * a.N * D, j0, a.N, lane);
+                    stage_chunks<D>(xt, Lds::XST, kc, lane);
+#pragma unroll
+                    for (int blk = 0; blk < D / 32; ++blk)
+                        kf[blk] = *reinterpret_cast<const bf16x8 *>(xt + n * Lds::XST + (blk * 32 + 8 * g) * 2);
+                    __builtin_amdgcn_wave_barrier();
+                }
+                const f32x4 acc = frags_dot<D>(qf[t], kf);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) S[h * HST + (4 * g + r) * SST + n] = acc[r] * a.scale;
             }
         } else {
             scores_phase<H, D, HW>(S, a, Qb, Kb, i0, j0, wave, g, n);
